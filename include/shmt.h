@@ -1,0 +1,200 @@
+/*
+ * shmt.h — C ABI of libshmt.so: the GPU-cache hot path of ShmTensor
+ * (static hashmap, cached feature fetch/set, cached neighbour sampling,
+ * relabel, scan) as hand-written HIP for gfx950 (MI355X).
+ *
+ * Conventions
+ *  - Every pointer is a raw address the GPU can dereference: device memory,
+ *    or host memory that is pinned and device-mapped (see shmt_host_devptr).
+ *    No torch types cross this boundary; callers allocate every buffer,
+ *    including scratch, and pass element SIZES in bytes (4 or 8 for integer
+ *    ids; any size for feature rows, which are copied bit for bit).
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *    All work is enqueued on it; no entry point synchronises unless it says so.
+ *  - Return value: 0 on success, a negative SHMT_E* code on failure, with a
+ *    human readable message available from shmt_last_error() (thread local).
+ *    The library never calls exit()/abort() (the reference does on any CUDA
+ *    error: include/common.h:15-27).
+ *  - Zero-length inputs are valid and are no-ops (the reference launches a
+ *    zero-size grid and exits: src/cache_feature_fetch.cu:77-83).
+ *
+ * Each entry point cites the reference interface (file:line under the
+ * ShmTensor source tree) that it replaces.
+ */
+#ifndef SHMT_H_
+#define SHMT_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SHMT_OK 0
+#define SHMT_EINVAL (-1)  /* bad argument (null pointer, size, dtype width) */
+#define SHMT_EHIP (-2)    /* a HIP runtime call failed                       */
+#define SHMT_ENOTPINNED (-3) /* host pointer is not device-accessible        */
+#define SHMT_ENOMEM (-4)  /* caller-provided buffer too small                */
+
+#define SHMT_ABI_VERSION 1
+
+/* Library identification / error channel (no counterpart in the reference,
+ * whose errors are c10 exceptions or exit(): include/common.h:10-27). */
+int shmt_abi_version(void);
+const char *shmt_last_error(void);
+
+/* ------------------------------------------------------------------ */
+/* Host memory: PinMemory / UnpinMemory, src/cache_feature_fetch.cu:6-13
+ * (cudaHostRegister(ptr, nbytes, cudaHostRegisterPortable) /
+ * cudaHostUnregister), and the registration done by
+ * include/shm_memory.h:19-21,35-37 and src/mmap_tensor.cc:42-45.          */
+
+/* Page-lock and device-map an existing host range in place. */
+int shmt_host_register(void *host_ptr, int64_t nbytes);
+int shmt_host_unregister(void *host_ptr);
+/* Translate a pointer a kernel is about to dereference. Device pointers
+ * pass through unchanged; pinned host pointers (registered here, or
+ * allocated pinned by the caller) yield their device-side alias, interior
+ * pointers included; ordinary pageable host memory fails with
+ * SHMT_ENOTPINNED instead of faulting inside a kernel.                     */
+int shmt_host_devptr(const void *ptr, void **dev_ptr_out);
+
+/* ------------------------------------------------------------------ */
+/* Static hashmap: pycuco::CUCOHashmapWrapper, src/cuco_hashmap.cu:10-41,
+ * include/cuco_hashmap.cuh:49-93 (cuco::static_map, linear probing, empty
+ * key -1 / empty value -1), pybind class CUCOStaticHashmap
+ * src/pybind.cc:60-64.                                                     */
+typedef struct shmt_hashmap shmt_hashmap_t;
+
+/* capacity() as the reference reports it: (int64)ceil(n / load_factor),
+ * include/cuco_hashmap.cuh:62,75.                                          */
+int64_t shmt_hashmap_capacity(int64_t n, double load_factor);
+/* Bytes of device memory the table needs (what memory_usage() returns;
+ * include/cuco_hashmap.cuh:25,76). key_bytes, val_bytes in {4, 8}.          */
+int64_t shmt_hashmap_table_bytes(int64_t n, double load_factor, int key_bytes,
+                                 int val_bytes);
+/* Build (constructor, include/cuco_hashmap.cuh:57-77): fills `table_mem`
+ * (device, >= shmt_hashmap_table_bytes, 128-byte aligned) with sentinels
+ * and inserts keys[i] -> vals[i] for i < n. Keys equal to -1 are not
+ * representable (sentinel). The table memory stays owned by the caller and
+ * must outlive the handle. Asynchronous on `stream`.                       */
+int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys,
+                        const void *vals, int64_t n, int key_bytes,
+                        int val_bytes, double load_factor, void *table_mem,
+                        int64_t table_bytes, void *stream);
+/* Bulk lookup (query, src/cuco_hashmap.cu:24-34 + include/cuco_hashmap.cuh:
+ * 81-87): requests of width req_bytes in {4,8} are first converted to the
+ * key width (two's-complement narrowing / sign extension, as
+ * requests.to(key_type_)), out[i] (width = val_bytes) = value or -1.        */
+int shmt_hashmap_query(const shmt_hashmap_t *map, const void *requests,
+                       int req_bytes, int64_t n, void *out, void *stream);
+int shmt_hashmap_key_bytes(const shmt_hashmap_t *map);
+int shmt_hashmap_val_bytes(const shmt_hashmap_t *map);
+int64_t shmt_hashmap_size(const shmt_hashmap_t *map);
+void shmt_hashmap_destroy(shmt_hashmap_t *map);
+
+/* ------------------------------------------------------------------ */
+/* Feature fetch: UVATensorFetch src/cache_feature_fetch.cu:47-87,
+ * CacheTensorFetch :131-185, CacheTensorFetchWithMask :226-272.
+ *   out[i,:] = slot_i >= 0 ? cache_data[slot_i,:] : miss_data[indices[i],:]
+ * with slot_i = map.find(indices[i]) (map != NULL), mask[i] (mask != NULL)
+ * or -1 (both NULL: the all-miss "uva" form; cache_data may be NULL).
+ * Rows are `row_bytes` long and contiguous; indices are idx_bytes in {4,8}
+ * wide; mask entries mask_bytes in {4,8} wide. `miss_data` is normally the
+ * device alias of pinned host memory, but any device-addressable table
+ * works. out has Q rows.                                                   */
+int shmt_fetch(const void *miss_data, const void *cache_data,
+               const void *indices, int idx_bytes, const shmt_hashmap_t *map,
+               const void *mask, int mask_bytes, void *out, int64_t Q,
+               int64_t row_bytes, void *stream);
+
+/* Feature set: UVATensorSet src/cache_feature_set.cu:39-75, CacheTensorSet
+ * :118-165, CacheTensorSetWithMask :209-248. Mirror of shmt_fetch:
+ *   (slot_i >= 0 ? cache_data[slot_i,:] : miss_data[indices[i],:]) = update[i,:]
+ * A hit does not write the miss-side row. Duplicate indices race, as in
+ * the reference.                                                           */
+int shmt_set(void *miss_data, void *cache_data, const void *indices,
+             int idx_bytes, const shmt_hashmap_t *map, const void *mask,
+             int mask_bytes, const void *update, int64_t Q, int64_t row_bytes,
+             void *stream);
+
+/* ------------------------------------------------------------------ */
+/* Scan. shmt_exclusive_scan: cub_exclusiveSum, src/tensor_relabel.cu:11-26
+ * and src/cache_graph_sampling.cu:30-45 — in-place exclusive prefix sum over
+ * `len` integers of elem_bytes in {4,8} (wraparound arithmetic); callers pass
+ * len = n + 1 so that the last output is the total.
+ * shmt_inclusive_scan_i32: thrust_scan, src/thrust_scan.cu:9-18
+ * (ptr[i] += ptr[i-1] in program order = in-place inclusive sum, int32).
+ * `tmp` is device scratch of at least shmt_scan_tmp_bytes(len) bytes.       */
+int64_t shmt_scan_tmp_bytes(int64_t len);
+int shmt_exclusive_scan(void *data, int64_t len, int elem_bytes, void *tmp,
+                        int64_t tmp_bytes, void *stream);
+int shmt_inclusive_scan_i32(void *data, int64_t len, void *tmp,
+                            int64_t tmp_bytes, void *stream);
+
+/* ------------------------------------------------------------------ */
+/* Relabel: TensorRelabel, src/tensor_relabel.cu:125-209 (RelabelHashmap
+ * :68-123). Input: N integers (elem_bytes in {4,8}), the concatenation of the
+ * caller's tensors. Output: unique_out[0..U) = distinct values in order of
+ * first occurrence, labels_out[i] = position of total[i] in unique_out,
+ * both of width elem_bytes; *count_out = U (int64). count_out must be
+ * device-accessible; when it points into pinned host memory the caller reads
+ * it after synchronising the stream. unique_out must hold N elements. The
+ * value -1 is not representable (empty key, src/tensor_relabel.cu:119).
+ * N < 2^31.                                                                */
+int64_t shmt_relabel_scratch_bytes(int64_t N);
+int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
+                 int64_t scratch_bytes, void *unique_out, void *labels_out,
+                 int64_t *count_out, void *stream);
+
+/* ------------------------------------------------------------------ */
+/* Neighbour sampling: CSRWiseSampling src/cache_graph_sampling.cu:179-220
+ * (GetSubIndptr :47-89, kernels :91-177) and CSRWiseCacheSampling :382-426
+ * (GetSubIndptrWithCache :222-289, kernels :291-380).
+ *
+ * Step 1, shmt_sample_plan: per seed s, adjacency = cached row
+ * cache_indptr[slot..slot+1] when map finds seeds[s] (map may be NULL: no
+ * cache), else indptr[v..v+1]; cnt = replace ? (deg > 0 ? k : 0)
+ * : min(deg, k); sub_indptr[0..S] = exclusive scan of cnt with total at [S]
+ * (width ptr_bytes, the indptr width). Also writes *nnz_out (int64,
+ * device-accessible) = total and the per-seed plan (row start, degree,
+ * source) into `plan` (>= shmt_sample_plan_bytes(S) bytes).
+ * Step 2, shmt_sample_pick: fills sub_indices[sub_indptr[s] ..) for every
+ * seed from the plan: whole adjacency in CSR order when deg <= k
+ * (replace = 0), k independent uniform picks (replace = 1), or a uniformly
+ * distributed k-subset (replace = 0, deg > k). Random choices are a pure
+ * function of (rng_seed, rng_stream, node id, k, degree) via Philox4x32-10,
+ * so they do not depend on batch composition or on whether the row was
+ * cached. sub_indices has width idx_bytes (the indices width) and room for
+ * the total (<= S * k).
+ * The reference fixes its RNG seed to 7777
+ * (src/cache_graph_sampling.cu:204,407).                                   */
+int64_t shmt_sample_plan_bytes(int64_t S);
+int shmt_sample_plan(const void *indptr, int ptr_bytes,
+                     const void *cache_indptr, const shmt_hashmap_t *map,
+                     const void *seeds, int seed_bytes, int64_t S, int64_t k,
+                     int replace, void *sub_indptr, void *plan,
+                     int64_t plan_bytes, int64_t *nnz_out, void *stream);
+int shmt_sample_pick(const void *indices, const void *cache_indices,
+                     int idx_bytes, const void *seeds, int seed_bytes,
+                     int64_t S, int64_t k, int replace, const void *sub_indptr,
+                     int ptr_bytes, const void *plan, void *sub_indices,
+                     uint64_t rng_seed, uint32_t rng_stream, void *stream);
+
+/* Cached sub-CSR: CreateCacheCSR, src/cache_graph_sampling.cu:455-492
+ * (CSRIndicesCopyKernel :428-453). Step 1 writes
+ * cache_indptr[0..C] = exclusive scan of deg(seeds[i]) (width ptr_bytes) and
+ * *nnz_out; step 2 copies the adjacency lists, in seeds order, into
+ * cache_indices (width idx_bytes).                                         */
+int shmt_subcsr_plan(const void *indptr, int ptr_bytes, const void *seeds,
+                     int seed_bytes, int64_t C, void *cache_indptr, void *tmp,
+                     int64_t tmp_bytes, int64_t *nnz_out, void *stream);
+int shmt_subcsr_copy(const void *indptr, const void *indices, int ptr_bytes,
+                     int idx_bytes, const void *seeds, int seed_bytes,
+                     int64_t C, const void *cache_indptr, int64_t nnz,
+                     void *cache_indices, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHMT_H_ */

@@ -1,0 +1,77 @@
+"""ctypes bindings of the C ABI declared in include/shmt.h.
+
+Thin and explicit: pointers are passed as integers (tensor.data_ptr()), the
+stream as the raw hipStream_t of torch's current stream. The library must
+have been built (python -m shmtensor_amd.build); there is no fallback path.
+"""
+import ctypes
+import os
+
+from .build import LIB_PATH
+
+_c = ctypes
+_vp, _i64, _int, _dbl = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_double
+
+SIGNATURES = {
+    "shmt_abi_version": (_int, []),
+    "shmt_last_error": (_c.c_char_p, []),
+    "shmt_host_register": (_int, [_vp, _i64]),
+    "shmt_host_unregister": (_int, [_vp]),
+    "shmt_host_devptr": (_int, [_vp, _c.POINTER(_vp)]),
+    "shmt_hashmap_capacity": (_i64, [_i64, _dbl]),
+    "shmt_hashmap_table_bytes": (_i64, [_i64, _dbl, _int, _int]),
+    "shmt_hashmap_create": (_int, [_c.POINTER(_vp), _vp, _vp, _i64, _int, _int, _dbl, _vp, _i64, _vp]),
+    "shmt_hashmap_query": (_int, [_vp, _vp, _int, _i64, _vp, _vp]),
+    "shmt_hashmap_key_bytes": (_int, [_vp]),
+    "shmt_hashmap_val_bytes": (_int, [_vp]),
+    "shmt_hashmap_size": (_i64, [_vp]),
+    "shmt_hashmap_destroy": (None, [_vp]),
+    "shmt_fetch": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
+    "shmt_set": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
+    "shmt_scan_tmp_bytes": (_i64, [_i64]),
+    "shmt_exclusive_scan": (_int, [_vp, _i64, _int, _vp, _i64, _vp]),
+    "shmt_inclusive_scan_i32": (_int, [_vp, _i64, _vp, _i64, _vp]),
+    "shmt_relabel_scratch_bytes": (_i64, [_i64]),
+    "shmt_relabel": (_int, [_vp, _i64, _int, _vp, _i64, _vp, _vp, _vp, _vp]),
+    "shmt_sample_plan_bytes": (_i64, [_i64]),
+    "shmt_sample_plan": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _i64, _int, _vp, _vp, _i64, _vp, _vp]),
+    "shmt_sample_pick": (_int, [_vp, _vp, _int, _vp, _int, _i64, _i64, _int, _vp, _int, _vp, _vp,
+                                _c.c_uint64, _c.c_uint32, _vp]),
+    "shmt_subcsr_plan": (_int, [_vp, _int, _vp, _int, _i64, _vp, _vp, _i64, _vp, _vp]),
+    "shmt_subcsr_copy": (_int, [_vp, _vp, _int, _int, _vp, _int, _i64, _vp, _i64, _vp, _vp]),
+}
+
+_lib = None
+
+
+class ShmtError(RuntimeError):
+    pass
+
+
+def load():
+    """Load libshmt.so (after torch, so that both share one HIP runtime)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ShmtError("libshmt.so is not built: run `python -m shmtensor_amd.build`")
+    import torch  # noqa: F401  (loads the HIP runtime this library must share)
+    lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.shmt_abi_version() != 1:
+        raise ShmtError("libshmt.so ABI version mismatch")
+    _lib = lib
+    return lib
+
+
+def check(rc):
+    if rc != 0:
+        raise ShmtError(load().shmt_last_error().decode() or "shmt error %d" % rc)
+
+
+def current_stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream

@@ -1,0 +1,290 @@
+// Static hashmap: build and bulk query.
+// Replaces pycuco::CUCOHashmap (include/cuco_hashmap.cuh:49-93 in the
+// ShmTensor tree): same contract (immutable id -> value map, -1 for absent),
+// own bucketed layout and wavefront-cooperative probing (see hashmap_dev.h).
+#include <math.h>
+#include <stdlib.h>
+
+#include "common.h"
+#include "hashmap.h"
+#include "hashmap_dev.h"
+#include "launchers.h"
+
+namespace shmt {
+
+static int64_t slots_needed(int64_t n, double lf) {
+  // Honour the requested load factor but always leave at least one empty slot
+  // so that a probe for an absent key terminates before wrapping around.
+  int64_t cap = shmt_hashmap_capacity(n, lf);
+  if (cap < n + 1) cap = n + 1;
+  return cap;
+}
+
+static int format_for(int key_bytes, int val_bytes) {
+  return (key_bytes == 4 && val_bytes == 4) ? kSlot8 : kSlot16;
+}
+
+static int64_t buckets_for(int64_t n, double lf, int fmt) {
+  int64_t slots_per_bucket = kBucketBytes / fmt;
+  int64_t slots = slots_needed(n, lf);
+  return (slots + slots_per_bucket - 1) / slots_per_bucket;
+}
+
+// ---- kernels ---------------------------------------------------------------
+
+// Group insert of one (key, value) into the wide table. All 8 lanes of the
+// probe group call with the same arguments.
+__device__ __forceinline__ void group_insert16(uint64_t *table, uint32_t nbuckets,
+                                               int64_t key, int64_t val) {
+  const int sub = lane_id() & (kProbeGroup - 1);
+  const int gbase = lane_id() & ~(kProbeGroup - 1);
+  uint32_t b = reduce_range(hash_id(key), nbuckets);
+  uint32_t probes = 0;
+  while (probes < nbuckets) {
+    uint64_t *slot = table + (static_cast<size_t>(b) * kProbeGroup + sub) * 2;
+    // Fresh (L2-coherent) read of the slot key: another workgroup may have
+    // claimed it since this CU last cached the line.
+    int64_t k = static_cast<int64_t>(
+        __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    if (group_ballot<kProbeGroup>(k == key)) return;  // duplicate key: first one wins
+    uint64_t em = group_ballot<kProbeGroup>(k == -1);
+    if (!em) {
+      b = (b + 1 == nbuckets) ? 0 : b + 1;
+      ++probes;
+      continue;
+    }
+    const int target = __builtin_ctzll(em);
+    int64_t old = 0;
+    if (sub == target) {
+      unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long *>(slot),
+                                          ~0ull, static_cast<unsigned long long>(key));
+      old = static_cast<int64_t>(prev);
+      if (old == -1) slot[1] = static_cast<uint64_t>(val);
+    }
+    old = shfl64(old, gbase + target);
+    if (old == -1 || old == key) return;
+    // lost the race for that slot to a different key: look at the bucket again
+  }
+}
+
+// Narrow table: each lane owns two 8-byte {key,value} words and claims one
+// with a single 64-bit compare-and-swap.
+__device__ __forceinline__ void group_insert8(uint64_t *table, uint32_t nbuckets,
+                                              int32_t key, int32_t val) {
+  const int sub = lane_id() & (kProbeGroup - 1);
+  const int gbase = lane_id() & ~(kProbeGroup - 1);
+  uint32_t b = reduce_range(hash_id(static_cast<int64_t>(key)), nbuckets);
+  const uint64_t word = (static_cast<uint64_t>(static_cast<uint32_t>(val)) << 32) |
+                        static_cast<uint32_t>(key);
+  uint32_t probes = 0;
+  while (probes < nbuckets) {
+    uint64_t *slot = table + (static_cast<size_t>(b) * kProbeGroup + sub) * 2;
+    uint64_t w0 = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t w1 = __hip_atomic_load(slot + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool match = static_cast<int32_t>(static_cast<uint32_t>(w0)) == key ||
+                 static_cast<int32_t>(static_cast<uint32_t>(w1)) == key;
+    if (group_ballot<kProbeGroup>(match)) return;
+    bool e0 = (w0 == ~0ull), e1 = (w1 == ~0ull);
+    uint64_t em = group_ballot<kProbeGroup>(e0 || e1);
+    if (!em) {
+      b = (b + 1 == nbuckets) ? 0 : b + 1;
+      ++probes;
+      continue;
+    }
+    const int target = __builtin_ctzll(em);
+    int64_t old = 0;
+    if (sub == target) {
+      unsigned long long prev = atomicCAS(
+          reinterpret_cast<unsigned long long *>(slot + (e0 ? 0 : 1)), ~0ull,
+          static_cast<unsigned long long>(word));
+      old = static_cast<int64_t>(prev);
+    }
+    old = shfl64(old, gbase + target);
+    if (old == -1 || static_cast<int32_t>(static_cast<uint32_t>(static_cast<uint64_t>(old))) == key)
+      return;
+  }
+}
+
+// One wave takes 64 consecutive (key, value) pairs with coalesced loads; in
+// step j the probe group g inserts pair g*8+j, so 8 inserts proceed per wave
+// at a time and every bucket read is a full-line transaction.
+template <int FMT>
+__global__ __launch_bounds__(256) void hashmap_insert_kernel(
+    uint64_t *table, uint32_t nbuckets, const void *keys, const void *vals,
+    int64_t n, int key_bytes, int val_bytes) {
+  const int lane = lane_id();
+  const int gbase = lane & ~(kProbeGroup - 1);
+  const int64_t waves_per_block = blockDim.x / kWave;
+  int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + threadIdx.x / kWave;
+  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
+  for (int64_t base = wave * kWave; base < n; base += nwaves * kWave) {
+    int64_t i = base + lane;
+    int64_t mykey = -1, myval = -1;
+    if (i < n) {
+      mykey = load_int(keys, i, key_bytes);
+      myval = load_int(vals, i, val_bytes);
+    }
+#pragma unroll 1
+    for (int j = 0; j < kProbeGroup; ++j) {
+      int64_t k = shfl64(mykey, gbase + j);
+      int64_t v = shfl64(myval, gbase + j);
+      if (base + gbase + j < n) {
+        if (FMT == kSlot16)
+          group_insert16(table, nbuckets, k, v);
+        else
+          group_insert8(table, nbuckets, static_cast<int32_t>(k), static_cast<int32_t>(v));
+      }
+    }
+  }
+}
+
+// Bulk query: a wave owns 64 consecutive requests. The eight bucket loads of
+// a probe group (one per step) are all issued before the first is examined,
+// which keeps 8 KiB of table reads in flight per wave; results are gathered
+// back to the lane that loaded the request, so request reads and result
+// writes are both fully coalesced.
+template <int FMT>
+__global__ __launch_bounds__(256) void hashmap_query_kernel(
+    MapView m, const void *req, int req_bytes, void *out, int out_bytes, int64_t n) {
+  const int lane = lane_id();
+  const int sub = lane & (kProbeGroup - 1);
+  const int gbase = lane & ~(kProbeGroup - 1);
+  const int64_t waves_per_block = blockDim.x / kWave;
+  int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + threadIdx.x / kWave;
+  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
+  for (int64_t base = wave * kWave; base < n; base += nwaves * kWave) {
+    const int64_t i = base + lane;
+    int64_t mykey = -1;  // tail lanes look up the sentinel, which resolves to -1
+    if (i < n) mykey = map_key(m, load_int(req, i, req_bytes));
+    int64_t key[kProbeGroup];
+    uint32_t bkt[kProbeGroup];
+    uint4 frag[kProbeGroup];
+#pragma unroll
+    for (int j = 0; j < kProbeGroup; ++j) {
+      key[j] = shfl64(mykey, gbase + j);
+      bkt[j] = map_bucket(m, key[j]);
+      frag[j] = m.buckets[static_cast<size_t>(bkt[j]) * kProbeGroup + sub];
+    }
+    int64_t myres = -1;
+#pragma unroll
+    for (int j = 0; j < kProbeGroup; ++j) {
+      int64_t val = -1;
+      if (!probe_step<FMT>(frag[j], key[j], &val)) {
+        // first bucket was full of other keys: continue along the probe sequence
+        uint32_t b = bkt[j];
+        for (uint32_t probes = 1; probes < m.nbuckets; ++probes) {
+          b = (b + 1 == m.nbuckets) ? 0 : b + 1;
+          uint4 f = m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
+          if (probe_step<FMT>(f, key[j], &val)) break;
+        }
+      }
+      if (sub == j) myres = val;
+    }
+    if (i < n) store_int(out, i, out_bytes, myres);
+  }
+}
+
+}  // namespace shmt
+
+using namespace shmt;
+
+extern "C" {
+
+int64_t shmt_hashmap_capacity(int64_t n, double load_factor) {
+  if (n < 0 || !(load_factor > 0.0)) return -1;
+  return static_cast<int64_t>(ceil(static_cast<double>(n) / load_factor));
+}
+
+int64_t shmt_hashmap_table_bytes(int64_t n, double load_factor, int key_bytes, int val_bytes) {
+  if (n < 0 || !(load_factor > 0.0) || !(load_factor <= 1.0) || !width_ok(key_bytes) ||
+      !width_ok(val_bytes)) {
+    set_error("shmt_hashmap_table_bytes: bad arguments (n=%lld, load_factor=%g, key_bytes=%d, val_bytes=%d)",
+              static_cast<long long>(n), load_factor, key_bytes, val_bytes);
+    return -1;
+  }
+  return buckets_for(n, load_factor, format_for(key_bytes, val_bytes)) * kBucketBytes;
+}
+
+int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys, const void *vals, int64_t n,
+                        int key_bytes, int val_bytes, double load_factor, void *table_mem,
+                        int64_t table_bytes, void *stream) {
+  SHMT_REQUIRE(out != nullptr, "shmt_hashmap_create: out is null");
+  *out = nullptr;
+  SHMT_REQUIRE(n >= 0, "shmt_hashmap_create: n must be >= 0");
+  SHMT_REQUIRE(width_ok(key_bytes) && width_ok(val_bytes),
+               "shmt_hashmap_create: ID can only be int32 or int64 (key_bytes=%d, val_bytes=%d)",
+               key_bytes, val_bytes);
+  SHMT_REQUIRE(load_factor > 0.0 && load_factor <= 1.0,
+               "shmt_hashmap_create: load_factor must be in (0, 1], got %g", load_factor);
+  SHMT_REQUIRE(n == 0 || (keys != nullptr && vals != nullptr),
+               "shmt_hashmap_create: keys/vals are null");
+  const int fmt = format_for(key_bytes, val_bytes);
+  const int64_t nb = buckets_for(n, load_factor, fmt);
+  SHMT_REQUIRE(nb < (1ll << 31), "shmt_hashmap_create: table too large (%lld buckets)",
+               static_cast<long long>(nb));
+  if (table_mem == nullptr || table_bytes < nb * kBucketBytes) {
+    set_error("shmt_hashmap_create: table_mem too small (%lld < %lld bytes)",
+              static_cast<long long>(table_bytes), static_cast<long long>(nb * kBucketBytes));
+    return SHMT_ENOMEM;
+  }
+  SHMT_REQUIRE((reinterpret_cast<uintptr_t>(table_mem) & 127) == 0,
+               "shmt_hashmap_create: table_mem must be 128-byte aligned");
+
+  hipStream_t s = as_stream(stream);
+  int rc = launch_fill_ones(table_mem, nb * (kBucketBytes / 16), s);
+  if (rc) return rc;
+  if (n > 0) {
+    unsigned grid = grid_for(n, 256);
+    if (fmt == kSlot16)
+      hipLaunchKernelGGL(hashmap_insert_kernel<kSlot16>, dim3(grid), dim3(256), 0, s,
+                         static_cast<uint64_t *>(table_mem), static_cast<uint32_t>(nb), keys,
+                         vals, n, key_bytes, val_bytes);
+    else
+      hipLaunchKernelGGL(hashmap_insert_kernel<kSlot8>, dim3(grid), dim3(256), 0, s,
+                         static_cast<uint64_t *>(table_mem), static_cast<uint32_t>(nb), keys,
+                         vals, n, key_bytes, val_bytes);
+    SHMT_LAUNCH_CHECK();
+  }
+
+  shmt_hashmap *h = static_cast<shmt_hashmap *>(calloc(1, sizeof(shmt_hashmap)));
+  if (h == nullptr) {
+    set_error("shmt_hashmap_create: out of host memory");
+    return SHMT_ENOMEM;
+  }
+  h->view.buckets = static_cast<const uint4 *>(table_mem);
+  h->view.nbuckets = static_cast<uint32_t>(nb);
+  h->view.key32 = (key_bytes == 4);
+  h->fmt = fmt;
+  h->key_bytes = key_bytes;
+  h->val_bytes = val_bytes;
+  h->n = n;
+  h->table_bytes = nb * kBucketBytes;
+  *out = h;
+  return SHMT_OK;
+}
+
+int shmt_hashmap_query(const shmt_hashmap_t *map, const void *requests, int req_bytes,
+                       int64_t n, void *out, void *stream) {
+  SHMT_REQUIRE(map != nullptr, "shmt_hashmap_query: map is null");
+  SHMT_REQUIRE(n >= 0, "shmt_hashmap_query: n must be >= 0");
+  SHMT_REQUIRE(width_ok(req_bytes), "shmt_hashmap_query: ID can only be int32 or int64");
+  if (n == 0) return SHMT_OK;
+  SHMT_REQUIRE(requests != nullptr && out != nullptr, "shmt_hashmap_query: null buffer");
+  unsigned grid = grid_for(n, 256);
+  hipStream_t s = as_stream(stream);
+  if (map->fmt == kSlot16)
+    hipLaunchKernelGGL(hashmap_query_kernel<kSlot16>, dim3(grid), dim3(256), 0, s, map->view,
+                       requests, req_bytes, out, map->val_bytes, n);
+  else
+    hipLaunchKernelGGL(hashmap_query_kernel<kSlot8>, dim3(grid), dim3(256), 0, s, map->view,
+                       requests, req_bytes, out, map->val_bytes, n);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+int shmt_hashmap_key_bytes(const shmt_hashmap_t *map) { return map ? map->key_bytes : 0; }
+int shmt_hashmap_val_bytes(const shmt_hashmap_t *map) { return map ? map->val_bytes : 0; }
+int64_t shmt_hashmap_size(const shmt_hashmap_t *map) { return map ? map->n : 0; }
+void shmt_hashmap_destroy(shmt_hashmap_t *map) { free(map); }
+
+}  // extern "C"

@@ -1,0 +1,93 @@
+// Device-side view of the static hashmap and the cooperative probe used by
+// every kernel that consults it (bulk query, fetch/set, sampling plan).
+//
+// Layout in HBM: the table is an array of 128-byte buckets, one HBM/L2 line
+// each. A probe group of 8 adjacent lanes reads one whole bucket with a
+// single coalesced 16-byte-per-lane load and decides hit / miss / continue
+// with a ballot, so one memory transaction inspects every slot of the line.
+//   wide   (kSlot16): 8 slots {int64 key, int64 value}; used whenever the key
+//                     or the value is 8 bytes wide (4-byte members are
+//                     sign-extended on insert).
+//   narrow (kSlot8) : 16 slots {int32 key, int32 value}; each lane sees two.
+// Empty slots hold key = value = -1 (all bits set). Keys probe buckets
+// linearly from hash(key) and are always placed in the first bucket of their
+// probe sequence that still has a free slot, so a lookup stops at the first
+// bucket that contains either the key or an empty slot.
+#pragma once
+#include "wave.h"
+
+namespace shmt {
+
+enum SlotFormat : int { kSlot16 = 16, kSlot8 = 8 };
+
+constexpr int kProbeGroup = 8;      // lanes that cooperate on one key
+constexpr int kBucketBytes = 128;
+
+struct MapView {
+  const uint4 *buckets;   // nbuckets * 8 uint4
+  uint32_t nbuckets;
+  int key32;              // 1: keys are int32 -> narrow requests before hashing
+};
+
+// Normalise a request to the key domain of the map (what requests.to(key
+// dtype) does in the reference): int32-keyed maps see the low 32 bits,
+// sign-extended.
+__device__ __forceinline__ int64_t map_key(const MapView &m, int64_t req) {
+  return m.key32 ? static_cast<int64_t>(static_cast<int32_t>(req)) : req;
+}
+
+__device__ __forceinline__ uint32_t map_bucket(const MapView &m, int64_t key) {
+  return reduce_range(hash_id(key), m.nbuckets);
+}
+
+// Examine one already-loaded bucket fragment. Returns true when the group is
+// done with this key (value written to *val: the mapped value, or -1 when the
+// bucket proved the key absent); false when the bucket was full of other keys.
+template <int FMT>
+__device__ __forceinline__ bool probe_step(const uint4 frag, int64_t key, int64_t *val) {
+  const int gbase = lane_id() & ~(kProbeGroup - 1);
+  bool match, empty;
+  int64_t v;
+  if (FMT == kSlot16) {
+    int64_t k = static_cast<int64_t>((static_cast<uint64_t>(frag.y) << 32) | frag.x);
+    v = static_cast<int64_t>((static_cast<uint64_t>(frag.w) << 32) | frag.z);
+    match = (k == key);
+    empty = (k == -1);
+  } else {
+    int32_t k32 = static_cast<int32_t>(key);
+    bool m0 = static_cast<int32_t>(frag.x) == k32;
+    bool m1 = static_cast<int32_t>(frag.z) == k32;
+    match = m0 || m1;
+    v = static_cast<int64_t>(static_cast<int32_t>(m0 ? frag.y : frag.w));
+    empty = (frag.x == 0xFFFFFFFFu) || (frag.z == 0xFFFFFFFFu);
+  }
+  uint64_t mm = group_ballot<kProbeGroup>(match);
+  if (mm) {
+    *val = shfl64(v, gbase + __builtin_ctzll(mm));
+    return true;
+  }
+  if (group_ballot<kProbeGroup>(empty)) {
+    *val = -1;
+    return true;
+  }
+  return false;
+}
+
+// Cooperative find: the 8 lanes of an aligned probe group call this with the
+// same (already normalised) key; all of them receive the value or -1. The
+// probe count is bounded by the number of buckets, so a completely full
+// table still terminates.
+template <int FMT>
+__device__ __forceinline__ int64_t group_find(const MapView &m, int64_t key) {
+  const int sub = lane_id() & (kProbeGroup - 1);
+  uint32_t b = map_bucket(m, key);
+  int64_t val = -1;
+  for (uint32_t probes = 0; probes < m.nbuckets; ++probes) {
+    uint4 frag = m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
+    if (probe_step<FMT>(frag, key, &val)) return val;
+    b = (b + 1 == m.nbuckets) ? 0 : b + 1;
+  }
+  return -1;
+}
+
+}  // namespace shmt

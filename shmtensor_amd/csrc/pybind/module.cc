@@ -1,0 +1,452 @@
+// ShmTensorLib: the Python operator surface of the GPU-cache hot path, with
+// the names, argument names, defaults and return structure of the reference
+// module (src/pybind.cc:16-65 in the ShmTensor tree). Host C++ only: every
+// operator validates its tensors, allocates outputs and scratch from torch's
+// caching allocator and calls the C ABI of libshmt.so (include/shmt.h) on
+// torch's current HIP stream. Failures raise RuntimeError; nothing exits.
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <mutex>
+#include <optional>
+#include <unordered_map>
+#include <vector>
+
+#include "shmt.h"
+
+namespace py = pybind11;
+
+namespace {
+
+void check(int rc) { TORCH_CHECK(rc == SHMT_OK, shmt_last_error()); }
+
+void *current_stream() {
+  return static_cast<void *>(c10::hip::getCurrentHIPStream().stream());
+}
+
+void sync_current_stream() { c10::hip::getCurrentHIPStream().synchronize(); }
+
+int id_bytes(const torch::Tensor &t, const char *name) {
+  // the reference aborts with "ID can only be int32 or int64" (include/common.h:29-40)
+  TORCH_CHECK(t.scalar_type() == torch::kInt32 || t.scalar_type() == torch::kInt64, name,
+              ": ID can only be int32 or int64, got ", t.scalar_type());
+  return static_cast<int>(t.element_size());
+}
+
+torch::Tensor cuda_ids(const torch::Tensor &t, const char *name) {
+  TORCH_CHECK(t.is_cuda(), name, " must be a CUDA tensor");
+  id_bytes(t, name);
+  return t.contiguous();
+}
+
+// Address a kernel may dereference for tensor `t`: device tensors as they
+// are, CPU tensors through the device alias of their pinned storage.
+void *device_address(const torch::Tensor &t, const char *name) {
+  if (t.numel() == 0) return t.data_ptr();
+  if (t.is_cuda()) return t.data_ptr();
+  void *dev = nullptr;
+  int rc = shmt_host_devptr(t.data_ptr(), &dev);
+  TORCH_CHECK(rc == SHMT_OK, name,
+              " is a CPU tensor whose memory the GPU cannot address; call pin_memory() on it "
+              "first (",
+              shmt_last_error(), ")");
+  return dev;
+}
+
+// One int64 in pinned host memory that kernels write totals into (nnz, number
+// of unique ids); read after synchronising the stream.
+struct Readback {
+  torch::Tensor host;
+  int64_t *dev = nullptr;
+  int64_t *get() {
+    if (!host.defined()) {
+      host = torch::zeros({16}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+      void *d = nullptr;
+      check(shmt_host_devptr(host.data_ptr(), &d));
+      dev = static_cast<int64_t *>(d);
+    }
+    return dev;
+  }
+  int64_t value() {
+    sync_current_stream();
+    return *static_cast<volatile int64_t *>(host.data_ptr<int64_t>());
+  }
+};
+
+Readback &readback() {
+  static Readback r;
+  return r;
+}
+
+torch::Tensor device_bytes(int64_t nbytes) {
+  return torch::empty({nbytes > 0 ? nbytes : 1},
+                      torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCUDA));
+}
+
+// ---- hashmap ---------------------------------------------------------------
+
+class StaticHashmap {
+ public:
+  StaticHashmap(torch::Tensor keys, torch::Tensor values, double load_factor) {
+    TORCH_CHECK(keys.is_cuda(), "keys must be a CUDA tensor");
+    TORCH_CHECK(values.is_cuda(), "values must be a CUDA tensor");
+    key_type_ = keys.scalar_type();
+    value_type_ = values.scalar_type();
+    const int kb = id_bytes(keys, "keys"), vb = id_bytes(values, "values");
+    TORCH_CHECK(keys.numel() == values.numel(), "keys and values must have the same length");
+    TORCH_CHECK(load_factor > 0.0 && load_factor <= 1.0, "load_factor must be in (0, 1]");
+    keys = keys.contiguous();
+    values = values.contiguous();
+    const int64_t n = keys.numel();
+    capacity_ = shmt_hashmap_capacity(n, load_factor);
+    const int64_t bytes = shmt_hashmap_table_bytes(n, load_factor, kb, vb);
+    TORCH_CHECK(bytes > 0, shmt_last_error());
+    table_ = device_bytes(bytes);
+    memory_usage_ = bytes;
+    check(shmt_hashmap_create(&handle_, keys.data_ptr(), values.data_ptr(), n, kb, vb, load_factor,
+                              table_.data_ptr(), bytes, current_stream()));
+  }
+  ~StaticHashmap() { shmt_hashmap_destroy(handle_); }
+  StaticHashmap(const StaticHashmap &) = delete;
+  StaticHashmap &operator=(const StaticHashmap &) = delete;
+
+  torch::Tensor query(torch::Tensor requests) {
+    TORCH_CHECK(requests.is_cuda(), "requests must be a CUDA tensor");
+    if (requests.scalar_type() != torch::kInt32 && requests.scalar_type() != torch::kInt64)
+      requests = requests.to(key_type_);  // src/cuco_hashmap.cu:29
+    requests = requests.contiguous();
+    torch::Tensor result = torch::empty_like(requests, requests.options().dtype(value_type_));
+    check(shmt_hashmap_query(handle_, requests.data_ptr(), static_cast<int>(requests.element_size()),
+                             requests.numel(), result.data_ptr(), current_stream()));
+    return result;
+  }
+  int64_t capacity() const { return capacity_; }
+  int64_t memory_usage() const { return memory_usage_; }
+  const shmt_hashmap_t *handle() const { return handle_; }
+
+ private:
+  shmt_hashmap_t *handle_ = nullptr;
+  torch::Tensor table_;
+  torch::ScalarType key_type_, value_type_;
+  int64_t capacity_ = 0, memory_usage_ = 0;
+};
+
+// ---- pin / unpin -----------------------------------------------------------
+
+std::mutex g_pin_mutex;
+std::unordered_map<void *, int64_t> g_registered;  // ranges registered in place by pin_memory
+
+// PinMemory, src/cache_feature_fetch.cu:6-9. Registers the tensor's memory in
+// place. Where the driver refuses to register existing memory, the tensor is
+// re-homed instead: its contents move into freshly allocated pinned memory
+// and the same Python tensor object now views that memory.
+void pin_memory(torch::Tensor &data) {
+  TORCH_CHECK(!data.is_cuda(), "data must be a CPU tensor");
+  if (data.numel() == 0) return;
+  TORCH_CHECK(data.is_contiguous(), "data must be contiguous");
+  void *dev = nullptr;
+  if (shmt_host_devptr(data.data_ptr(), &dev) == SHMT_OK) return;  // already addressable
+  if (shmt_host_register(data.data_ptr(), static_cast<int64_t>(data.nbytes())) == SHMT_OK) {
+    std::lock_guard<std::mutex> lock(g_pin_mutex);
+    g_registered[data.data_ptr()] = static_cast<int64_t>(data.nbytes());
+    return;
+  }
+  torch::Tensor pinned = torch::empty_like(data, data.options().pinned_memory(true));
+  pinned.copy_(data);
+  data.set_data(pinned);
+}
+
+// UnpinMemory, src/cache_feature_fetch.cu:11-13.
+void unpin_memory(torch::Tensor &data) {
+  if (data.numel() == 0) return;
+  std::lock_guard<std::mutex> lock(g_pin_mutex);
+  auto it = g_registered.find(data.data_ptr());
+  if (it == g_registered.end()) return;  // pinned at allocation: released with the tensor
+  g_registered.erase(it);
+  check(shmt_host_unregister(data.data_ptr()));
+}
+
+// ---- fetch / set -----------------------------------------------------------
+
+struct RowShape {
+  int64_t row_bytes;
+  std::vector<int64_t> out_sizes;
+};
+
+// Output shape rules of src/cache_feature_fetch.cu:137-163: 1-D data gives
+// [numel]; otherwise [numel, *data.shape[1:]].
+RowShape row_shape(const torch::Tensor &data, int64_t numel) {
+  RowShape r;
+  r.out_sizes.push_back(numel);
+  int64_t dim = 1;
+  for (int64_t i = 1; i < data.dim(); ++i) {
+    dim *= data.size(i);
+    r.out_sizes.push_back(data.size(i));
+  }
+  r.row_bytes = dim * static_cast<int64_t>(data.element_size());
+  return r;
+}
+
+void check_tables(const torch::Tensor &uva_data, const torch::Tensor *gpu_data) {
+  TORCH_CHECK(uva_data.dim() >= 1, "data must have at least one dimension");
+  TORCH_CHECK(uva_data.is_contiguous(), "data must be contiguous");
+  if (gpu_data) {
+    TORCH_CHECK(gpu_data->is_cuda(), "gpu_data must be a CUDA tensor");
+    TORCH_CHECK(gpu_data->is_contiguous(), "gpu_data must be contiguous");
+    TORCH_CHECK(gpu_data->scalar_type() == uva_data.scalar_type(),
+                "uva_data and gpu_data must have the same dtype");
+    TORCH_CHECK(row_shape(*gpu_data, 0).row_bytes == row_shape(uva_data, 0).row_bytes,
+                "uva_data and gpu_data must have the same row shape");
+  }
+}
+
+torch::Tensor fetch_impl(const torch::Tensor &uva_data, const torch::Tensor *gpu_data,
+                         torch::Tensor indices, const StaticHashmap *map,
+                         const torch::Tensor *mask) {
+  check_tables(uva_data, gpu_data);
+  indices = cuda_ids(indices, "indices");
+  const int64_t numel = indices.numel();
+  const RowShape rs = row_shape(uva_data, numel);
+  torch::Tensor output = torch::empty(rs.out_sizes, uva_data.options().device(torch::kCUDA));
+  torch::Tensor m;
+  if (mask) {
+    m = cuda_ids(*mask, "mask");
+    TORCH_CHECK(m.numel() == numel, "mask and indices must have the same length");
+  }
+  if (numel == 0 || rs.row_bytes == 0) return output;
+  check(shmt_fetch(device_address(uva_data, "uva_data"), gpu_data ? gpu_data->data_ptr() : nullptr,
+                   indices.data_ptr(), static_cast<int>(indices.element_size()),
+                   map ? map->handle() : nullptr, mask ? m.data_ptr() : nullptr,
+                   mask ? static_cast<int>(m.element_size()) : 0, output.data_ptr(), numel,
+                   rs.row_bytes, current_stream()));
+  return output;
+}
+
+void set_impl(torch::Tensor &uva_data, torch::Tensor *gpu_data, torch::Tensor indices,
+              torch::Tensor update, const StaticHashmap *map, const torch::Tensor *mask) {
+  check_tables(uva_data, gpu_data);
+  indices = cuda_ids(indices, "indices");
+  const int64_t numel = indices.numel();
+  const RowShape rs = row_shape(uva_data, numel);
+  TORCH_CHECK(update.is_cuda(), "update must be a CUDA tensor");
+  TORCH_CHECK(update.scalar_type() == uva_data.scalar_type(),
+              "update must have the dtype of the data");
+  update = update.contiguous();
+  TORCH_CHECK(update.numel() * static_cast<int64_t>(update.element_size()) == numel * rs.row_bytes,
+              "update must hold one row per index");
+  torch::Tensor m;
+  if (mask) {
+    m = cuda_ids(*mask, "mask");
+    TORCH_CHECK(m.numel() == numel, "mask and indices must have the same length");
+  }
+  if (numel == 0 || rs.row_bytes == 0) return;
+  check(shmt_set(device_address(uva_data, "uva_data"), gpu_data ? gpu_data->data_ptr() : nullptr,
+                 indices.data_ptr(), static_cast<int>(indices.element_size()),
+                 map ? map->handle() : nullptr, mask ? m.data_ptr() : nullptr,
+                 mask ? static_cast<int>(m.element_size()) : 0, update.data_ptr(), numel,
+                 rs.row_bytes, current_stream()));
+}
+
+torch::Tensor uva_fetch(torch::Tensor &data, torch::Tensor &indices) {
+  return fetch_impl(data, nullptr, indices, nullptr, nullptr);
+}
+torch::Tensor cache_fetch(torch::Tensor uva_data, torch::Tensor gpu_data, torch::Tensor indices,
+                          StaticHashmap &hashmap) {
+  return fetch_impl(uva_data, &gpu_data, indices, &hashmap, nullptr);
+}
+torch::Tensor cache_fetch_with_mask(torch::Tensor uva_data, torch::Tensor gpu_data,
+                                    torch::Tensor indices, torch::Tensor mask) {
+  return fetch_impl(uva_data, &gpu_data, indices, nullptr, &mask);
+}
+void uva_set(torch::Tensor &data, torch::Tensor &indices, torch::Tensor &update) {
+  set_impl(data, nullptr, indices, update, nullptr, nullptr);
+}
+void cache_set(torch::Tensor uva_data, torch::Tensor gpu_data, torch::Tensor indices,
+               torch::Tensor update, StaticHashmap &hashmap) {
+  set_impl(uva_data, &gpu_data, indices, update, &hashmap, nullptr);
+}
+void cache_set_with_mask(torch::Tensor uva_data, torch::Tensor gpu_data, torch::Tensor indices,
+                         torch::Tensor update, torch::Tensor mask) {
+  set_impl(uva_data, &gpu_data, indices, update, nullptr, &mask);
+}
+
+// ---- scan --------------------------------------------------------------------
+
+// thrust_scan, src/thrust_scan.cu:9-18: in-place inclusive sum over int32.
+void thrust_scan(torch::Tensor tensor) {
+  TORCH_CHECK(tensor.scalar_type() == torch::kInt32, "thrust_scan expects an int32 tensor");
+  TORCH_CHECK(tensor.is_contiguous(), "tensor must be contiguous");
+  const int64_t n = tensor.numel();
+  if (n == 0) return;
+  const int64_t tmp_bytes = shmt_scan_tmp_bytes(n);
+  torch::Tensor tmp = device_bytes(tmp_bytes);
+  check(shmt_inclusive_scan_i32(device_address(tensor, "tensor"), n, tmp.data_ptr(), tmp_bytes,
+                                current_stream()));
+}
+
+// ---- sampling ------------------------------------------------------------------
+
+constexpr uint64_t kDefaultSeed = 7777;  // src/cache_graph_sampling.cu:204,407
+constexpr int64_t kEagerOutputLimit = 1ll << 27;
+
+std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor &indptr,
+                                                     const torch::Tensor &indices,
+                                                     const torch::Tensor *gpu_indptr,
+                                                     const torch::Tensor *gpu_indices,
+                                                     const StaticHashmap *map, torch::Tensor seeds,
+                                                     int64_t num_picks, bool replace,
+                                                     std::optional<int64_t> seed,
+                                                     int64_t stream_id) {
+  const int pb = id_bytes(indptr, "indptr"), ib = id_bytes(indices, "indices");
+  TORCH_CHECK(indptr.is_contiguous() && indices.is_contiguous(), "CSR arrays must be contiguous");
+  TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0");
+  seeds = cuda_ids(seeds, "seeds");
+  if (map) {
+    TORCH_CHECK(gpu_indptr->is_cuda() && gpu_indices->is_cuda(),
+                "gpu_indptr and gpu_indices must be CUDA tensors");
+    TORCH_CHECK(gpu_indptr->scalar_type() == indptr.scalar_type() &&
+                    gpu_indices->scalar_type() == indices.scalar_type(),
+                "cached CSR must have the dtypes of the full CSR");
+    TORCH_CHECK(gpu_indptr->is_contiguous() && gpu_indices->is_contiguous(),
+                "cached CSR arrays must be contiguous");
+  }
+  const int64_t S = seeds.numel();
+  const auto dev = torch::kCUDA;
+  torch::Tensor sub_indptr = torch::empty({S + 1}, indptr.options().device(dev));
+  const int64_t plan_bytes = shmt_sample_plan_bytes(S);
+  torch::Tensor plan = device_bytes(plan_bytes);
+  Readback &rb = readback();
+  void *stream = current_stream();
+  check(shmt_sample_plan(device_address(indptr, "indptr"), pb,
+                         map ? gpu_indptr->data_ptr() : nullptr, map ? map->handle() : nullptr,
+                         seeds.data_ptr(), static_cast<int>(seeds.element_size()), S, num_picks,
+                         replace, sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, rb.get(),
+                         stream));
+  // Output size is data dependent. When the bound S*k is modest, sample into a
+  // buffer of that size and read the total once at the end (one host sync per
+  // call); otherwise read the total first and allocate exactly.
+  const bool eager = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
+  int64_t nnz = -1;
+  torch::Tensor sub_indices;
+  if (eager) {
+    sub_indices = torch::empty({S * num_picks}, indices.options().device(dev));
+  } else {
+    nnz = rb.value();
+    sub_indices = torch::empty({nnz}, indices.options().device(dev));
+  }
+  check(shmt_sample_pick(device_address(indices, "indices"),
+                         map ? gpu_indices->data_ptr() : nullptr, ib, seeds.data_ptr(),
+                         static_cast<int>(seeds.element_size()), S, num_picks, replace,
+                         sub_indptr.data_ptr(), pb, plan.data_ptr(), sub_indices.data_ptr(),
+                         static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
+                         static_cast<uint32_t>(stream_id), stream));
+  if (eager) {
+    nnz = rb.value();
+    sub_indices = sub_indices.narrow(0, 0, nnz);
+  }
+  return std::make_tuple(sub_indptr, sub_indices);
+}
+
+std::tuple<torch::Tensor, torch::Tensor> csr_sampling(torch::Tensor indptr, torch::Tensor indices,
+                                                      torch::Tensor seeds, int64_t num_picks,
+                                                      bool replace, std::optional<int64_t> seed,
+                                                      int64_t stream_id) {
+  return sample_impl(indptr, indices, nullptr, nullptr, nullptr, seeds, num_picks, replace, seed,
+                     stream_id);
+}
+
+std::tuple<torch::Tensor, torch::Tensor> csr_cache_sampling(
+    torch::Tensor uva_indptr, torch::Tensor uva_indices, torch::Tensor gpu_indptr,
+    torch::Tensor gpu_indices, StaticHashmap &hashmap, torch::Tensor seeds, int64_t num_picks,
+    bool replace, std::optional<int64_t> seed, int64_t stream_id) {
+  return sample_impl(uva_indptr, uva_indices, &gpu_indptr, &gpu_indices, &hashmap, seeds, num_picks,
+                     replace, seed, stream_id);
+}
+
+// CreateCacheCSR, src/cache_graph_sampling.cu:455-492.
+std::tuple<torch::Tensor, torch::Tensor> create_subcsr(torch::Tensor uva_indptr,
+                                                       torch::Tensor uva_indices,
+                                                       torch::Tensor seeds) {
+  const int pb = id_bytes(uva_indptr, "uva_indptr"), ib = id_bytes(uva_indices, "uva_indices");
+  TORCH_CHECK(uva_indptr.is_contiguous() && uva_indices.is_contiguous(),
+              "CSR arrays must be contiguous");
+  seeds = cuda_ids(seeds, "seeds");
+  const int64_t C = seeds.numel();
+  torch::Tensor gpu_indptr = torch::empty({C + 1}, uva_indptr.options().device(torch::kCUDA));
+  const int64_t tmp_bytes = shmt_scan_tmp_bytes(C + 1);
+  torch::Tensor tmp = device_bytes(tmp_bytes);
+  Readback &rb = readback();
+  void *stream = current_stream();
+  void *indptr_dev = device_address(uva_indptr, "uva_indptr");
+  check(shmt_subcsr_plan(indptr_dev, pb, seeds.data_ptr(), static_cast<int>(seeds.element_size()), C,
+                         gpu_indptr.data_ptr(), tmp.data_ptr(), tmp_bytes, rb.get(), stream));
+  const int64_t nnz = rb.value();
+  torch::Tensor gpu_indices = torch::empty({nnz}, uva_indices.options().device(torch::kCUDA));
+  check(shmt_subcsr_copy(indptr_dev, device_address(uva_indices, "uva_indices"), pb, ib,
+                         seeds.data_ptr(), static_cast<int>(seeds.element_size()), C,
+                         gpu_indptr.data_ptr(), nnz, gpu_indices.data_ptr(), stream));
+  return std::make_tuple(gpu_indptr, gpu_indices);
+}
+
+// ---- relabel ---------------------------------------------------------------------
+
+// TensorRelabel, src/tensor_relabel.cu:125-209.
+std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
+    std::vector<torch::Tensor> tensors) {
+  TORCH_CHECK(!tensors.empty(), "tensor_relabel needs at least one tensor");
+  std::vector<int64_t> split_sizes;
+  for (auto &t : tensors) {
+    TORCH_CHECK(t.is_cuda(), "tensor_relabel expects CUDA tensors");
+    split_sizes.push_back(t.numel());
+  }
+  torch::Tensor total = torch::cat(tensors, 0).contiguous();
+  const int eb = id_bytes(total, "tensors");
+  const int64_t N = total.numel();
+  torch::Tensor unique = torch::empty({N}, total.options());
+  torch::Tensor labels = torch::empty({N}, total.options());
+  if (N == 0) return std::make_tuple(unique, labels.split_with_sizes(split_sizes, 0));
+  const int64_t scratch_bytes = shmt_relabel_scratch_bytes(N);
+  torch::Tensor scratch = device_bytes(scratch_bytes);
+  Readback &rb = readback();
+  check(shmt_relabel(total.data_ptr(), N, eb, scratch.data_ptr(), scratch_bytes, unique.data_ptr(),
+                     labels.data_ptr(), rb.get(), current_stream()));
+  const int64_t U = rb.value();
+  return std::make_tuple(unique.narrow(0, 0, U), labels.split_with_sizes(split_sizes, 0));
+}
+
+}  // namespace
+
+PYBIND11_MODULE(ShmTensorLib, m) {
+  m.doc() = "MI355X-native ShmTensor GPU-cache operators (HIP, gfx950)";
+
+  m.def("thrust_scan", &thrust_scan, py::arg("tensor"));
+
+  m.def("pin_memory", &pin_memory, py::arg("data"))
+      .def("unpin_memory", &unpin_memory, py::arg("data"))
+      .def("uva_fetch", &uva_fetch, py::arg("data"), py::arg("indices"))
+      .def("cache_fetch", &cache_fetch, py::arg("uva_data"), py::arg("gpu_data"),
+           py::arg("indices"), py::arg("hashmap"))
+      .def("cache_fetch_with_mask", &cache_fetch_with_mask, py::arg("uva_data"),
+           py::arg("gpu_data"), py::arg("indices"), py::arg("mask"))
+      .def("uva_set", &uva_set, py::arg("data"), py::arg("indices"), py::arg("update"))
+      .def("cache_set", &cache_set, py::arg("uva_data"), py::arg("gpu_data"), py::arg("indices"),
+           py::arg("update"), py::arg("hashmap"))
+      .def("cache_set_with_mask", &cache_set_with_mask, py::arg("uva_data"), py::arg("gpu_data"),
+           py::arg("indices"), py::arg("update"), py::arg("mask"))
+      .def("csr_sampling", &csr_sampling, py::arg("indptr"), py::arg("indices"), py::arg("seeds"),
+           py::arg("num_picks"), py::arg("replace"), py::arg("seed") = py::none(),
+           py::arg("stream_id") = 0)
+      .def("csr_cache_sampling", &csr_cache_sampling, py::arg("uva_indptr"),
+           py::arg("uva_indices"), py::arg("gpu_indptr"), py::arg("gpu_indices"),
+           py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"), py::arg("replace"),
+           py::arg("seed") = py::none(), py::arg("stream_id") = 0)
+      .def("create_subcsr", &create_subcsr, py::arg("uva_indptr"), py::arg("uva_indices"),
+           py::arg("seeds"))
+      .def("tensor_relabel", &tensor_relabel, py::arg("tensors"));
+
+  py::class_<StaticHashmap>(m, "CUCOStaticHashmap")
+      .def(py::init<torch::Tensor, torch::Tensor, double>())
+      .def("query", &StaticHashmap::query)
+      .def("capacity", &StaticHashmap::capacity)
+      .def("memory_usage", &StaticHashmap::memory_usage);
+}

@@ -1,0 +1,487 @@
+// Uniform neighbour sampling over a CSR split between an HBM-resident cache
+// of hot rows and a cold copy in pinned host memory, and construction of that
+// cache. Replaces src/cache_graph_sampling.cu:47-492 in the ShmTensor tree.
+//
+// plan:  probe the cache map for 64 consecutive seeds per wave (8 cooperative
+//        probes at a time), read the two row offsets from the cached or the
+//        cold indptr, derive the output count and prefix-sum the counts in the
+//        same kernel. Up to kPlanSingleMax seeds run in one workgroup (one
+//        launch); beyond that each 1024-seed tile scans locally and two short
+//        kernels add the tile offsets.
+// pick:  a sub-wave group of G >= k lanes owns a seed. Rows with deg <= k are
+//        copied in CSR order. Otherwise the k draws of Floyd's subset
+//        algorithm are generated in parallel (one Philox block per lane) and
+//        resolved in k ballot steps inside the group, so the cost is O(k) per
+//        seed whatever the degree; the reference draws O(deg) numbers per seed
+//        (src/cache_graph_sampling.cu:329-336). k > 64 uses one wave per seed
+//        with the chosen set staged in LDS.
+#include "common.h"
+#include "hashmap.h"
+#include "hashmap_dev.h"
+#include "launchers.h"
+#include "philox.h"
+#include "scan_dev.h"
+
+namespace shmt {
+
+constexpr int kPlanBlock = 1024;
+constexpr int64_t kPlanSingleMax = 4096;
+constexpr int64_t kCachedTag = 1ll << 62;  // plan.begin carries the source in bit 62
+constexpr int kWideMaxPicks = 8192;
+
+struct SeedPlan {
+  int64_t begin;  // first adjacency element, | kCachedTag when it lives in the cache
+  int64_t deg;
+};
+
+struct PlanArgs {
+  const void *indptr;
+  const void *cache_indptr;
+  const void *seeds;
+  void *sub_indptr;
+  SeedPlan *plan;
+  uint64_t *partials;
+  int64_t *nnz_out;
+  MapView map;
+  int64_t S;
+  int64_t k;
+  int ptr_bytes;
+  int seed_bytes;
+  int replace;
+};
+
+// Slot of this lane's seed in the cache map (or -1): the wave's 64 seeds are
+// resolved by its 8 probe groups in 8 steps, result returned to the owner lane.
+template <int FMT>
+__device__ __forceinline__ int64_t wave_lookup(const MapView &m, int64_t node) {
+  const int lane = lane_id();
+  const int sub = lane & (kProbeGroup - 1);
+  const int gbase = lane & ~(kProbeGroup - 1);
+  const int64_t mykey = map_key(m, node);
+  int64_t res = -1;
+#pragma unroll 2
+  for (int j = 0; j < kProbeGroup; ++j) {
+    int64_t v = group_find<FMT>(m, shfl64(mykey, gbase + j));
+    if (sub == j) res = v;
+  }
+  return res;
+}
+
+// MODE 0: no cache; 1: wide map; 2: narrow map.
+template <int MODE>
+__device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
+  // called by whole waves; lanes past S use a harmless key and produce cnt 0
+  const bool live = i < a.S;
+  int64_t node = live ? load_int(a.seeds, i, a.seed_bytes) : -1;
+  int64_t slot = -1;
+  if (MODE == 1) slot = wave_lookup<kSlot16>(a.map, node);
+  if (MODE == 2) slot = wave_lookup<kSlot8>(a.map, node);
+  int64_t cnt = 0;
+  if (live) {
+    int64_t begin, end;
+    if (slot >= 0) {
+      begin = load_int(a.cache_indptr, slot, a.ptr_bytes);
+      end = load_int(a.cache_indptr, slot + 1, a.ptr_bytes);
+    } else {
+      begin = load_int(a.indptr, node, a.ptr_bytes);
+      end = load_int(a.indptr, node + 1, a.ptr_bytes);
+    }
+    const int64_t deg = end - begin;
+    a.plan[i].begin = begin | (slot >= 0 ? kCachedTag : 0);
+    a.plan[i].deg = deg;
+    cnt = a.replace ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
+  }
+  return cnt;
+}
+
+// One workgroup walks all seeds with a running carry and writes final offsets.
+template <int MODE>
+__global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
+  __shared__ uint64_t lds[kPlanBlock / kWave];
+  uint64_t carry = 0;
+  for (int64_t base = 0; base < a.S; base += kPlanBlock) {
+    const int64_t i = base + threadIdx.x;
+    const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, i));
+    uint64_t total;
+    const uint64_t ex = block_exclusive_scan<uint64_t, kPlanBlock>(cnt, lds, &total);
+    if (i < a.S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(carry + ex));
+    carry += total;
+  }
+  if (threadIdx.x == 0) {
+    store_int(a.sub_indptr, a.S, a.ptr_bytes, static_cast<int64_t>(carry));
+    *a.nnz_out = static_cast<int64_t>(carry);
+    __threadfence_system();
+  }
+}
+
+// Multi-workgroup form: tile-local offsets + one total per tile.
+template <int MODE>
+__global__ __launch_bounds__(kPlanBlock) void plan_tile_kernel(PlanArgs a) {
+  __shared__ uint64_t lds[kPlanBlock / kWave];
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kPlanBlock + threadIdx.x;
+  const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, i));
+  uint64_t total;
+  const uint64_t ex = block_exclusive_scan<uint64_t, kPlanBlock>(cnt, lds, &total);
+  if (i < a.S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(ex));
+  if (threadIdx.x == 0) {
+    a.partials[blockIdx.x] = total;
+    if (blockIdx.x == 0) a.partials[gridDim.x] = 0;  // becomes the grand total after the scan
+  }
+}
+
+// Adds the scanned tile offsets to the tile-local offsets. partials holds
+// nb + 1 scanned entries: partials[t] = sum of the tiles before t, and
+// partials[nb] = grand total, which becomes data[n] and *total_out.
+__global__ __launch_bounds__(256) void add_tile_offsets_kernel(void *data, int eb, int64_t n,
+                                                               const uint64_t *partials,
+                                                               int64_t tile, int64_t nb,
+                                                               int64_t *total_out) {
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (; i <= n; i += stride) {
+    if (i < n) {
+      store_int(data, i, eb, load_int(data, i, eb) + static_cast<int64_t>(partials[i / tile]));
+    } else {
+      const int64_t t = static_cast<int64_t>(partials[nb]);
+      store_int(data, n, eb, t);
+      *total_out = t;
+      __threadfence_system();
+    }
+  }
+}
+
+// ---- pick ------------------------------------------------------------------
+
+struct PickArgs {
+  const void *indices;
+  const void *cache_indices;
+  const void *seeds;
+  const void *sub_indptr;
+  const SeedPlan *plan;
+  void *out;
+  int64_t S;
+  int64_t k;
+  uint64_t rng_seed;
+  uint32_t rng_stream;
+  int idx_bytes;
+  int seed_bytes;
+  int ptr_bytes;
+  int replace;
+  int log2_group;  // lanes per seed (narrow kernel)
+};
+
+__device__ __forceinline__ int64_t load_adj(const PickArgs &a, int64_t begin_tagged, int64_t pos) {
+  const void *base = (begin_tagged & kCachedTag) ? a.cache_indices : a.indices;
+  return load_int(base, (begin_tagged & ~kCachedTag) + pos, a.idx_bytes);
+}
+
+// k <= 64: group of G = 2^log2_group >= k lanes per seed.
+__global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
+  const int lane = lane_id();
+  const int G = 1 << a.log2_group;
+  const int gl = lane & (G - 1);
+  const int gbase = lane & ~(G - 1);
+  const int groups_per_wave = kWave >> a.log2_group;
+  const int64_t waves_per_block = blockDim.x / kWave;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + threadIdx.x / kWave;
+  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
+  const int k = static_cast<int>(a.k);
+
+  for (int64_t s0 = wave * groups_per_wave; s0 < a.S; s0 += nwaves * groups_per_wave) {
+    const int64_t s = s0 + (lane >> a.log2_group);
+    if (s >= a.S) continue;  // uniform within the group
+    const SeedPlan p = a.plan[s];
+    const int64_t deg = p.deg;
+    if (deg <= 0) continue;
+    const int64_t optr = load_int(a.sub_indptr, s, a.ptr_bytes);
+    if (a.replace) {
+      if (gl < k) {
+        const int64_t node = load_int(a.seeds, s, a.seed_bytes);
+        const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
+        store_int(a.out, optr + gl, a.idx_bytes, load_adj(a, p.begin, static_cast<int64_t>(r)));
+      }
+    } else if (deg <= k) {
+      if (gl < deg) store_int(a.out, optr + gl, a.idx_bytes, load_adj(a, p.begin, gl));
+    } else {
+      // Floyd: for J = deg-k .. deg-1 draw t in [0, J]; take t unless already
+      // taken, then take J. Draws in parallel, resolution in k ballot steps.
+      const int64_t node = load_int(a.seeds, s, a.seed_bytes);
+      int64_t t = 0;
+      if (gl < k)
+        t = static_cast<int64_t>(sample_draw(a.rng_seed, a.rng_stream, node, gl,
+                                             static_cast<uint64_t>(deg - k + gl + 1)));
+      int64_t mine = -1;
+      for (int step = 0; step < k; ++step) {
+        const int64_t ts = shfl64(t, gbase + step);
+        const bool taken = group_ballot_dyn(gl < step && mine == ts, G) != 0;
+        if (gl == step) mine = taken ? (deg - k + step) : ts;
+      }
+      if (gl < k) store_int(a.out, optr + gl, a.idx_bytes, load_adj(a, p.begin, mine));
+    }
+  }
+}
+
+// k > 64: one wave (= one 64-thread workgroup) per seed, chosen positions in LDS.
+__global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
+  extern __shared__ int64_t chosen[];
+  const int lane = threadIdx.x;
+  const int64_t k = a.k;
+  for (int64_t s = blockIdx.x; s < a.S; s += gridDim.x) {
+    const SeedPlan p = a.plan[s];
+    const int64_t deg = p.deg;
+    if (deg <= 0) continue;
+    const int64_t optr = load_int(a.sub_indptr, s, a.ptr_bytes);
+    const int64_t node = load_int(a.seeds, s, a.seed_bytes);
+    if (a.replace) {
+      for (int64_t j = lane; j < k; j += kWave) {
+        const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(j),
+                                       static_cast<uint64_t>(deg));
+        store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, static_cast<int64_t>(r)));
+      }
+    } else if (deg <= k) {
+      for (int64_t j = lane; j < deg; j += kWave)
+        store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, j));
+    } else {
+      for (int64_t step = 0; step < k; ++step) {
+        const int64_t J = deg - k + step;
+        const int64_t t = static_cast<int64_t>(sample_draw(
+            a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(step), static_cast<uint64_t>(J + 1)));
+        bool taken = false;
+        for (int64_t q = lane; q < step; q += kWave) taken |= (chosen[q] == t);
+        const bool any = __builtin_amdgcn_ballot_w64(taken) != 0;
+        __syncthreads();
+        if (lane == 0) chosen[step] = any ? J : t;
+        __syncthreads();
+      }
+      for (int64_t j = lane; j < k; j += kWave)
+        store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, chosen[j]));
+      __syncthreads();
+    }
+  }
+}
+
+// ---- cached sub-CSR ----------------------------------------------------------
+
+__global__ __launch_bounds__(256) void subcsr_degree_kernel(const void *indptr, int ptr_bytes,
+                                                            const void *seeds, int seed_bytes,
+                                                            int64_t C, void *cache_indptr) {
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (; i <= C; i += stride) {
+    int64_t d = 0;
+    if (i < C) {
+      const int64_t v = load_int(seeds, i, seed_bytes);
+      d = load_int(indptr, v + 1, ptr_bytes) - load_int(indptr, v, ptr_bytes);
+    }
+    store_int(cache_indptr, i, ptr_bytes, d);
+  }
+}
+
+__global__ void copy_total_kernel(const void *data, int eb, int64_t n, int64_t *total_out) {
+  *total_out = load_int(data, n, eb);
+  __threadfence_system();
+}
+
+// Last row r in [lo, hi] with offsets[r] <= e.
+__device__ __forceinline__ int64_t row_of(const void *offsets, int eb, int64_t lo, int64_t hi,
+                                          int64_t e) {
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (load_int(offsets, mid, eb) <= e)
+      lo = mid;
+    else
+      hi = mid - 1;
+  }
+  return lo;
+}
+
+constexpr int kCopyChunk = 256 * 8;
+
+// Element-parallel copy: a workgroup owns a contiguous chunk of the output,
+// brackets the rows that chunk can touch once, and every element then finds
+// its row inside that bracket, so hub rows and empty rows cost the same.
+__global__ __launch_bounds__(256) void subcsr_copy_kernel(const void *indptr, const void *indices,
+                                                          int ptr_bytes, int idx_bytes,
+                                                          const void *seeds, int seed_bytes,
+                                                          int64_t C, const void *cache_indptr,
+                                                          int64_t nnz, void *cache_indices) {
+  __shared__ int64_t bracket[2];
+  const int64_t nchunks = (nnz + kCopyChunk - 1) / kCopyChunk;
+  for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+    const int64_t e0 = c * kCopyChunk;
+    const int64_t e1 = (e0 + kCopyChunk < nnz ? e0 + kCopyChunk : nnz) - 1;
+    if (threadIdx.x < 2)
+      bracket[threadIdx.x] = row_of(cache_indptr, ptr_bytes, 0, C - 1, threadIdx.x == 0 ? e0 : e1);
+    __syncthreads();
+    const int64_t rlo = bracket[0], rhi = bracket[1];
+#pragma unroll 2
+    for (int j = 0; j < 8; ++j) {
+      const int64_t e = e0 + j * 256 + threadIdx.x;
+      if (e <= e1) {
+        const int64_t r = row_of(cache_indptr, ptr_bytes, rlo, rhi, e);
+        const int64_t v = load_int(seeds, r, seed_bytes);
+        const int64_t src = load_int(indptr, v, ptr_bytes) + (e - load_int(cache_indptr, r, ptr_bytes));
+        store_int(cache_indices, e, idx_bytes, load_int(indices, src, idx_bytes));
+      }
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace shmt
+
+using namespace shmt;
+
+extern "C" {
+
+int64_t shmt_sample_plan_bytes(int64_t S) {
+  if (S < 0) return -1;
+  const int64_t nb = (S + kPlanBlock - 1) / kPlanBlock;
+  return S * static_cast<int64_t>(sizeof(SeedPlan)) + (nb + 2) * 8;
+}
+
+int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr,
+                     const shmt_hashmap_t *map, const void *seeds, int seed_bytes, int64_t S,
+                     int64_t k, int replace, void *sub_indptr, void *plan, int64_t plan_bytes,
+                     int64_t *nnz_out, void *stream) {
+  SHMT_REQUIRE(S >= 0, "shmt_sample_plan: S must be >= 0");
+  SHMT_REQUIRE(k >= 0, "shmt_sample_plan: num_picks must be >= 0");
+  SHMT_REQUIRE(width_ok(ptr_bytes) && width_ok(seed_bytes),
+               "shmt_sample_plan: ID can only be int32 or int64");
+  SHMT_REQUIRE(sub_indptr != nullptr && nnz_out != nullptr, "shmt_sample_plan: null output");
+  SHMT_REQUIRE(indptr != nullptr, "shmt_sample_plan: indptr is null");
+  SHMT_REQUIRE(map == nullptr || cache_indptr != nullptr, "shmt_sample_plan: cache_indptr is null");
+  if (S > 0) {
+    SHMT_REQUIRE(seeds != nullptr, "shmt_sample_plan: seeds is null");
+    if (plan == nullptr || plan_bytes < shmt_sample_plan_bytes(S)) {
+      set_error("shmt_sample_plan: plan buffer too small (%lld < %lld bytes)",
+                static_cast<long long>(plan_bytes), static_cast<long long>(shmt_sample_plan_bytes(S)));
+      return SHMT_ENOMEM;
+    }
+    SHMT_REQUIRE((reinterpret_cast<uintptr_t>(plan) & 15) == 0,
+                 "shmt_sample_plan: plan must be 16-byte aligned");
+  }
+  hipStream_t s = as_stream(stream);
+  PlanArgs a;
+  a.indptr = indptr;
+  a.cache_indptr = cache_indptr;
+  a.seeds = seeds;
+  a.sub_indptr = sub_indptr;
+  a.plan = static_cast<SeedPlan *>(plan);
+  a.partials = S > 0 ? reinterpret_cast<uint64_t *>(static_cast<char *>(plan) + S * sizeof(SeedPlan))
+                     : nullptr;
+  a.nnz_out = nnz_out;
+  if (map) a.map = map->view; else a.map = MapView{nullptr, 1, 0};
+  a.S = S;
+  a.k = k;
+  a.ptr_bytes = ptr_bytes;
+  a.seed_bytes = seed_bytes;
+  a.replace = replace ? 1 : 0;
+  const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
+
+  if (S <= kPlanSingleMax) {
+    switch (mode) {
+      case 0: hipLaunchKernelGGL(plan_single_kernel<0>, dim3(1), dim3(kPlanBlock), 0, s, a); break;
+      case 1: hipLaunchKernelGGL(plan_single_kernel<1>, dim3(1), dim3(kPlanBlock), 0, s, a); break;
+      default: hipLaunchKernelGGL(plan_single_kernel<2>, dim3(1), dim3(kPlanBlock), 0, s, a); break;
+    }
+    SHMT_LAUNCH_CHECK();
+    return SHMT_OK;
+  }
+  const int64_t nb = (S + kPlanBlock - 1) / kPlanBlock;
+  SHMT_REQUIRE(nb < (1ll << 31), "shmt_sample_plan: too many seeds");
+  const dim3 grid(static_cast<unsigned>(nb));
+  switch (mode) {
+    case 0: hipLaunchKernelGGL(plan_tile_kernel<0>, grid, dim3(kPlanBlock), 0, s, a); break;
+    case 1: hipLaunchKernelGGL(plan_tile_kernel<1>, grid, dim3(kPlanBlock), 0, s, a); break;
+    default: hipLaunchKernelGGL(plan_tile_kernel<2>, grid, dim3(kPlanBlock), 0, s, a); break;
+  }
+  SHMT_LAUNCH_CHECK();
+  int rc = launch_scan_partials(a.partials, nb + 1, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(add_tile_offsets_kernel, dim3(grid_for(S + 1, 256)), dim3(256), 0, s,
+                     sub_indptr, ptr_bytes, S, a.partials, static_cast<int64_t>(kPlanBlock), nb,
+                     nnz_out);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_bytes,
+                     const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
+                     const void *sub_indptr, int ptr_bytes, const void *plan, void *sub_indices,
+                     uint64_t rng_seed, uint32_t rng_stream, void *stream) {
+  SHMT_REQUIRE(S >= 0 && k >= 0, "shmt_sample_pick: S and num_picks must be >= 0");
+  SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes),
+               "shmt_sample_pick: ID can only be int32 or int64");
+  if (S == 0 || k == 0) return SHMT_OK;
+  SHMT_REQUIRE(indices && seeds && sub_indptr && plan && sub_indices,
+               "shmt_sample_pick: null buffer");
+  SHMT_REQUIRE(k <= kWideMaxPicks, "shmt_sample_pick: num_picks > %d is not supported", kWideMaxPicks);
+  PickArgs a;
+  a.indices = indices;
+  a.cache_indices = cache_indices ? cache_indices : indices;
+  a.seeds = seeds;
+  a.sub_indptr = sub_indptr;
+  a.plan = static_cast<const SeedPlan *>(plan);
+  a.out = sub_indices;
+  a.S = S;
+  a.k = k;
+  a.rng_seed = rng_seed;
+  a.rng_stream = rng_stream;
+  a.idx_bytes = idx_bytes;
+  a.seed_bytes = seed_bytes;
+  a.ptr_bytes = ptr_bytes;
+  a.replace = replace ? 1 : 0;
+  a.log2_group = 0;
+  hipStream_t s = as_stream(stream);
+  if (k <= kWave) {
+    int lg = 2;
+    while ((1 << lg) < k) ++lg;
+    a.log2_group = lg;
+    const int seeds_per_block = 4 * (kWave >> lg);
+    hipLaunchKernelGGL(pick_narrow_kernel, dim3(grid_for(S, seeds_per_block)), dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(pick_wide_kernel, dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
+                       static_cast<size_t>(k) * sizeof(int64_t), s, a);
+  }
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+int shmt_subcsr_plan(const void *indptr, int ptr_bytes, const void *seeds, int seed_bytes,
+                     int64_t C, void *cache_indptr, void *tmp, int64_t tmp_bytes,
+                     int64_t *nnz_out, void *stream) {
+  SHMT_REQUIRE(C >= 0, "shmt_subcsr_plan: C must be >= 0");
+  SHMT_REQUIRE(width_ok(ptr_bytes) && width_ok(seed_bytes),
+               "shmt_subcsr_plan: ID can only be int32 or int64");
+  SHMT_REQUIRE(indptr && cache_indptr && nnz_out, "shmt_subcsr_plan: null buffer");
+  SHMT_REQUIRE(C == 0 || seeds != nullptr, "shmt_subcsr_plan: seeds is null");
+  hipStream_t s = as_stream(stream);
+  hipLaunchKernelGGL(subcsr_degree_kernel, dim3(grid_for(C + 1, 256)), dim3(256), 0, s, indptr,
+                     ptr_bytes, seeds, seed_bytes, C, cache_indptr);
+  SHMT_LAUNCH_CHECK();
+  int rc = shmt_exclusive_scan(cache_indptr, C + 1, ptr_bytes, tmp, tmp_bytes, stream);
+  if (rc) return rc;
+  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(1), 0, s, cache_indptr, ptr_bytes, C, nnz_out);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+int shmt_subcsr_copy(const void *indptr, const void *indices, int ptr_bytes, int idx_bytes,
+                     const void *seeds, int seed_bytes, int64_t C, const void *cache_indptr,
+                     int64_t nnz, void *cache_indices, void *stream) {
+  SHMT_REQUIRE(C >= 0 && nnz >= 0, "shmt_subcsr_copy: C and nnz must be >= 0");
+  SHMT_REQUIRE(width_ok(ptr_bytes) && width_ok(idx_bytes) && width_ok(seed_bytes),
+               "shmt_subcsr_copy: ID can only be int32 or int64");
+  if (C == 0 || nnz == 0) return SHMT_OK;
+  SHMT_REQUIRE(indptr && indices && seeds && cache_indptr && cache_indices,
+               "shmt_subcsr_copy: null buffer");
+  const int64_t nchunks = (nnz + kCopyChunk - 1) / kCopyChunk;
+  hipLaunchKernelGGL(subcsr_copy_kernel, dim3(grid_for(nchunks, 1)), dim3(256), 0, as_stream(stream),
+                     indptr, indices, ptr_bytes, idx_bytes, seeds, seed_bytes, C, cache_indptr, nnz,
+                     cache_indices);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+}  // extern "C"
