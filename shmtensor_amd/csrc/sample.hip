@@ -27,7 +27,7 @@ namespace shmt {
 constexpr int kPlanBlock = 1024;
 constexpr int64_t kPlanSingleMax = 4096;
 constexpr int64_t kCachedTag = 1ll << 62;  // plan.begin carries the source in bit 62
-constexpr int kWideMaxPicks = 8192;
+constexpr int kWideMaxPicks = 8192;  // chosen set of 8 B entries must fit 64 KiB of LDS
 
 struct SeedPlan {
   int64_t begin;  // first adjacency element, | kCachedTag when it lives in the cache
@@ -221,9 +221,13 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
   }
 }
 
-// k > 64: one wave (= one 64-thread workgroup) per seed, chosen positions in LDS.
+// k > 64: one wave (= one 64-thread workgroup) per seed. The chosen positions
+// are staged in LDS when k fits (IN_LDS), otherwise in the seed's own output
+// segment, which is overwritten by the gathered neighbours at the end
+// (positions are < deg and therefore fit the index width).
+template <bool IN_LDS>
 __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
-  extern __shared__ int64_t chosen[];
+  extern __shared__ int64_t chosen_lds[];
   const int lane = threadIdx.x;
   const int64_t k = a.k;
   for (int64_t s = blockIdx.x; s < a.S; s += gridDim.x) {
@@ -247,14 +251,26 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
         const int64_t t = static_cast<int64_t>(sample_draw(
             a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(step), static_cast<uint64_t>(J + 1)));
         bool taken = false;
-        for (int64_t q = lane; q < step; q += kWave) taken |= (chosen[q] == t);
+        for (int64_t q = lane; q < step; q += kWave) {
+          const int64_t c = IN_LDS ? chosen_lds[q] : load_int(a.out, optr + q, a.idx_bytes);
+          taken |= (c == t);
+        }
         const bool any = __builtin_amdgcn_ballot_w64(taken) != 0;
-        __syncthreads();
-        if (lane == 0) chosen[step] = any ? J : t;
-        __syncthreads();
+        if (lane == 0) {
+          if (IN_LDS)
+            chosen_lds[step] = any ? J : t;
+          else
+            store_int(a.out, optr + step, a.idx_bytes, any ? J : t);
+        }
+        __syncthreads();  // single-wave workgroup: orders the staging write before the next reads
       }
-      for (int64_t j = lane; j < k; j += kWave)
-        store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, chosen[j]));
+      for (int64_t j0 = 0; j0 < k; j0 += kWave) {
+        const int64_t j = j0 + lane;
+        int64_t c = 0;
+        if (j < k) c = IN_LDS ? chosen_lds[j] : load_int(a.out, optr + j, a.idx_bytes);
+        __syncthreads();
+        if (j < k) store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, c));
+      }
       __syncthreads();
     }
   }
@@ -416,7 +432,6 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
   if (S == 0 || k == 0) return SHMT_OK;
   SHMT_REQUIRE(indices && seeds && sub_indptr && plan && sub_indices,
                "shmt_sample_pick: null buffer");
-  SHMT_REQUIRE(k <= kWideMaxPicks, "shmt_sample_pick: num_picks > %d is not supported", kWideMaxPicks);
   PickArgs a;
   a.indices = indices;
   a.cache_indices = cache_indices ? cache_indices : indices;
@@ -440,9 +455,11 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
     a.log2_group = lg;
     const int seeds_per_block = 4 * (kWave >> lg);
     hipLaunchKernelGGL(pick_narrow_kernel, dim3(grid_for(S, seeds_per_block)), dim3(256), 0, s, a);
-  } else {
-    hipLaunchKernelGGL(pick_wide_kernel, dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
+  } else if (k <= kWideMaxPicks) {
+    hipLaunchKernelGGL(pick_wide_kernel<true>, dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
                        static_cast<size_t>(k) * sizeof(int64_t), s, a);
+  } else {
+    hipLaunchKernelGGL(pick_wide_kernel<false>, dim3(grid_for(S, 1, 256 * 32)), dim3(kWave), 0, s, a);
   }
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;

@@ -1,0 +1,169 @@
+"""Feature fetch / set through the HBM cache: the assertions of
+example/test_cache_fetch.py:24-105 and example/test_cache_set.py:24-147, the CPU
+oracle on the same inputs, and a routing check in which cache rows differ from
+host rows so that hit/miss selection itself is observable."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _cache(capi, data, ids, lf=0.8, val_dtype=torch.int64):
+    gpu_data = data[ids.cpu()].cuda()
+    h = capi.CUCOStaticHashmap(ids, torch.arange(ids.numel(), device="cuda", dtype=val_dtype), lf)
+    return gpu_data, h
+
+
+@pytest.mark.parametrize("shape", [(100,), (100, 100, 100)])
+def test_reference_unit_cases(capi, shape):
+    # example/test_cache_fetch.py:24-105
+    torch.manual_seed(0)
+    data = (torch.arange(100).float() if len(shape) == 1 else torch.randn(shape)).pin_memory()
+    indices = torch.randint(0, 100, (10,)).long().cuda()
+    assert torch.equal(capi.uva_fetch(data, indices), data.cuda()[indices])
+    ids = torch.randint(0, 100, (50,)).long().unique().cuda()
+    gpu_data, h = _cache(capi, data, ids)
+    query = torch.randint(0, 100, (20,)).long().cuda()
+    expect = data[query.cpu()].cuda()
+    assert torch.equal(capi.cache_fetch(data, gpu_data, query, h), expect)
+    assert torch.equal(capi.cache_fetch_with_mask(data, gpu_data, query, h.query(query)), expect)
+
+
+@pytest.mark.parametrize("D,dtype", [(1, torch.float32), (3, torch.float32), (7, torch.int8),
+                                      (100, torch.float32), (128, torch.float32), (129, torch.float32),
+                                      (128, torch.float16), (128, torch.bfloat16), (256, torch.float32),
+                                      (10000, torch.float32), (33, torch.int16), (5, torch.float64)])
+@pytest.mark.parametrize("idx_dtype", [torch.int32, torch.int64])
+def test_fetch_matches_oracle_with_distinct_cache_rows(capi, oracle, D, dtype, idx_dtype):
+    rng = np.random.default_rng(D * 7 + idx_dtype.itemsize)
+    n = 3000 if D <= 256 else 300
+    raw = torch.from_numpy(rng.integers(-120, 120, size=(n, D)).astype(np.int8 if dtype == torch.int8 else np.float32))
+    data = raw.to(dtype).pin_memory()
+    ids = torch.from_numpy(rng.choice(n, size=n // 4, replace=False)).cuda()
+    gpu_data = (data[ids.cpu()].float() + 1).to(dtype).cuda()       # differs from the host rows
+    h = capi.CUCOStaticHashmap(ids, torch.arange(ids.numel(), device="cuda"), 0.8)
+    q = torch.from_numpy(rng.integers(0, n, size=1501)).to(idx_dtype).cuda()
+    view = torch.int16 if dtype in (torch.float16, torch.bfloat16) else dtype    # compare raw bit patterns
+    ref_h = oracle.Hashmap(ids.cpu().numpy(), np.arange(ids.numel()), 0.8)
+    expect = oracle.fetch(data.view(view).numpy(), gpu_data.cpu().view(view).numpy(), q.cpu().numpy(), hashmap=ref_h)
+    got = capi.cache_fetch(data, gpu_data, q, h)
+    assert got.dtype == dtype and got.shape == (q.numel(), D)
+    assert np.array_equal(got.cpu().view(view).numpy(), expect)
+    for mask_dtype in (torch.int32, torch.int64):
+        got_m = capi.cache_fetch_with_mask(data, gpu_data, q, h.query(q).to(mask_dtype))
+        assert np.array_equal(got_m.cpu().view(view).numpy(), expect)
+    assert torch.equal(capi.uva_fetch(data, q).cpu().view(view), data.view(view)[q.cpu().long()])
+
+
+@pytest.mark.parametrize("hit", [0.0, 1.0])
+def test_all_miss_and_all_hit(capi, hit):
+    torch.manual_seed(3)
+    data = torch.randn(5000, 128).pin_memory()
+    ids = torch.randperm(5000)[:2000].cuda()
+    gpu_data, h = _cache(capi, data, ids)
+    cached = torch.zeros(5000, dtype=torch.bool)
+    cached[ids.cpu()] = True
+    pool = torch.nonzero(cached if hit else ~cached).flatten()
+    q = pool[torch.randint(0, pool.numel(), (4096,))].cuda()
+    assert ((h.query(q) >= 0).float().mean().item()) == hit
+    assert torch.equal(capi.cache_fetch(data, gpu_data, q, h), data[q.cpu()].cuda())
+
+
+def test_device_resident_table_and_empty_query(capi):
+    data = torch.randn(1000, 16).cuda()      # the "uva" table may live on the device too
+    q = torch.randint(0, 1000, (100,)).cuda()
+    assert torch.equal(capi.uva_fetch(data, q), data[q])
+    out = capi.uva_fetch(data, torch.zeros(0, dtype=torch.int64).cuda())
+    assert out.shape == (0, 16)
+
+
+def test_unpinned_host_tensor_is_an_error(capi):
+    data = torch.randn(100, 8)
+    with pytest.raises(RuntimeError, match="pin_memory"):
+        capi.uva_fetch(data, torch.tensor([1]).cuda())
+
+
+@pytest.mark.parametrize("shape", [(100_000,), (100_000, 128)])
+def test_set_then_fetch_reference_case(capi, shape):
+    # example/test_cache_set.py:24-147, sizes scaled down 10x
+    torch.manual_seed(1)
+    n = shape[0]
+    data = torch.randn(shape).pin_memory()
+    for size in [10, 1000, 100_000]:
+        idx = torch.randint(0, n, (size,)).long().cuda().unique()
+        upd = torch.randn((idx.numel(),) + shape[1:]).cuda()
+        capi.uva_set(data, idx, upd)
+        assert torch.equal(capi.uva_fetch(data, idx), upd)
+    ids = torch.randperm(n).long().cuda()[: int(n * 0.7)]
+    gpu_data, h = _cache(capi, data, ids)
+    for size in [10, 1000, 100_000]:
+        idx = torch.randint(0, n, (size,)).long().cuda().unique()
+        upd = torch.randn((idx.numel(),) + shape[1:]).cuda()
+        capi.cache_set(data, gpu_data, idx, upd, h)
+        assert torch.equal(capi.cache_fetch(data, gpu_data, idx, h), upd)
+        upd2 = torch.randn_like(upd)
+        capi.cache_set_with_mask(data, gpu_data, idx, upd2, h.query(idx))
+        assert torch.equal(capi.cache_fetch_with_mask(data, gpu_data, idx, h.query(idx)), upd2)
+
+
+def test_set_final_state_matches_oracle(capi, oracle):
+    rng = np.random.default_rng(11)
+    host = rng.standard_normal((4000, 24)).astype(np.float32)
+    ids = rng.choice(4000, size=1500, replace=False)
+    gpu = host[ids] + 1
+    q = np.unique(rng.integers(0, 4000, size=3000))
+    upd = rng.standard_normal((q.size, 24)).astype(np.float32)
+    data_t = torch.from_numpy(host.copy()).pin_memory()
+    gpu_t = torch.from_numpy(gpu.copy()).cuda()
+    h = capi.CUCOStaticHashmap(torch.from_numpy(ids).cuda(), torch.arange(ids.size).cuda(), 0.8)
+    capi.cache_set(data_t, gpu_t, torch.from_numpy(q).cuda(), torch.from_numpy(upd).cuda(), h)
+    torch.cuda.synchronize()
+    ref_h = oracle.Hashmap(ids, np.arange(ids.size), 0.8)
+    oracle.set_rows(host, gpu, q, upd, hashmap=ref_h)
+    assert np.array_equal(data_t.numpy(), host)        # hits leave the host row stale, misses write it
+    assert np.array_equal(gpu_t.cpu().numpy(), gpu)
+
+
+def test_config1_small_fetch(capi, oracle):
+    """BASELINE config 1: 200,000 x 128 f32 table, 50,000 cached ids, 65,536 uniform queries."""
+    torch.manual_seed(0)
+    table = torch.randn(200_000, 128).pin_memory()
+    ids = torch.randperm(200_000)[:50_000]
+    gpu_data = table[ids].cuda()
+    h = capi.CUCOStaticHashmap(ids.cuda(), torch.arange(50_000).cuda(), 0.8)
+    q = torch.randint(0, 200_000, (65_536,))
+    out = capi.cache_fetch(table, gpu_data, q.cuda(), h)
+    hit = (h.query(q.cuda()) >= 0).float().mean().item()
+    assert 0.23 < hit < 0.27
+    ref_h = oracle.Hashmap(ids.numpy(), np.arange(50_000), 0.8)
+    expect = oracle.fetch(table.numpy(), gpu_data.cpu().numpy(), q.numpy(), hashmap=ref_h)
+    assert np.array_equal(out.cpu().numpy(), expect)
+    assert torch.equal(out.cpu(), torch.index_select(table, 0, q))
+
+
+def test_direct_c_abi_fetch(cabi):
+    """Same operator called straight through the C ABI (raw pointers, sizes, stream)."""
+    import ctypes
+    lib = cabi.load()
+    data = torch.randn(1000, 64).cuda()
+    idx = torch.randint(0, 1000, (333,), dtype=torch.int32).cuda()
+    out = torch.empty(333, 64).cuda()
+    cabi.check(lib.shmt_fetch(data.data_ptr(), None, idx.data_ptr(), 4, None, None, 0, out.data_ptr(),
+                              333, 256, cabi.current_stream()))
+    assert torch.equal(out, data[idx.long()])
+    keys = torch.arange(0, 2000, 2).cuda()
+    vals = torch.arange(1000).cuda()
+    nbytes = lib.shmt_hashmap_table_bytes(1000, 0.8, 8, 8)
+    table = torch.empty(nbytes, dtype=torch.uint8).cuda()
+    hnd = ctypes.c_void_p()
+    cabi.check(lib.shmt_hashmap_create(ctypes.byref(hnd), keys.data_ptr(), vals.data_ptr(), 1000, 8, 8, 0.8,
+                                       table.data_ptr(), nbytes, cabi.current_stream()))
+    req = torch.arange(2000).cuda()
+    res = torch.empty(2000, dtype=torch.int64).cuda()
+    cabi.check(lib.shmt_hashmap_query(hnd, req.data_ptr(), 8, 2000, res.data_ptr(), cabi.current_stream()))
+    expect = torch.where(req % 2 == 0, req // 2, torch.full_like(req, -1))
+    assert torch.equal(res, expect)
+    assert lib.shmt_hashmap_create(ctypes.byref(ctypes.c_void_p()), keys.data_ptr(), vals.data_ptr(), 1000, 8, 8,
+                                   0.8, table.data_ptr(), 128, None) == -4          # table too small
+    lib.shmt_hashmap_destroy(hnd)

@@ -1,0 +1,104 @@
+"""Scan and relabel on the GPU: reference KAT (example/test_cache_sampling.py:129-140),
+the CPU oracle, closed forms and the edge cases of the capacity rule."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import load_golden
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 1023, 1024, 1025, 8192, 65536, 65537, 1_000_003, 5_000_000])
+def test_thrust_scan_inclusive_int32(capi, oracle, n):
+    rng = np.random.default_rng(n)
+    a = rng.integers(-1000, 1000, size=n).astype(np.int32)
+    t = torch.from_numpy(a.copy()).cuda()
+    capi.thrust_scan(t)
+    assert np.array_equal(t.cpu().numpy(), oracle.inclusive_scan_i32(a))
+    assert np.array_equal(t.cpu().numpy(), np.cumsum(a, dtype=np.int32))
+
+
+def test_thrust_scan_wraps_and_pinned_host(capi):
+    a = torch.full((3_000_000,), 2**30, dtype=torch.int32).cuda()
+    capi.thrust_scan(a)
+    assert np.array_equal(a.cpu().numpy(), np.cumsum(np.full(3_000_000, 2**30, np.int32), dtype=np.int32))
+    h = torch.arange(100, dtype=torch.int32).pin_memory()      # device-addressable host memory
+    capi.thrust_scan(h)
+    torch.cuda.synchronize()
+    assert torch.equal(h, torch.cumsum(torch.arange(100), 0).int())
+
+
+@pytest.mark.parametrize("bytes_", [4, 8])
+@pytest.mark.parametrize("n", [1, 100, 4096, 65536, 65537, 2_000_000])
+def test_exclusive_scan_c_abi(cabi, oracle, bytes_, n):
+    lib = cabi.load()
+    dt = np.int32 if bytes_ == 4 else np.int64
+    rng = np.random.default_rng(n + bytes_)
+    a = rng.integers(0, 2**30 if bytes_ == 4 else 2**61, size=n + 1).astype(dt)     # wraps
+    t = torch.from_numpy(a.copy()).cuda()
+    tmp_bytes = lib.shmt_scan_tmp_bytes(n + 1)
+    tmp = torch.empty(max(tmp_bytes, 1), dtype=torch.uint8).cuda()
+    cabi.check(lib.shmt_exclusive_scan(t.data_ptr(), n + 1, bytes_, tmp.data_ptr(), tmp_bytes, cabi.current_stream()))
+    assert np.array_equal(t.cpu().numpy(), oracle.exclusive_scan(a))
+
+
+def test_relabel_reference_kat(capi):
+    g = load_golden("relabel_kat.json")
+    u, labels = capi.tensor_relabel([torch.tensor(x).cuda() for x in g["inputs"]])
+    assert u.tolist() == g["unique"]
+    assert [l.tolist() for l in labels] == g["labels"]
+    assert isinstance(labels, list) and u.dtype == torch.int64
+
+
+@pytest.mark.parametrize("n", [1, 2, 7, 8, 9, 255, 256, 257, 2047, 2048, 2049, 100_000, 3_000_000])
+@pytest.mark.parametrize("dt", [np.int32, np.int64])
+def test_relabel_matches_oracle(capi, oracle, n, dt):
+    rng = np.random.default_rng(n)
+    hi = 2**31 if dt == np.int64 else 0
+    a = (rng.integers(0, max(2, n // 3), size=n) + hi).astype(dt)
+    b = rng.integers(0, max(2, n // 3), size=n // 2 + 1).astype(dt)
+    u, (la, lb) = capi.tensor_relabel([torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()])
+    eu, (ea, eb) = oracle.relabel([a, b])
+    assert u.dtype == la.dtype == torch.from_numpy(a).dtype
+    assert np.array_equal(u.cpu().numpy(), eu)
+    assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
+
+
+def test_relabel_mixed_dtypes_prefix_property(capi, oracle):
+    # the dataloader's call: [int64 seeds, int32 sub_indices] (python/shmtensor/sampling.py:137-138)
+    rng = np.random.default_rng(5)
+    seeds = rng.choice(100_000, size=1024, replace=False).astype(np.int64)
+    nbrs = rng.integers(0, 100_000, size=15_000).astype(np.int32)
+    u, (ls, ln) = capi.tensor_relabel([torch.from_numpy(seeds).cuda(), torch.from_numpy(nbrs).cuda()])
+    assert u.dtype == torch.int64 and ln.dtype == torch.int64
+    assert torch.equal(u[:1024].cpu(), torch.from_numpy(seeds))
+    assert torch.equal(ls.cpu(), torch.arange(1024))
+    assert torch.equal(u[ln].cpu(), torch.from_numpy(nbrs).long())
+    eu, (es, en) = oracle.relabel([seeds, nbrs])
+    assert np.array_equal(u.cpu().numpy(), eu) and np.array_equal(ln.cpu().numpy(), en)
+
+
+def test_relabel_degenerate_inputs(capi):
+    u, (l,) = capi.tensor_relabel([torch.full((1000,), 7).cuda()])
+    assert u.tolist() == [7] and l.tolist() == [0] * 1000
+    x = torch.randperm(5000).cuda()
+    u, (l,) = capi.tensor_relabel([x])
+    assert torch.equal(u, x) and torch.equal(l, torch.arange(5000).cuda())
+    u, (l1, l2) = capi.tensor_relabel([torch.zeros(0, dtype=torch.int64).cuda(), torch.tensor([3, 3, 1]).cuda()])
+    assert u.tolist() == [3, 1] and l1.numel() == 0 and l2.tolist() == [0, 0, 1]
+    u, (l,) = capi.tensor_relabel([torch.zeros(0, dtype=torch.int64).cuda()])
+    assert u.numel() == 0 and l.numel() == 0
+
+
+def test_relabel_full_size_properties(capi):
+    """N = 16M (config 5 scale): labels invert unique, unique is duplicate free
+    and ordered by first occurrence (checked through the monotone first-index property)."""
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randint(0, 4_000_000, (16_000_000,), device="cuda", generator=g)
+    u, (l,) = capi.tensor_relabel([x])
+    assert torch.equal(u[l], x)
+    assert u.numel() == torch.unique(x).numel()
+    first = torch.full((u.numel(),), x.numel(), device="cuda", dtype=torch.int64)
+    first.scatter_reduce_(0, l, torch.arange(x.numel(), device="cuda"), reduce="amin")
+    assert bool((first[1:] > first[:-1]).all())
