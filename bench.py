@@ -1,0 +1,352 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPU-cache hot path on one MI355X.
+
+Headline ("step"): one cache_fetch call over one batch of BASELINE config 4 —
+100,000,000 x 128 fp16 feature table in pinned host memory, the 40,000,000
+lowest ids cached in HBM, 1,048,576 int64 queries drawn from Zipf(1.1) over the
+node rank. value = feature bytes delivered per second (Q * row_bytes / t), with
+queries, cache and map resident in HBM when the timed region starts.
+
+The same JSON line carries the roofline of the fetch kernel, the CPU baseline
+(oracle gather on the host cores, bounded sample) and, under "extra", the
+all-hit / all-miss fetch rates, the cache_set pass, the hashmap microbenchmark
+(config 2) and cached 3-hop sampling with relabel (config 3) beside its CPU
+baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,sampling]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gpu_time_ms(fn, iters, warmup=3):
+    """Median / mean / min of per-call durations measured with events on the
+    current stream (the stream every operator launches on)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(iters):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    times.sort()
+    return {"median": times[len(times) // 2], "mean": sum(times) / len(times), "min": times[0]}
+
+
+# ---------------------------------------------------------------------------
+# config 4 (+ all-hit / all-miss / set): feature fetch
+
+def build_feature_table(n_rows, dim, n_cached, seed):
+    """fp16 N(0,1) table generated chunk-wise on the GPU and copied into pinned
+    host memory; the first n_cached rows also stay in HBM as the cache."""
+    import torch
+    host = torch.empty((n_rows, dim), dtype=torch.float16, pin_memory=True)
+    cache = torch.empty((n_cached, dim), dtype=torch.float16, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    chunk = 4_000_000
+    for lo in range(0, n_rows, chunk):
+        hi = min(n_rows, lo + chunk)
+        block = torch.randn((hi - lo, dim), device="cuda", generator=g).to(torch.float16)
+        host[lo:hi].copy_(block, non_blocking=True)
+        if lo < n_cached:
+            c_hi = min(hi, n_cached)
+            cache[lo:c_hi].copy_(block[: c_hi - lo])
+        torch.cuda.synchronize()
+    return host, cache
+
+
+def bench_fetch(capi, args, result):
+    import numpy as np
+    import torch
+    from shmtensor_amd.synthetic import zipf_ranks
+    from oracle import oracle as orc
+
+    N, D, C, Q = args.fetch_rows, 128, int(args.fetch_rows * 0.4), 1 << 20
+    R = D * 2
+    t0 = time.time()
+    host, cache = build_feature_table(N, D, C, seed=2)
+    log("[fetch] table %d x %d fp16 (%.1f GB pinned), cache %d rows (%.2f GB HBM): %.1f s"
+        % (N, D, N * R / 1e9, C, C * R / 1e9, time.time() - t0))
+    keys = torch.arange(C, device="cuda")
+    hmap = capi.CUCOStaticHashmap(keys, keys.clone(), 0.8)
+    del keys
+    nb = 8
+    batches = [zipf_ranks(Q, N, 1.1, seed=100 + i) for i in range(nb)]
+    hit_rate = float((batches[0] < C).float().mean())
+
+    # correctness of the timed operator on the timed input (bit patterns)
+    out = capi.cache_fetch(host, cache, batches[0], hmap)
+    ref = torch.index_select(host.view(torch.int16), 0, batches[0].cpu())
+    assert torch.equal(out.cpu().view(torch.int16), ref), "cache_fetch differs from index_select"
+    del out, ref
+
+    W, K = args.warmup, args.steps
+    for i in range(W):
+        capi.cache_fetch(host, cache, batches[i % nb], hmap)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+    t0 = time.perf_counter()
+    for i in range(K):
+        ev[i][0].record()
+        capi.cache_fetch(host, cache, batches[i % nb], hmap)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = sum(a.elapsed_time(b) for a, b in ev) / K
+    ms_per_step = wall * 1e3 / K
+    value = Q * R / (ms_per_step * 1e-3) / 1e9
+    algo_bytes = Q * (2 * R + 8)
+    achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
+    result.update({
+        "value": round(value, 2), "ms_per_step": round(ms_per_step, 4),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "rows_kernel<u32x4, map16, fetch>", "kernel_ms": round(kern_ms, 4),
+                     "bytes_per_launch": algo_bytes},
+    })
+    result["config"].update({"workload": "config 4: cache_fetch, %d x %d fp16 table pinned, %d rows cached, "
+                             "Q=%d Zipf(1.1)" % (N, D, C, Q), "hit_rate": round(hit_rate, 4),
+                             "row_bytes": R, "queries_per_step": Q})
+    extra = result["extra"]
+
+    # pinned host -> device copy ceiling (DMA engine), the miss-path roofline
+    nbytes = min(1 << 30, host.numel() * 2)
+    rows = nbytes // R
+    dst = torch.empty((rows, D), dtype=torch.float16, device="cuda")
+    t = gpu_time_ms(lambda: dst.copy_(host[:rows], non_blocking=True), 10)
+    h2d = nbytes / (t["median"] * 1e-3) / 1e9
+    del dst
+    extra["pinned_h2d_copy_GBs"] = round(h2d, 2)
+
+    # streaming ceiling of the same kernel: sequential ids on the HBM table (a plain copy)
+    qs = torch.arange(Q, device="cuda")
+    t = gpu_time_ms(lambda: capi.uva_fetch(cache, qs), 30)
+    extra["sequential_copy_same_kernel"] = {"ms": round(t["median"], 4),
+                                            "algorithmic_GBs": round(algo_bytes / t["median"] / 1e6, 1)}
+    # all-hit: uniform queries over the cached ids (no locality), HBM bound
+    qh = torch.randint(0, C, (Q,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
+    t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qh, hmap), 30)
+    a = algo_bytes / (t["median"] * 1e-3) / 1e9
+    extra["fetch_all_hit"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(a, 1),
+                              "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 1)}
+    tm = gpu_time_ms(lambda: capi.cache_fetch_with_mask(host, cache, qh, qh), 30)
+    a = algo_bytes / (tm["median"] * 1e-3) / 1e9
+    extra["fetch_all_hit_with_mask"] = {"ms": round(tm["median"], 4), "algorithmic_GBs": round(a, 1),
+                                        "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
+    # all-miss: uniform queries over the uncached ids, host-link bound
+    qm = torch.randint(C, N, (Q,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
+    t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qm, hmap), 10)
+    m = Q * R / (t["median"] * 1e-3) / 1e9
+    extra["fetch_all_miss"] = {"ms": round(t["median"], 4), "host_link_GBs": round(m, 2),
+                               "frac_of_pinned_copy": round(m / h2d, 4)}
+    t = gpu_time_ms(lambda: capi.uva_fetch(host, qm), 10)
+    m = Q * R / (t["median"] * 1e-3) / 1e9
+    extra["uva_fetch"] = {"ms": round(t["median"], 4), "host_link_GBs": round(m, 2),
+                          "frac_of_pinned_copy": round(m / h2d, 4)}
+
+    # cache_set pass of config 4: 262,144 unique cached rows
+    ns = 262_144
+    sidx = torch.randperm(C, device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))[:ns].contiguous()
+    upd = torch.randn((ns, D), device="cuda").to(torch.float16)
+    t = gpu_time_ms(lambda: capi.cache_set(host, cache, sidx, upd, hmap), 30)
+    assert torch.equal(capi.cache_fetch(host, cache, sidx, hmap), upd)
+    a = ns * (2 * R + 8) / (t["median"] * 1e-3) / 1e9
+    extra["cache_set_262144"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(a, 1),
+                                 "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
+
+    # CPU baseline: the reference's cpu_fetch idiom is data[query.cpu()] (example/test_cache_fetch.py:138);
+    # timed here as the oracle's OpenMP gather and as torch.index_select on the same batch
+    if not args.no_cpu:
+        q_cpu = batches[0].cpu().numpy()
+        host_np = host.view(torch.int16).numpy()
+        threads = orc.num_threads()
+        orc.fetch(host_np, None, q_cpu)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < args.cpu_seconds:
+            orc.fetch(host_np, None, q_cpu)
+            reps += 1
+        cpu_t = (time.perf_counter() - t0) / reps
+        qt = batches[0].cpu()
+        torch.index_select(host, 0, qt)
+        t1 = time.perf_counter()
+        for _ in range(5):
+            torch.index_select(host, 0, qt)
+        torch_t = (time.perf_counter() - t1) / 5
+        result["cpu_baseline"] = {
+            "value": round(Q * R / cpu_t / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "%d passes of one 1,048,576-query Zipf batch over the same host table (oracle gather, "
+                      "OpenMP); torch.index_select with %d threads on the same batch: %.2f GB/s"
+                      % (reps, torch.get_num_threads(), Q * R / torch_t / 1e9)}
+    del host, cache, hmap
+
+
+# ---------------------------------------------------------------------------
+# config 2: static hashmap
+
+def bench_hashmap(capi, args, result):
+    import torch
+    n, nq = 4_194_304, 16_777_216
+    g = torch.Generator(device="cuda").manual_seed(22)
+    keys = torch.unique(torch.randint(0, 1 << 40, (n + n // 8,), device="cuda", generator=g))
+    keys = keys[torch.randperm(keys.numel(), device="cuda", generator=g)][:n].contiguous()
+    vals = torch.arange(n, device="cuda")
+    pick = torch.randint(0, n, (nq // 2,), device="cuda", generator=g)
+    non = torch.randint(0, 1 << 40, (nq // 2,), device="cuda", generator=g) | (1 << 41)
+    perm = torch.randperm(nq, device="cuda", generator=g)
+    req = torch.cat([keys[pick], non])[perm].contiguous()
+    expect = torch.cat([pick, torch.full_like(non, -1)])[perm]
+    del non, perm, pick
+    tb = gpu_time_ms(lambda: capi.CUCOStaticHashmap(keys, vals, 0.5), 10)
+    h = capi.CUCOStaticHashmap(keys, vals, 0.5)
+    assert torch.equal(h.query(req), expect)
+    tq = gpu_time_ms(lambda: h.query(req), 30)
+    result["extra"]["hashmap_config2"] = {
+        "build_ms": round(tb["median"], 4), "build_Mkeys_s": round(n / tb["median"] / 1e3, 1),
+        "query_ms": round(tq["median"], 4), "query_Mkeys_s": round(nq / tq["median"] / 1e3, 1),
+        "query_algorithmic_GBs": round(nq * 32 / tq["median"] / 1e6, 1),
+        "query_frac_hbm_peak": round(nq * 32 / tq["median"] / 1e6 / HBM_PEAK_GBS, 4),
+        "table_bytes": h.memory_usage()}
+    if not args.no_cpu:
+        from oracle import oracle as orc
+        k_np, v_np, r_np = keys.cpu().numpy(), vals.cpu().numpy(), req[: nq // 4].cpu().numpy()
+        t0 = time.perf_counter()
+        m = orc.Hashmap(k_np, v_np, 0.5)
+        tbuild = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        m.query(r_np)
+        tquery = time.perf_counter() - t0
+        result["extra"]["hashmap_config2"]["cpu_oracle"] = {
+            "build_Mkeys_s": round(n / tbuild / 1e6, 2), "query_Mkeys_s": round(r_np.size / tquery / 1e6, 2),
+            "cores": orc.num_threads(), "sample": "build 4,194,304 keys (1 thread); query 4,194,304 requests (OpenMP)"}
+
+
+# ---------------------------------------------------------------------------
+# config 3: cached 3-hop sampling + relabel
+
+def bench_sampling(capi, args, result):
+    import numpy as np
+    import torch
+    from shmtensor_amd.synthetic import rmat_csr
+    t0 = time.time()
+    indptr_d, indices_d = rmat_csr(args.sampling_scale, 30, seed=1)
+    n = indptr_d.numel() - 1
+    indptr = indptr_d.cpu().pin_memory()
+    indices = indices_d.cpu().pin_memory()
+    deg = indptr_d[1:] - indptr_d[:-1]
+    hot = torch.sort(deg, descending=True, stable=True).indices[: n * 3 // 10].contiguous()
+    del indptr_d, indices_d
+    gp, gi = capi.create_subcsr(indptr, indices, hot)
+    hmap = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel(), device="cuda"), 0.8)
+    log("[sampling] R-MAT scale %d: %d nodes, %d edges, cache %d rows / %d edges (%.0f %% of edges): %.1f s"
+        % (args.sampling_scale, n, indices.numel(), hot.numel(), gi.numel(),
+           100.0 * gi.numel() / indices.numel(), time.time() - t0))
+    fanouts, S, nbatch = [15, 10, 5], 1024, args.sampling_batches
+    g = torch.Generator(device="cuda").manual_seed(33)
+    seed_batches = [torch.randperm(n, device="cuda", generator=g)[:S].contiguous() for _ in range(nbatch)]
+
+    def run_batch(seeds, b):
+        edges = 0
+        for hop, k in enumerate(reversed(fanouts)):       # python/shmtensor/sampling.py:128
+            sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, hmap, seeds, k, False, seed=7777 + b,
+                                             stream_id=hop)
+            uniq, (_, rel) = capi.tensor_relabel([seeds, si])
+            edges += si.numel()
+            seeds = uniq
+        return edges
+
+    for b in range(3):
+        run_batch(seed_batches[b], b)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    edges = sum(run_batch(seed_batches[b], b) for b in range(nbatch))
+    torch.cuda.synchronize()
+    gpu_t = time.perf_counter() - t0
+    res = {"graph": "R-MAT scale %d ef 30 symmetrised: %d nodes, %d edges; top 30 %% by degree cached"
+                    % (args.sampling_scale, n, indices.numel()),
+           "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
+           "edges_per_batch": edges // nbatch, "ms_per_batch": round(gpu_t * 1e3 / nbatch, 4),
+           "sampled_edges_per_s": round(edges / gpu_t, 1)}
+    if not args.no_cpu:
+        from oracle import oracle as orc
+        ip, ix = indptr.numpy(), indices.numpy().astype(np.int64)
+        nb_cpu = min(nbatch, 20)
+        t0 = time.perf_counter()
+        cpu_edges = 0
+        for b in range(nb_cpu):
+            seeds = seed_batches[b].cpu().numpy()
+            for hop, k in enumerate(reversed(fanouts)):
+                sp, si = orc.sample(ip, ix, seeds, k, False, seed=7777 + b, stream=hop, algo="reservoir")
+                uniq, _ = orc.relabel([seeds, si])
+                cpu_edges += si.size
+                seeds = uniq
+        cpu_t = time.perf_counter() - t0
+        res["cpu_baseline"] = {"sampled_edges_per_s": round(cpu_edges / cpu_t, 1), "cores": orc.num_threads(),
+                               "kind": "port", "sample": "%d batches, Algorithm-R sampler + hash relabel (oracle, OpenMP)" % nb_cpu}
+        res["speedup_vs_cpu"] = round((edges / gpu_t) / (cpu_edges / cpu_t), 2)
+    result["extra"]["sampling_config3"] = res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workloads", default="fetch,hashmap,sampling")
+    ap.add_argument("--fetch-rows", type=int, default=100_000_000)
+    ap.add_argument("--sampling-scale", type=int, default=21)
+    ap.add_argument("--sampling-batches", type=int, default=50)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import shmtensor_amd
+    capi = shmtensor_amd.install_aliases()        # raises if the HIP extension is missing
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+
+    result = {"metric": "cache-fetch GB/s + sampled edges/sec on 1 MI355X; % of HBM / host-link roofline",
+              "value": None, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+              "dtype": "u8", "data": "synthetic", "config": {"workload": None},
+              "roofline": None, "cpu_baseline": None,
+              "extra": {"host_threads": {"os_cpu_count": os.cpu_count(), "torch": torch.get_num_threads(),
+                                         "OMP_NUM_THREADS": os.environ.get("OMP_NUM_THREADS")}}}
+    todo = args.workloads.split(",")
+    if "fetch" in todo:
+        bench_fetch(capi, args, result)
+        torch.cuda.empty_cache()
+    if "hashmap" in todo:
+        bench_hashmap(capi, args, result)
+        torch.cuda.empty_cache()
+    if "sampling" in todo:
+        bench_sampling(capi, args, result)
+        s = result["extra"]["sampling_config3"]
+        result["sampled_edges_per_s"] = s["sampled_edges_per_s"]
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,10 +1,27 @@
 // Feature row gather (fetch) and scatter (set) through the HBM cache.
 // Replaces the twelve kernels of src/cache_feature_fetch.cu:15-224 and
 // src/cache_feature_set.cu:6-207 in the ShmTensor tree with one templated
-// kernel: a sub-wave group of L lanes owns one row, the first 8 lanes of the
-// group resolve the row's cache slot (cooperative hashmap probe, or a mask
-// load), and the group then moves the row with the widest vector access the
-// row size and the base pointers allow (16 bytes per lane when aligned).
+// kernel.
+//
+// A workgroup of four waves owns a block tile; each wave owns up to 64
+// consecutive rows of it.
+// Phase 1 (lane per row): coalesced load of the ids, then the cache slot of
+// every row at once: the wave's eight probe groups look the ids up
+// cooperatively (one 128-byte bucket line per probe, all probes of a round in
+// flight together), or the mask is loaded. Each lane ends up holding the
+// source (fetch) or destination (set) address of its row.
+// Phase 2 (sub-wave group of L lanes per row): row addresses are broadcast
+// with lane shuffles and rows are moved with the widest vector access the row
+// size and base pointers allow (16 bytes per lane when aligned), eight rows
+// per group in flight at a time. The dependent chain id -> bucket -> row is
+// paid once per 64 rows instead of once per row.
+// Hit/miss separation (fetch through a map or mask): loads return to a wave
+// in issue order, so one host-link read (microseconds, plus address
+// translation of a cold host page) would hold back every HBM row issued
+// after it. The rows of a block tile that missed the cache are therefore
+// compacted into an LDS list and handed to the first wave(s) of the
+// workgroup, which issue them all at once; the other waves only ever touch
+// HBM and retire quickly, so few wave slots wait on the host link.
 #include "common.h"
 #include "hashmap.h"
 #include "hashmap_dev.h"
@@ -24,62 +41,179 @@ struct RowArgs {
   int64_t row_bytes;
   int idx_bytes;
   int mask_bytes;
-  int log2_lanes;      // lanes per row = 1 << log2_lanes, in [8, 64]
+  int log2_lanes;      // lanes per row in phase 2 = 1 << log2_lanes, in [8, 64]
+  int log2_tile;       // rows per wave tile = 1 << log2_tile, in [64 / lanes, 64]
 };
 
-template <typename VT, bool SET>
-__device__ __forceinline__ void move_vec(char *table_row, char *dense_row, int64_t off) {
-  if (SET)
-    *reinterpret_cast<VT *>(table_row + off) = *reinterpret_cast<const VT *>(dense_row + off);
-  else
-    *reinterpret_cast<VT *>(dense_row + off) = *reinterpret_cast<const VT *>(table_row + off);
-}
+// Native vector types (the non-temporal builtins do not take HIP's struct vectors).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-template <typename VT, int MODE, bool SET>
-__global__ __launch_bounds__(256) void rows_kernel(RowArgs a) {
+constexpr int kRowsBlock = 256;   // threads per workgroup
+constexpr int kRowsWaves = kRowsBlock / kWave;
+constexpr int kRowsInFlight = 8;  // rows a lane group moves concurrently (single-vector rows)
+constexpr int kMissPerWave = 32;  // miss rows one wave takes before another wave is drafted
+
+// Moves rows [0, count) of a work list. Entry p is described by its table-side
+// row address and its dense row number: taken from the lanes of this wave
+// (FROM_LDS = false: lane p holds the address, dense row = dense_base + p, a
+// zero address marks a row to skip) or from the workgroup's LDS miss list.
+// Must be called by all 64 lanes.
+template <typename VT, bool SET, bool ONE_VEC, bool FROM_LDS>
+__device__ __forceinline__ void move_rows_list(const RowArgs &a, int count, int64_t my_table_row,
+                                               int64_t dense_base, const int64_t *lds_addr,
+                                               const int *lds_row, int list_begin) {
   const int lane = lane_id();
   const int L = 1 << a.log2_lanes;
   const int gl = lane & (L - 1);
   const int grp = lane >> a.log2_lanes;
-  const int rows_per_wave = kWave >> a.log2_lanes;
-  const int64_t waves_per_block = blockDim.x / kWave;
-  const int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + threadIdx.x / kWave;
-  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
+  const int rows_per_step = kWave >> a.log2_lanes;
   const int64_t R = a.row_bytes;
   const int64_t step = static_cast<int64_t>(L) * sizeof(VT);
+  const int64_t my_off = static_cast<int64_t>(gl) * sizeof(VT);
 
-  for (int64_t row0 = wave * rows_per_wave; row0 < a.Q; row0 += nwaves * rows_per_wave) {
-    const int64_t row = row0 + grp;
-    if (row >= a.Q) continue;  // uniform within the row group
-    const int64_t idx = load_int(a.indices, row, a.idx_bytes);
+  if (ONE_VEC) {
+    // row_bytes <= L * sizeof(VT): one vector per lane per row
+    const bool in = my_off < R;
+    for (int r0 = 0; r0 < count; r0 += kRowsInFlight * rows_per_step) {
+      VT v[kRowsInFlight];
+      char *trow[kRowsInFlight];
+      // shuffles run with every lane active: a lane can only read the address
+      // held by a lane that takes part in the same instruction
+#pragma unroll
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int p = r0 + u * rows_per_step + grp;
+        if (FROM_LDS)
+          trow[u] = p < count ? reinterpret_cast<char *>(lds_addr[list_begin + p]) : nullptr;
+        else
+          trow[u] = reinterpret_cast<char *>(shfl64(my_table_row, p & (kWave - 1)));
+      }
+#pragma unroll
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int p = r0 + u * rows_per_step + grp;
+        if (p < count && in && trow[u] != nullptr) {
+          if (SET) {
+            const int64_t drow = FROM_LDS ? lds_row[list_begin + p] : p;
+            v[u] = __builtin_nontemporal_load(
+                reinterpret_cast<const VT *>(a.dense + (dense_base + drow) * R + my_off));
+          } else {
+            v[u] = *reinterpret_cast<const VT *>(trow[u] + my_off);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kRowsInFlight; ++u) {
+        const int p = r0 + u * rows_per_step + grp;
+        if (p < count && in && trow[u] != nullptr) {
+          if (SET) {
+            *reinterpret_cast<VT *>(trow[u] + my_off) = v[u];
+          } else {
+            const int64_t drow = FROM_LDS ? lds_row[list_begin + p] : p;
+            __builtin_nontemporal_store(
+                v[u], reinterpret_cast<VT *>(a.dense + (dense_base + drow) * R + my_off));
+          }
+        }
+      }
+    }
+  } else {
+    for (int r0 = 0; r0 < count; r0 += rows_per_step) {
+      const int p = r0 + grp;
+      char *trow;
+      if (FROM_LDS)
+        trow = p < count ? reinterpret_cast<char *>(lds_addr[list_begin + p]) : nullptr;
+      else
+        trow = reinterpret_cast<char *>(shfl64(my_table_row, p & (kWave - 1)));
+      if (p >= count || trow == nullptr) continue;
+      const int64_t drow_i = FROM_LDS ? lds_row[list_begin + p] : p;
+      char *drow = a.dense + (dense_base + drow_i) * R;
+      const char *src = SET ? drow : trow;
+      char *dst = SET ? trow : drow;
+      int64_t off = my_off;
+      for (; off + 3 * step < R; off += 4 * step) {
+        const VT v0 = *reinterpret_cast<const VT *>(src + off);
+        const VT v1 = *reinterpret_cast<const VT *>(src + off + step);
+        const VT v2 = *reinterpret_cast<const VT *>(src + off + 2 * step);
+        const VT v3 = *reinterpret_cast<const VT *>(src + off + 3 * step);
+        *reinterpret_cast<VT *>(dst + off) = v0;
+        *reinterpret_cast<VT *>(dst + off + step) = v1;
+        *reinterpret_cast<VT *>(dst + off + 2 * step) = v2;
+        *reinterpret_cast<VT *>(dst + off + 3 * step) = v3;
+      }
+      for (; off < R; off += step)
+        *reinterpret_cast<VT *>(dst + off) = *reinterpret_cast<const VT *>(src + off);
+    }
+  }
+}
+
+template <typename VT, int MODE, bool SET, bool ONE_VEC>
+__global__ __launch_bounds__(kRowsBlock) void rows_kernel(RowArgs a) {
+  // misses are set apart only where they are slow reads: fetch through a map or mask
+  constexpr bool kSeparate = !SET && MODE != kDirect;
+  __shared__ int64_t lds_addr[kSeparate ? kRowsBlock : 1];
+  __shared__ int lds_row[kSeparate ? kRowsBlock : 1];
+  __shared__ int lds_nmiss;
+
+  const int lane = lane_id();
+  const int w = threadIdx.x / kWave;
+  const int tile = 1 << a.log2_tile;
+  const int64_t block_rows = static_cast<int64_t>(kRowsWaves) * tile;
+  const int64_t R = a.row_bytes;
+
+  for (int64_t block_base = blockIdx.x * block_rows; block_base < a.Q;
+       block_base += gridDim.x * block_rows) {
+    if (kSeparate) {
+      if (threadIdx.x == 0) lds_nmiss = 0;
+      __syncthreads();
+    }
+    // ---- phase 1: where does each row of this wave's tile live? ----
+    const int64_t base = block_base + static_cast<int64_t>(w) * tile;
+    const int64_t i = base + lane;
+    const bool live = lane < tile && i < a.Q;
+    const int64_t idx = live ? load_int(a.indices, i, a.idx_bytes) : 0;
     int64_t slot = -1;
     if (MODE == kMask) {
-      slot = load_int(a.mask, row, a.mask_bytes);
-    } else if (MODE == kMap16 || MODE == kMap8) {
-      int64_t v = -1;
-      if (gl < kProbeGroup)
-        v = group_find<MODE == kMap16 ? kSlot16 : kSlot8>(a.map, map_key(a.map, idx));
-      slot = shfl64(v, lane & ~(L - 1));
+      if (live) slot = load_int(a.mask, i, a.mask_bytes);
+    } else if (MODE == kMap16) {
+      slot = wave_find<kSlot16>(a.map, live ? map_key(a.map, idx) : -1);
+    } else if (MODE == kMap8) {
+      slot = wave_find<kSlot8>(a.map, live ? map_key(a.map, idx) : -1);
     }
-    char *table_row = slot >= 0 ? a.cache + slot * R : a.miss + idx * R;
-    char *dense_row = a.dense + row * R;
+    int64_t my_table_row =
+        reinterpret_cast<int64_t>(slot >= 0 ? a.cache + slot * R : a.miss + idx * R);
+    const int64_t left = a.Q - base;
+    const int nrows = static_cast<int>(left < 0 ? 0 : (left < tile ? left : tile));
 
-    int64_t off = static_cast<int64_t>(gl) * sizeof(VT);
-    // four independent vector moves per lane per trip keep loads in flight
-    for (; off + 3 * step < R; off += 4 * step) {
-      VT v0, v1, v2, v3;
-      const char *src = SET ? dense_row : table_row;
-      char *dst = SET ? table_row : dense_row;
-      v0 = *reinterpret_cast<const VT *>(src + off);
-      v1 = *reinterpret_cast<const VT *>(src + off + step);
-      v2 = *reinterpret_cast<const VT *>(src + off + 2 * step);
-      v3 = *reinterpret_cast<const VT *>(src + off + 3 * step);
-      *reinterpret_cast<VT *>(dst + off) = v0;
-      *reinterpret_cast<VT *>(dst + off + step) = v1;
-      *reinterpret_cast<VT *>(dst + off + 2 * step) = v2;
-      *reinterpret_cast<VT *>(dst + off + 3 * step) = v3;
+    if (kSeparate) {
+      // compact this wave's misses into the workgroup list
+      const bool is_miss = live && slot < 0;
+      const uint64_t mm = __builtin_amdgcn_ballot_w64(is_miss);
+      if (mm) {
+        int off = 0;
+        if (lane == 0) off = atomicAdd(&lds_nmiss, __builtin_popcountll(mm));
+        off = __shfl(off, 0, kWave);
+        if (is_miss) {
+          const int pos = off + __builtin_popcountll(mm & ((1ull << lane) - 1ull));
+          lds_addr[pos] = my_table_row;
+          lds_row[pos] = w * tile + lane;
+          my_table_row = 0;  // skipped by this wave's own pass
+        }
+      }
+      __syncthreads();
+      const int nmiss = lds_nmiss;
+      const int miss_waves = (nmiss + kMissPerWave - 1) / kMissPerWave < kRowsWaves
+                                 ? (nmiss + kMissPerWave - 1) / kMissPerWave
+                                 : kRowsWaves;
+      if (w < miss_waves) {
+        const int chunk = (nmiss + miss_waves - 1) / miss_waves;
+        const int begin = w * chunk;
+        const int count = nmiss - begin < chunk ? nmiss - begin : chunk;
+        if (count > 0)
+          move_rows_list<VT, SET, ONE_VEC, true>(a, count, 0, block_base, lds_addr, lds_row, begin);
+      }
     }
-    for (; off < R; off += step) move_vec<VT, SET>(table_row, dense_row, off);
+    // ---- phase 2: this wave's own rows (hits only when misses were set apart) ----
+    move_rows_list<VT, SET, ONE_VEC, false>(a, nrows, my_table_row, base, nullptr, nullptr, 0);
+    if (kSeparate) __syncthreads();  // the list is reused by the next block tile
   }
 }
 
@@ -92,22 +226,30 @@ static int pick_vector_bytes(int64_t row_bytes, const void *p0, const void *p1, 
   return v;
 }
 
-template <typename VT, bool SET>
+template <typename VT, bool SET, bool ONE_VEC>
 static void launch_mode(int mode, unsigned grid, hipStream_t s, const RowArgs &a) {
   switch (mode) {
     case kDirect:
-      hipLaunchKernelGGL((rows_kernel<VT, kDirect, SET>), dim3(grid), dim3(256), 0, s, a);
+      hipLaunchKernelGGL((rows_kernel<VT, kDirect, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
     case kMap16:
-      hipLaunchKernelGGL((rows_kernel<VT, kMap16, SET>), dim3(grid), dim3(256), 0, s, a);
+      hipLaunchKernelGGL((rows_kernel<VT, kMap16, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
     case kMap8:
-      hipLaunchKernelGGL((rows_kernel<VT, kMap8, SET>), dim3(grid), dim3(256), 0, s, a);
+      hipLaunchKernelGGL((rows_kernel<VT, kMap8, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
     default:
-      hipLaunchKernelGGL((rows_kernel<VT, kMask, SET>), dim3(grid), dim3(256), 0, s, a);
+      hipLaunchKernelGGL((rows_kernel<VT, kMask, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
   }
+}
+
+template <typename VT, bool SET>
+static void launch_vec(bool one_vec, int mode, unsigned grid, hipStream_t s, const RowArgs &a) {
+  if (one_vec)
+    launch_mode<VT, SET, true>(mode, grid, s, a);
+  else
+    launch_mode<VT, SET, false>(mode, grid, s, a);
 }
 
 template <bool SET>
@@ -148,15 +290,20 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   int log2_lanes = 3;
   while (log2_lanes < 6 && (1ll << log2_lanes) < nvec) ++log2_lanes;
   a.log2_lanes = log2_lanes;
-  const int rows_per_block = 4 * (kWave >> log2_lanes);
-  const unsigned grid = grid_for(Q, rows_per_block);
+  // Tile of 64 rows per wave when there are rows enough to occupy the chip
+  // (256 CUs x 8 waves); fewer rows per wave otherwise, down to one phase-2 step.
+  int log2_tile = 6;
+  while (log2_tile > 6 - log2_lanes && (Q >> log2_tile) < 2048) --log2_tile;
+  a.log2_tile = log2_tile;
+  const unsigned grid = grid_for(Q, static_cast<int64_t>(kRowsWaves) << log2_tile);
   hipStream_t s = as_stream(stream);
+  const bool one_vec = nvec <= (1ll << log2_lanes);
   switch (vb) {
-    case 16: launch_mode<uint4, SET>(mode, grid, s, a); break;
-    case 8: launch_mode<uint2, SET>(mode, grid, s, a); break;
-    case 4: launch_mode<uint32_t, SET>(mode, grid, s, a); break;
-    case 2: launch_mode<uint16_t, SET>(mode, grid, s, a); break;
-    default: launch_mode<uint8_t, SET>(mode, grid, s, a); break;
+    case 16: launch_vec<u32x4, SET>(one_vec, mode, grid, s, a); break;
+    case 8: launch_vec<u32x2, SET>(one_vec, mode, grid, s, a); break;
+    case 4: launch_vec<uint32_t, SET>(one_vec, mode, grid, s, a); break;
+    case 2: launch_vec<uint16_t, SET>(one_vec, mode, grid, s, a); break;
+    default: launch_vec<uint8_t, SET>(one_vec, mode, grid, s, a); break;
   }
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;

@@ -90,4 +90,43 @@ __device__ __forceinline__ int64_t group_find(const MapView &m, int64_t key) {
   return -1;
 }
 
+// Whole-wave find: every lane brings its own (already normalised) key; the
+// wave's eight probe groups resolve the 64 keys, eight keys per group. Probing
+// proceeds in rounds: in round r every still-unresolved key of a group has its
+// (home + r)-th bucket loaded, all loads of the round are issued before any is
+// examined, so the number of dependent HBM round trips is the longest probe
+// chain among the 64 keys, not the sum. Every lane gets the value for its own
+// key (or -1). All 64 lanes must be active; lanes with nothing to look up
+// pass -1 (the empty sentinel, which resolves to -1 in one round).
+template <int FMT>
+__device__ __forceinline__ int64_t wave_find(const MapView &m, int64_t mykey) {
+  const int sub = lane_id() & (kProbeGroup - 1);
+  const int gbase = lane_id() & ~(kProbeGroup - 1);
+  int64_t res = -1;
+  uint32_t pending = (1u << kProbeGroup) - 1;  // bit j: key j of this group unresolved
+  for (uint32_t round = 0; round < m.nbuckets; ++round) {
+    uint4 frag[kProbeGroup];
+#pragma unroll
+    for (int j = 0; j < kProbeGroup; ++j) {
+      if (pending & (1u << j)) {
+        uint32_t b = map_bucket(m, shfl64(mykey, gbase + j)) + round;
+        if (b >= m.nbuckets) b -= m.nbuckets;
+        frag[j] = m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kProbeGroup; ++j) {
+      if (pending & (1u << j)) {
+        int64_t val;
+        if (probe_step<FMT>(frag[j], shfl64(mykey, gbase + j), &val)) {
+          pending &= ~(1u << j);
+          if (sub == j) res = val;
+        }
+      }
+    }
+    if (pending == 0) break;
+  }
+  return res;
+}
+
 }  // namespace shmt

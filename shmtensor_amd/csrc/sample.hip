@@ -50,23 +50,6 @@ struct PlanArgs {
   int replace;
 };
 
-// Slot of this lane's seed in the cache map (or -1): the wave's 64 seeds are
-// resolved by its 8 probe groups in 8 steps, result returned to the owner lane.
-template <int FMT>
-__device__ __forceinline__ int64_t wave_lookup(const MapView &m, int64_t node) {
-  const int lane = lane_id();
-  const int sub = lane & (kProbeGroup - 1);
-  const int gbase = lane & ~(kProbeGroup - 1);
-  const int64_t mykey = map_key(m, node);
-  int64_t res = -1;
-#pragma unroll 2
-  for (int j = 0; j < kProbeGroup; ++j) {
-    int64_t v = group_find<FMT>(m, shfl64(mykey, gbase + j));
-    if (sub == j) res = v;
-  }
-  return res;
-}
-
 // MODE 0: no cache; 1: wide map; 2: narrow map.
 template <int MODE>
 __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
@@ -74,8 +57,8 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
   const bool live = i < a.S;
   int64_t node = live ? load_int(a.seeds, i, a.seed_bytes) : -1;
   int64_t slot = -1;
-  if (MODE == 1) slot = wave_lookup<kSlot16>(a.map, node);
-  if (MODE == 2) slot = wave_lookup<kSlot8>(a.map, node);
+  if (MODE == 1) slot = wave_find<kSlot16>(a.map, map_key(a.map, node));
+  if (MODE == 2) slot = wave_find<kSlot8>(a.map, map_key(a.map, node));
   int64_t cnt = 0;
   if (live) {
     int64_t begin, end;

@@ -30,7 +30,8 @@ def test_size_queries_and_validation(cabi):
     # 8 wide slots or 16 narrow slots per 128-byte bucket
     assert lib.shmt_hashmap_table_bytes(4194304, 0.5, 8, 8) == 8388608 * 16
     assert lib.shmt_hashmap_table_bytes(1000, 0.5, 4, 4) == 2000 * 8
-    assert lib.shmt_hashmap_table_bytes(8, 1.0, 8, 8) == 2 * 128      # one spare slot forces a 2nd bucket
+    assert lib.shmt_hashmap_table_bytes(8, 1.0, 8, 8) == 2 * 128      # never denser than 50 %: 16 slots
+    assert lib.shmt_hashmap_table_bytes(0, 0.5, 8, 8) == 128          # an empty map keeps one empty bucket
     assert lib.shmt_hashmap_table_bytes(10, 0.5, 3, 8) == -1
     assert b"bad arguments" in lib.shmt_last_error()
     assert lib.shmt_scan_tmp_bytes(1000) == 0 and lib.shmt_scan_tmp_bytes(1 << 20) == 512 * 8
