@@ -98,33 +98,39 @@ __device__ __forceinline__ int64_t group_find(const MapView &m, int64_t key) {
 // chain among the 64 keys, not the sum. Every lane gets the value for its own
 // key (or -1). All 64 lanes must be active; lanes with nothing to look up
 // pass -1 (the empty sentinel, which resolves to -1 in one round).
-template <int FMT>
+template <int FMT, int BATCH = kProbeGroup>
 __device__ __forceinline__ int64_t wave_find(const MapView &m, int64_t mykey) {
+  static_assert(kProbeGroup % BATCH == 0, "BATCH must divide the probe group size");
   const int sub = lane_id() & (kProbeGroup - 1);
   const int gbase = lane_id() & ~(kProbeGroup - 1);
   int64_t res = -1;
-  uint32_t pending = (1u << kProbeGroup) - 1;  // bit j: key j of this group unresolved
-  for (uint32_t round = 0; round < m.nbuckets; ++round) {
-    uint4 frag[kProbeGroup];
+  // BATCH keys of each group are in flight at a time (fewer live registers
+  // for smaller BATCH, at the price of kProbeGroup / BATCH sequential passes)
 #pragma unroll
-    for (int j = 0; j < kProbeGroup; ++j) {
-      if (pending & (1u << j)) {
-        uint32_t b = map_bucket(m, shfl64(mykey, gbase + j)) + round;
-        if (b >= m.nbuckets) b -= m.nbuckets;
-        frag[j] = m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
-      }
-    }
+  for (int j0 = 0; j0 < kProbeGroup; j0 += BATCH) {
+    uint32_t pending = (1u << BATCH) - 1;  // bit j: key j0 + j of this group unresolved
+    for (uint32_t round = 0; round < m.nbuckets; ++round) {
+      uint4 frag[BATCH];
 #pragma unroll
-    for (int j = 0; j < kProbeGroup; ++j) {
-      if (pending & (1u << j)) {
-        int64_t val;
-        if (probe_step<FMT>(frag[j], shfl64(mykey, gbase + j), &val)) {
-          pending &= ~(1u << j);
-          if (sub == j) res = val;
+      for (int j = 0; j < BATCH; ++j) {
+        if (pending & (1u << j)) {
+          uint32_t b = map_bucket(m, shfl64(mykey, gbase + j0 + j)) + round;
+          if (b >= m.nbuckets) b -= m.nbuckets;
+          frag[j] = m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
         }
       }
+#pragma unroll
+      for (int j = 0; j < BATCH; ++j) {
+        if (pending & (1u << j)) {
+          int64_t val;
+          if (probe_step<FMT>(frag[j], shfl64(mykey, gbase + j0 + j), &val)) {
+            pending &= ~(1u << j);
+            if (sub == j0 + j) res = val;
+          }
+        }
+      }
+      if (pending == 0) break;
     }
-    if (pending == 0) break;
   }
   return res;
 }
