@@ -26,6 +26,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the config-4 fetch kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/rows_kernel_fetch_config4_pmc.md): 71,373.5 KiB x 2.0 (copy-calibrated) read + 262,144.1 KiB written.
+CONFIG4_TRAFFIC_BYTES = 414_608_592
 
 
 def log(*a):
@@ -118,7 +121,8 @@ def bench_fetch(capi, args, result):
     result.update({
         "value": round(value, 2), "ms_per_step": round(ms_per_step, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": CONFIG4_TRAFFIC_BYTES if N == 100_000_000 else None,
                      "kernel": "rows_kernel<u32x4, map16, fetch>", "kernel_ms": round(kern_ms, 4),
                      "bytes_per_launch": algo_bytes},
     })
@@ -126,6 +130,9 @@ def bench_fetch(capi, args, result):
                              "Q=%d Zipf(1.1)" % (N, D, C, Q), "hit_rate": round(hit_rate, 4),
                              "row_bytes": R, "queries_per_step": Q})
     extra = result["extra"]
+    if args.headline_only:
+        del host, cache, hmap
+        return
 
     # pinned host -> device copy ceiling (DMA engine), the miss-path roofline
     nbytes = min(1 << 30, host.numel() * 2)
@@ -304,6 +311,22 @@ def bench_sampling(capi, args, result):
     result["extra"]["sampling_config3"] = res
 
 
+def probe_granularity(capi, args, result):
+    """Random rows of 16/32/64/128 bytes from a 4 GiB HBM table: run under
+    rocprofv3 --pmc FETCH_SIZE to see how many bytes one small random read costs."""
+    import torch
+    q_n = 1 << 22
+    res = {}
+    for rb in (16, 32, 64, 128):
+        n = (1 << 32) // rb
+        tab = torch.empty((n, rb), device="cuda", dtype=torch.uint8)
+        q = torch.randint(0, n, (q_n,), device="cuda")
+        t = gpu_time_ms(lambda: capi.uva_fetch(tab, q), 3, warmup=1)
+        res["row_bytes_%d" % rb] = {"rows": q_n, "ms": round(t["median"], 4)}
+        del tab
+    result["extra"]["granularity_probe"] = res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -315,6 +338,9 @@ def main():
     ap.add_argument("--sampling-batches", type=int, default=50)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="fetch workload: only the timed config-4 steps (used for profiler runs, so that "
+                         "every launch of the fetch kernel in the trace belongs to the headline workload)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
@@ -341,6 +367,8 @@ def main():
     if "hashmap" in todo:
         bench_hashmap(capi, args, result)
         torch.cuda.empty_cache()
+    if "granularity" in todo:
+        probe_granularity(capi, args, result)
     if "sampling" in todo:
         bench_sampling(capi, args, result)
         s = result["extra"]["sampling_config3"]
