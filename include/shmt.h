@@ -146,6 +146,18 @@ int64_t shmt_relabel_scratch_bytes(int64_t N);
 int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  int64_t scratch_bytes, void *unique_out, void *labels_out,
                  int64_t *count_out, void *stream);
+/* Same, with the concatenation of the caller's tensors (torch::cat,
+ * src/tensor_relabel.cu:131) done on the way in: nseg <= SHMT_RELABEL_MAX_SEGMENTS
+ * segments seg_ptrs[s] of seg_lens[s] ids, seg_bytes[s] in {4,8} wide, are
+ * widened to elem_bytes (the width torch::cat would promote to) and written
+ * to total_out (N = sum of seg_lens elements), which then plays the role of
+ * `total` above. The three arrays are host arrays read during the call.     */
+#define SHMT_RELABEL_MAX_SEGMENTS 8
+int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens,
+                          const int *seg_bytes, int nseg, int elem_bytes,
+                          void *total_out, void *scratch, int64_t scratch_bytes,
+                          void *unique_out, void *labels_out, int64_t *count_out,
+                          void *stream);
 
 /* ------------------------------------------------------------------ */
 /* Neighbour sampling: CSRWiseSampling src/cache_graph_sampling.cu:179-220

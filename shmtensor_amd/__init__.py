@@ -28,11 +28,22 @@ def _load_module():
     return _MODULE
 
 
+_ALIASING = False
+
+
 def install_aliases():
-    """Register the operator module under the name the reference scripts use
-    (`import ShmTensorLib as capi`). Returns the module."""
+    """Register the operator module and the Python package under the names the
+    reference scripts use (`import ShmTensorLib as capi`, `from shmtensor import
+    GPUSamplingDataloader`). Returns the operator module."""
+    global _ALIASING
     mod = _load_module()
     sys.modules.setdefault("ShmTensorLib", mod)
+    if not _ALIASING and "shmtensor" not in sys.modules:
+        _ALIASING = True
+        try:
+            sys.modules.setdefault("shmtensor", importlib.import_module("shmtensor_amd.shmtensor"))
+        finally:
+            _ALIASING = False
     return mod
 
 

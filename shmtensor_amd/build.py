@@ -71,7 +71,8 @@ def build_module():
         cmd += ["-isystem", inc]
     cmd += ["-isystem", "/opt/rocm/include", "-I" + sysconfig.get_paths()["include"],
             "-I" + INCLUDE]
-    cmd += [os.path.join(CSRC, "pybind", "module.cc"), "-o", module_path(),
+    cmd += [os.path.join(CSRC, "pybind", "module.cc"), os.path.join(CSRC, "pybind", "host_tensors.cc"),
+            "-o", module_path(),
             "-L" + tlib, "-L" + LIB_DIR, "-lshmt", "-ltorch", "-ltorch_cpu", "-ltorch_python",
             "-lc10", "-lc10_hip", "-ltorch_hip",
             "-Wl,-rpath,$ORIGIN/lib", "-Wl,-rpath," + tlib]

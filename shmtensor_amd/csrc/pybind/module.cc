@@ -399,25 +399,50 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
     TORCH_CHECK(t.is_cuda(), "tensor_relabel expects CUDA tensors");
     split_sizes.push_back(t.numel());
   }
-  torch::Tensor total = torch::cat(tensors, 0).contiguous();
-  const int eb = id_bytes(total, "tensors");
-  const int64_t N = total.numel();
-  torch::Tensor unique = torch::empty({N}, total.options());
-  torch::Tensor labels = torch::empty({N}, total.options());
+  // dtype of torch::cat(tensors): int64 as soon as one input is int64
+  int eb = 4;
+  for (auto &t : tensors) eb = std::max(eb, id_bytes(t, "tensors"));
+  const auto options = tensors[0].options().dtype(eb == 8 ? torch::kInt64 : torch::kInt32);
+  int64_t N = 0;
+  for (int64_t n : split_sizes) N += n;
+  torch::Tensor unique = torch::empty({N}, options);
+  torch::Tensor labels = torch::empty({N}, options);
   if (N == 0) return std::make_tuple(unique, labels.split_with_sizes(split_sizes, 0));
   const int64_t scratch_bytes = shmt_relabel_scratch_bytes(N);
   torch::Tensor scratch = device_bytes(scratch_bytes);
   Readback &rb = readback();
-  check(shmt_relabel(total.data_ptr(), N, eb, scratch.data_ptr(), scratch_bytes, unique.data_ptr(),
-                     labels.data_ptr(), rb.get(), current_stream()));
+  if (tensors.size() <= SHMT_RELABEL_MAX_SEGMENTS) {
+    // concatenation fused into the first relabel pass
+    std::vector<torch::Tensor> keep;
+    const void *ptrs[SHMT_RELABEL_MAX_SEGMENTS];
+    int64_t lens[SHMT_RELABEL_MAX_SEGMENTS];
+    int widths[SHMT_RELABEL_MAX_SEGMENTS];
+    for (size_t i = 0; i < tensors.size(); ++i) {
+      keep.push_back(tensors[i].contiguous());
+      ptrs[i] = keep[i].data_ptr();
+      lens[i] = keep[i].numel();
+      widths[i] = static_cast<int>(keep[i].element_size());
+    }
+    torch::Tensor total = torch::empty({N}, options);
+    check(shmt_relabel_segments(ptrs, lens, widths, static_cast<int>(tensors.size()), eb,
+                                total.data_ptr(), scratch.data_ptr(), scratch_bytes,
+                                unique.data_ptr(), labels.data_ptr(), rb.get(), current_stream()));
+  } else {
+    torch::Tensor total = torch::cat(tensors, 0).contiguous();
+    check(shmt_relabel(total.data_ptr(), N, eb, scratch.data_ptr(), scratch_bytes, unique.data_ptr(),
+                       labels.data_ptr(), rb.get(), current_stream()));
+  }
   const int64_t U = rb.value();
   return std::make_tuple(unique.narrow(0, 0, U), labels.split_with_sizes(split_sizes, 0));
 }
 
 }  // namespace
 
+void register_host_tensors(py::module &m);  // host_tensors.cc
+
 PYBIND11_MODULE(ShmTensorLib, m) {
   m.doc() = "MI355X-native ShmTensor GPU-cache operators (HIP, gfx950)";
+  register_host_tensors(m);
 
   m.def("thrust_scan", &thrust_scan, py::arg("tensor"));
 

@@ -4,10 +4,11 @@
 //
 // Passes over the N inputs (each a separate launch, no host round trip):
 //   fill     table slots {key = -1, first = 0xFFFFFFFF}
-//   insert   claim a slot per distinct key (64-bit CAS), atomicMin the index
+//   insert   per-workgroup de-duplication in LDS, then one global insert per
+//            distinct id of the tile (64-bit CAS on the key, atomicMin the index)
 //   first    first[i] = smallest index holding the same key (kept in the
 //            labels buffer); per-tile count of i with first[i] == i
-//   partials exclusive scan of the per-tile counts
+//   partials exclusive scan of the per-tile counts (own launch only beyond 4 M ids)
 //   unique   rank of every first occurrence; unique[rank] = key; rank_of[i]
 //   labels   labels[i] = rank_of[first[i]]
 // The table is touched only by `insert` and `first`; the last two passes read
@@ -23,6 +24,7 @@ namespace shmt {
 constexpr int kRlBlock = 256;
 constexpr int kRlItems = 8;
 constexpr int kRlTile = kRlBlock * kRlItems;
+constexpr int64_t kRlSelfPrefixTiles = 2048;  // up to 4 M ids the unique pass sums the tile counts itself
 
 struct RlSlot {
   int64_t key;
@@ -53,49 +55,110 @@ static RlLayout rl_layout(int64_t N) {
   return l;
 }
 
-__global__ __launch_bounds__(256) void rl_insert_kernel(RlSlot *tbl, uint32_t cap,
-                                                        const void *total, int eb, int64_t N) {
-  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (; i < N; i += stride) {
-    const int64_t key = load_int(total, i, eb);
-    uint32_t pos = reduce_range(hash_id(key), cap);
-    for (uint32_t probes = 0; probes < cap; ++probes) {
+// Claim a slot for `key` and lower its first index to `i`.
+__device__ __forceinline__ void rl_global_insert(RlSlot *tbl, uint32_t cap, int64_t key, uint32_t i) {
+  uint32_t pos = reduce_range(hash_id(key), cap);
+  for (uint32_t probes = 0; probes < cap; ++probes) {
+    // Look before the atomics: a stale cached view can only look emptier /
+    // larger than the truth, in which case the atomic below settles it.
+    const uint4 s = *reinterpret_cast<const uint4 *>(&tbl[pos]);
+    const int64_t seen = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
+    if (seen == key) {
+      if (s.z > i) atomicMin(&tbl[pos].first, i);
+      return;
+    }
+    if (seen == -1) {
       unsigned long long prev =
           atomicCAS(reinterpret_cast<unsigned long long *>(&tbl[pos].key), ~0ull,
                     static_cast<unsigned long long>(key));
       if (prev == ~0ull || static_cast<int64_t>(prev) == key) {
-        atomicMin(&tbl[pos].first, static_cast<uint32_t>(i));
-        break;
+        atomicMin(&tbl[pos].first, i);
+        return;
       }
-      pos = (pos + 1 == cap) ? 0 : pos + 1;
     }
-  }
-}
-
-__device__ __forceinline__ uint32_t rl_find_first(const RlSlot *tbl, uint32_t cap, int64_t key) {
-  uint32_t pos = reduce_range(hash_id(key), cap);
-  for (uint32_t probes = 0; probes < cap; ++probes) {
-    const uint4 s = *reinterpret_cast<const uint4 *>(&tbl[pos]);
-    const int64_t k = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
-    if (k == key) return s.z;
-    if (k == -1) break;
     pos = (pos + 1 == cap) ? 0 : pos + 1;
   }
-  return 0xFFFFFFFFu;
 }
 
+constexpr int kRlInsertTile = kRlBlock;          // ids per workgroup pass: one per thread
+constexpr int kRlLdsSlots = 2 * kRlInsertTile;   // per-workgroup staging table, load <= 0.5
+
+// Insert pass. Ids of hub nodes repeat thousands of times in a sampled batch,
+// and atomics on one address serialise in L2, so every workgroup first
+// de-duplicates its 256 ids in an LDS table (key -> smallest index among
+// them) and sends one global insert per distinct id; each thread then has at
+// most a couple of dependent global probe chains.
+__global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32_t cap,
+                                                             const void *total, int eb, int64_t N) {
+  __shared__ unsigned long long lkey[kRlLdsSlots];
+  __shared__ uint32_t lfirst[kRlLdsSlots];
+  const int64_t ntiles = (N + kRlInsertTile - 1) / kRlInsertTile;
+  for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    for (int t = threadIdx.x; t < kRlLdsSlots; t += kRlBlock) {
+      lkey[t] = ~0ull;
+      lfirst[t] = 0xFFFFFFFFu;
+    }
+    __syncthreads();
+    const int64_t i = tile * kRlInsertTile + threadIdx.x;
+    if (i < N) {
+      const int64_t key = load_int(total, i, eb);
+      uint32_t pos = hash_id(key) & (kRlLdsSlots - 1);
+      for (int probes = 0; probes < kRlLdsSlots; ++probes) {
+        const unsigned long long prev =
+            atomicCAS(&lkey[pos], ~0ull, static_cast<unsigned long long>(key));
+        if (prev == ~0ull || static_cast<int64_t>(prev) == key) {
+          atomicMin(&lfirst[pos], static_cast<uint32_t>(i));
+          break;
+        }
+        pos = (pos + 1) & (kRlLdsSlots - 1);
+      }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < kRlLdsSlots; t += kRlBlock) {
+      const unsigned long long k = lkey[t];
+      if (k != ~0ull) rl_global_insert(tbl, cap, static_cast<int64_t>(k), lfirst[t]);
+    }
+    __syncthreads();
+  }
+}
+
+// First-occurrence index of every element. The first-slot loads of a
+// thread's eight elements are issued together; only the rare longer probe
+// chains continue one by one.
 __global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
                                                             const void *total, int eb, int64_t N,
                                                             void *labels, uint64_t *partials) {
   __shared__ uint64_t lds[kRlBlock / kWave];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kRlTile;
+  int64_t key[kRlItems];
+  uint32_t pos[kRlItems];
+  uint4 slot[kRlItems];
+#pragma unroll
+  for (int j = 0; j < kRlItems; ++j) {
+    const int64_t i = base + j * kRlBlock + threadIdx.x;
+    key[j] = i < N ? load_int(total, i, eb) : -1;
+    pos[j] = reduce_range(hash_id(key[j]), cap);
+  }
+#pragma unroll
+  for (int j = 0; j < kRlItems; ++j) slot[j] = *reinterpret_cast<const uint4 *>(&tbl[pos[j]]);
   uint64_t cnt = 0;
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
     const int64_t i = base + j * kRlBlock + threadIdx.x;
     if (i < N) {
-      const uint32_t f = rl_find_first(tbl, cap, load_int(total, i, eb));
+      uint4 s = slot[j];
+      uint32_t p = pos[j];
+      uint32_t f = 0xFFFFFFFFu;
+      for (uint32_t probes = 0; probes < cap; ++probes) {
+        const int64_t k = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
+        if (k == key[j]) {
+          f = s.z;
+          break;
+        }
+        if (k == -1) break;
+        p = (p + 1 == cap) ? 0 : p + 1;
+        s = *reinterpret_cast<const uint4 *>(&tbl[p]);
+      }
       store_int(labels, i, eb, static_cast<int64_t>(f));
       cnt += (f == static_cast<uint32_t>(i));
     }
@@ -109,8 +172,21 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
                                                              const void *labels,
                                                              const uint64_t *partials,
                                                              void *unique_out, uint32_t *rank_of,
-                                                             int64_t *count_out) {
+                                                             int64_t *count_out, int scanned) {
   __shared__ uint32_t lds[kRlBlock / kWave];
+  __shared__ uint64_t lds64[kRlBlock / kWave];
+  // Tile prefix: either already scanned by a separate launch, or (few tiles)
+  // summed here from the raw per-tile counts.
+  uint64_t tile_prefix;
+  if (scanned) {
+    tile_prefix = partials[blockIdx.x];
+  } else {
+    uint64_t part = 0;
+    for (int t = threadIdx.x; t < static_cast<int>(blockIdx.x); t += kRlBlock) part += partials[t];
+    uint64_t below;
+    block_exclusive_scan<uint64_t, kRlBlock>(part, lds64, &below);
+    tile_prefix = below;
+  }
   const int64_t first_i = static_cast<int64_t>(blockIdx.x) * kRlTile +
                           static_cast<int64_t>(threadIdx.x) * kRlItems;
   bool win[kRlItems];
@@ -123,7 +199,7 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
   }
   uint32_t tile_total;
   uint32_t ex = block_exclusive_scan<uint32_t, kRlBlock>(mine, lds, &tile_total);
-  uint64_t rank = partials[blockIdx.x] + ex;
+  uint64_t rank = tile_prefix + ex;
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
     const int64_t i = first_i + j;
@@ -134,7 +210,7 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
     }
   }
   if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
-    *count_out = static_cast<int64_t>(partials[blockIdx.x] + tile_total);
+    *count_out = static_cast<int64_t>(tile_prefix + tile_total);
     __threadfence_system();
   }
 }
@@ -146,6 +222,31 @@ __global__ __launch_bounds__(256) void rl_labels_kernel(void *labels, int eb, in
   for (; i < N; i += stride) {
     const int64_t f = load_int(labels, i, eb);
     store_int(labels, i, eb, static_cast<int64_t>(rank_of[f]));
+  }
+}
+
+struct RlSegments {
+  const void *ptr[SHMT_RELABEL_MAX_SEGMENTS];
+  int64_t start[SHMT_RELABEL_MAX_SEGMENTS + 1];  // start[s] = first index of segment s in total
+  int bytes[SHMT_RELABEL_MAX_SEGMENTS];
+  int n;
+};
+
+// First pass when the input arrives as segments: empties the table and writes
+// the concatenated, widened ids in one sweep (both are streaming stores).
+__global__ __launch_bounds__(256) void rl_fill_concat_kernel(uint4 *tbl16, int64_t cap, RlSegments segs,
+                                                             void *total, int eb, int64_t N) {
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t span = cap > N ? cap : N;
+  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
+  for (; i < span; i += stride) {
+    if (i < cap) tbl16[i] = ones;
+    if (i < N) {
+      int sgm = 0;
+      while (sgm + 1 < segs.n && i >= segs.start[sgm + 1]) ++sgm;
+      store_int(total, i, eb, load_int(segs.ptr[sgm], i - segs.start[sgm], segs.bytes[sgm]));
+    }
   }
 }
 
@@ -165,9 +266,9 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
   return rl_layout(N).total;
 }
 
-int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
-                 int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
-                 void *stream) {
+static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, int elem_bytes,
+                        void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
+                        int64_t *count_out, void *stream) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
@@ -194,23 +295,73 @@ int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
   const int64_t nb = (N + kRlTile - 1) / kRlTile;
   const uint32_t cap = static_cast<uint32_t>(l.cap);
 
-  int rc = launch_fill_ones(tbl, l.cap, s);
-  if (rc) return rc;
-  hipLaunchKernelGGL(rl_insert_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, tbl, cap, total,
-                     elem_bytes, N);
+  int rc = SHMT_OK;
+  if (segs) {
+    const int64_t span = l.cap > N ? l.cap : N;
+    hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(span, 256 * 4)), dim3(256), 0, s,
+                       reinterpret_cast<uint4 *>(tbl), l.cap, *segs, const_cast<void *>(total),
+                       elem_bytes, N);
+    SHMT_LAUNCH_CHECK();
+  } else {
+    rc = launch_fill_ones(tbl, l.cap, s);
+    if (rc) return rc;
+  }
+  hipLaunchKernelGGL(rl_insert_kernel, dim3(grid_for(N, kRlInsertTile, 256 * 32)), dim3(kRlBlock), 0,
+                     s, tbl, cap, total, elem_bytes, N);
   SHMT_LAUNCH_CHECK();
   hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, tbl,
                      cap, total, elem_bytes, N, labels_out, partials);
   SHMT_LAUNCH_CHECK();
-  rc = launch_scan_partials(partials, nb, s);
-  if (rc) return rc;
+  const int scanned = nb > kRlSelfPrefixTiles;
+  if (scanned) {
+    rc = launch_scan_partials(partials, nb, s);
+    if (rc) return rc;
+  }
   hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s,
-                     total, elem_bytes, N, labels_out, partials, unique_out, rank_of, count_out);
+                     total, elem_bytes, N, labels_out, partials, unique_out, rank_of, count_out,
+                     scanned);
   SHMT_LAUNCH_CHECK();
   hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, labels_out,
                      elem_bytes, N, rank_of);
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;
+}
+
+int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
+                 int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
+                 void *stream) {
+  return relabel_impl(total, nullptr, N, elem_bytes, scratch, scratch_bytes, unique_out, labels_out,
+                      count_out, stream);
+}
+
+int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, const int *seg_bytes,
+                          int nseg, int elem_bytes, void *total_out, void *scratch,
+                          int64_t scratch_bytes, void *unique_out, void *labels_out,
+                          int64_t *count_out, void *stream) {
+  SHMT_REQUIRE(nseg >= 1 && nseg <= SHMT_RELABEL_MAX_SEGMENTS,
+               "shmt_relabel_segments: between 1 and %d segments", SHMT_RELABEL_MAX_SEGMENTS);
+  SHMT_REQUIRE(seg_ptrs && seg_lens && seg_bytes, "shmt_relabel_segments: null segment arrays");
+  RlSegments segs;
+  segs.n = nseg;
+  int64_t N = 0;
+  for (int i = 0; i < nseg; ++i) {
+    SHMT_REQUIRE(seg_lens[i] >= 0, "shmt_relabel_segments: negative segment length");
+    SHMT_REQUIRE(width_ok(seg_bytes[i]) && seg_bytes[i] <= elem_bytes,
+                 "shmt_relabel_segments: segment width must be 4 or 8 and not wider than the output");
+    SHMT_REQUIRE(seg_lens[i] == 0 || seg_ptrs[i] != nullptr, "shmt_relabel_segments: null segment");
+    segs.ptr[i] = seg_ptrs[i];
+    segs.bytes[i] = seg_bytes[i];
+    segs.start[i] = N;
+    N += seg_lens[i];
+  }
+  for (int i = nseg; i <= SHMT_RELABEL_MAX_SEGMENTS; ++i) segs.start[i] = N;
+  for (int i = nseg; i < SHMT_RELABEL_MAX_SEGMENTS; ++i) {
+    segs.ptr[i] = nullptr;
+    segs.bytes[i] = 8;
+  }
+  SHMT_REQUIRE(N == 0 || total_out != nullptr, "shmt_relabel_segments: total_out is null");
+  return relabel_impl(total_out, &segs, N, elem_bytes, scratch, scratch_bytes, unique_out,
+                      labels_out, count_out, stream);
 }
 
 }  // extern "C"

