@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GPU-cache hot path on one MI355X.
 
-Headline ("step"): one cache_fetch call over one batch of BASELINE config 4 —
+Headline ("step"): one cache_fetch call over one batch of benchmark configuration 4 —
 100,000,000 x 128 fp16 feature table in pinned host memory, the 40,000,000
 lowest ids cached in HBM, 1,048,576 int64 queries drawn from Zipf(1.1) over the
 node rank. value = feature bytes delivered per second (Q * row_bytes / t), with
@@ -10,10 +10,21 @@ queries, cache and map resident in HBM when the timed region starts.
 The same JSON line carries the roofline of the fetch kernel, the CPU baseline
 (oracle gather on the host cores, bounded sample) and, under "extra", the
 all-hit / all-miss fetch rates, the cache_set pass, the hashmap microbenchmark
-(config 2) and cached 3-hop sampling with relabel (config 3) beside its CPU
-baseline.
+(config 2), cached 3-hop sampling with relabel (config 3) beside its CPU
+baseline, and the end-to-end mini-batch of config 5 (per stage and whole batch).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,sampling]
+Benchmark configurations referred to by number in this file:
+  2  static hashmap: 4,194,304 unique int64 keys in [0, 2^40) -> insertion index, load factor 0.5;
+     16,777,216 queries, half members, half non-members
+  3  cached sampling: R-MAT scale 21, edge factor 30 (a,b,c,d = .57,.19,.19,.05), symmetrised; int64
+     indptr / int32 indices in pinned host memory, adjacency of the top 30 % of nodes by degree cached
+     in HBM; batches of 1,024 seeds, fanouts [15,10,5], relabel after every hop
+  4  large skewed fetch: the headline above, plus a cache_set pass over 262,144 cached rows
+  5  end-to-end mini-batch: R-MAT scale 24, edge factor 16, top 20 % adjacency cached; 16,777,216 x 256
+     f32 features in pinned host memory, top-degree 25 % cached; 4,096 seeds, fanouts [25,15,10],
+     relabel, then fetch of all input nodes
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,sampling,e2e]
 """
 import argparse
 import json
@@ -311,6 +322,83 @@ def bench_sampling(capi, args, result):
     result["extra"]["sampling_config3"] = res
 
 
+# ---------------------------------------------------------------------------
+# config 5: end-to-end mini-batch (sample 3 hops + relabel, then fetch the input nodes' features)
+
+def bench_e2e(capi, args, result):
+    import torch
+    from shmtensor_amd.synthetic import rmat_csr
+    t0 = time.time()
+    indptr_d, indices_d = rmat_csr(args.e2e_scale, 16, seed=3)
+    n = indptr_d.numel() - 1
+    indptr, indices = indptr_d.cpu().pin_memory(), indices_d.cpu().pin_memory()
+    deg = indptr_d[1:] - indptr_d[:-1]
+    by_degree = torch.sort(deg, descending=True, stable=True).indices
+    del indptr_d, indices_d, deg
+    hot_adj = by_degree[: n // 5].contiguous()
+    gp, gi = capi.create_subcsr(indptr, indices, hot_adj)
+    adj_map = capi.CUCOStaticHashmap(hot_adj, torch.arange(hot_adj.numel(), device="cuda"), 0.8)
+    D = 256
+    feats = torch.empty((n, D), dtype=torch.float32, pin_memory=True)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    for lo in range(0, n, 2_000_000):
+        hi = min(n, lo + 2_000_000)
+        feats[lo:hi].copy_(torch.randn((hi - lo, D), device="cuda", generator=g))
+    torch.cuda.synchronize()
+    hot_feat = by_degree[: n // 4].contiguous()
+    feat_cache = capi.uva_fetch(feats, hot_feat)
+    feat_map = capi.CUCOStaticHashmap(hot_feat, torch.arange(hot_feat.numel(), device="cuda"), 0.8)
+    log("[e2e] R-MAT scale %d ef 16: %d nodes, %d edges; adjacency cache %d rows / %d edges; features %.1f GB "
+        "pinned, %.1f GB cached: %.1f s" % (args.e2e_scale, n, indices.numel(), hot_adj.numel(), gi.numel(),
+                                            feats.numel() * 4 / 1e9, feat_cache.numel() * 4 / 1e9, time.time() - t0))
+    fanouts, S, nbatch = [25, 15, 10], 4096, args.e2e_batches
+    gs = torch.Generator(device="cuda").manual_seed(55)
+    batches = [torch.randperm(n, device="cuda", generator=gs)[:S].contiguous() for _ in range(nbatch + 1)]
+
+    def one(seeds, b, ev=None):
+        edges = 0
+        if ev: ev[0].record()
+        for hop, k in enumerate(reversed(fanouts)):
+            sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, adj_map, seeds, k, False, seed=7777 + b,
+                                             stream_id=hop)
+            uniq, (_, rel) = capi.tensor_relabel([seeds, si])
+            edges += si.numel()
+            seeds = uniq
+        if ev: ev[1].record()
+        x = capi.cache_fetch(feats, feat_cache, seeds, feat_map)
+        if ev: ev[2].record()
+        return edges, seeds, x
+
+    edges, inp, x = one(batches[nbatch], nbatch)          # warm-up + check
+    assert torch.equal(x.cpu(), torch.index_select(feats, 0, inp.cpu())), "e2e features differ from index_select"
+    hit = float((feat_map.query(inp) >= 0).float().mean())
+    del x
+    tot_edges = tot_nodes = 0
+    t_s = t_f = 0.0
+    torch.cuda.synchronize()
+    w0 = time.perf_counter()
+    for b in range(nbatch):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e, inp, x = one(batches[b], b, ev)
+        ev[2].synchronize()
+        t_s += ev[0].elapsed_time(ev[1])
+        t_f += ev[1].elapsed_time(ev[2])
+        tot_edges += e
+        tot_nodes += inp.numel()
+        del x
+    wall = time.perf_counter() - w0
+    result["extra"]["e2e_config5"] = {
+        "graph": "R-MAT scale %d ef 16 symmetrised: %d nodes, %d edges; top 20 %% adjacency cached; features %d x %d "
+                 "f32 pinned, top-degree 25 %% cached" % (args.e2e_scale, n, indices.numel(), n, D),
+        "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
+        "edges_per_batch": tot_edges // nbatch, "input_nodes_per_batch": tot_nodes // nbatch,
+        "feature_hit_rate": round(hit, 4),
+        "sample_relabel_ms": round(t_s / nbatch, 3), "fetch_ms": round(t_f / nbatch, 3),
+        "batch_ms_wall": round(wall * 1e3 / nbatch, 3), "batches_per_s": round(nbatch / wall, 2),
+        "sampled_edges_per_s": round(tot_edges / (t_s * 1e-3), 1),
+        "fetch_payload_GBs": round(tot_nodes * D * 4 / (t_f * 1e-3) / 1e9, 2)}
+
+
 def probe_granularity(capi, args, result):
     """Random rows of 16/32/64/128 bytes from a 4 GiB HBM table: run under
     rocprofv3 --pmc FETCH_SIZE to see how many bytes one small random read costs."""
@@ -332,10 +420,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workloads", default="fetch,hashmap,sampling")
+    ap.add_argument("--workloads", default="fetch,hashmap,sampling,e2e")
     ap.add_argument("--fetch-rows", type=int, default=100_000_000)
     ap.add_argument("--sampling-scale", type=int, default=21)
     ap.add_argument("--sampling-batches", type=int, default=50)
+    ap.add_argument("--e2e-scale", type=int, default=24)
+    ap.add_argument("--e2e-batches", type=int, default=8)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--headline-only", action="store_true",
@@ -373,6 +463,9 @@ def main():
         bench_sampling(capi, args, result)
         s = result["extra"]["sampling_config3"]
         result["sampled_edges_per_s"] = s["sampled_edges_per_s"]
+    if "e2e" in todo:
+        torch.cuda.empty_cache()
+        bench_e2e(capi, args, result)
     print(json.dumps(result), flush=True)
 
 

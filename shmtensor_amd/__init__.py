@@ -19,6 +19,11 @@ def _load_module():
     global _MODULE
     if _MODULE is None:
         import torch  # noqa: F401  (ShmTensorLib links against libtorch)
+        if "ShmTensorLib" in sys.modules:
+            # already imported top-level (this directory on PYTHONPATH): one
+            # extension module must not be initialised twice
+            _MODULE = sys.modules["ShmTensorLib"]
+            return _MODULE
         try:
             _MODULE = importlib.import_module("shmtensor_amd.ShmTensorLib")
         except ImportError as exc:

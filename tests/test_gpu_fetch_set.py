@@ -126,7 +126,7 @@ def test_set_final_state_matches_oracle(capi, oracle):
 
 
 def test_config1_small_fetch(capi, oracle):
-    """BASELINE config 1: 200,000 x 128 f32 table, 50,000 cached ids, 65,536 uniform queries."""
+    """Small fetch configuration: 200,000 x 128 f32 table, 50,000 cached ids, 65,536 uniform queries."""
     torch.manual_seed(0)
     table = torch.randn(200_000, 128).pin_memory()
     ids = torch.randperm(200_000)[:50_000]

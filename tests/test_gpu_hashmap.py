@@ -84,7 +84,7 @@ def test_errors_are_exceptions(capi):
 
 
 def test_full_size_membership_property(capi):
-    """BASELINE config 2 at full size: 4,194,304 unique keys in [0, 2^40), LF 0.5,
+    """Hashmap microbenchmark configuration at full size: 4,194,304 unique keys in [0, 2^40), LF 0.5,
     16,777,216 queries half members / half non-members. Checked through
     properties that need no CPU map: members return their insertion index,
     non-members return -1, and the sum of results is the closed form."""
