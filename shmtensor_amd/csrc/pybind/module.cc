@@ -7,6 +7,9 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
+#include <atomic>
+#include <chrono>
+#include <cstdint>
 #include <mutex>
 #include <optional>
 #include <unordered_map>
@@ -53,24 +56,59 @@ void *device_address(const torch::Tensor &t, const char *name) {
   return dev;
 }
 
-// One int64 in pinned host memory that kernels write totals into (nnz, number
-// of unique ids); read after synchronising the stream.
-struct Readback {
-  torch::Tensor host;
-  int64_t *dev = nullptr;
-  int64_t *get() {
-    if (!host.defined()) {
-      host = torch::zeros({16}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+// Totals whose value only the GPU knows (nnz of a sample, number of unique
+// ids) come back through int64 slots in pinned host memory. The host marks a
+// slot pending before the launches and the kernel overwrites it with the
+// total (always >= 0) followed by a system-scope fence; the host then watches
+// the slot instead of synchronising the stream, so it learns the total as
+// soon as the kernel that computes it has run, while later kernels of the
+// same operator are still queued or running. If the value does not show up
+// within the spin budget (a failed launch, a hung device) the wait falls back
+// to a stream synchronisation, which surfaces the error.
+class Readback {
+ public:
+  struct Slot {
+    volatile int64_t *host;
+    int64_t *dev;
+  };
+
+  Slot acquire() {
+    if (!host_.defined()) {
+      host_ = torch::zeros({kSlots}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
       void *d = nullptr;
-      check(shmt_host_devptr(host.data_ptr(), &d));
-      dev = static_cast<int64_t *>(d);
+      check(shmt_host_devptr(host_.data_ptr(), &d));
+      dev_ = static_cast<int64_t *>(d);
     }
-    return dev;
+    const int i = next_++ % kSlots;
+    Slot s{host_.data_ptr<int64_t>() + i, dev_ + i};
+    *s.host = kPending;
+    std::atomic_thread_fence(std::memory_order_seq_cst);
+    return s;
   }
-  int64_t value() {
+
+  static int64_t wait(const Slot &s) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint64_t spins = 0;; ++spins) {
+      const int64_t v = *s.host;
+      if (v != kPending) return v;
+      if ((spins & 1023) == 1023 &&
+          std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(kSpinBudgetMs))
+        break;
+      __builtin_ia32_pause();
+    }
     sync_current_stream();
-    return *static_cast<volatile int64_t *>(host.data_ptr<int64_t>());
+    const int64_t v = *s.host;
+    TORCH_CHECK(v != kPending, "the GPU did not report a result size (kernel failed?)");
+    return v;
   }
+
+ private:
+  static constexpr int kSlots = 16;
+  static constexpr int64_t kPending = INT64_MIN;
+  static constexpr int kSpinBudgetMs = 200;
+  torch::Tensor host_;
+  int64_t *dev_ = nullptr;
+  int next_ = 0;
 };
 
 Readback &readback() {
@@ -315,23 +353,23 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor &indptr
   torch::Tensor sub_indptr = torch::empty({S + 1}, indptr.options().device(dev));
   const int64_t plan_bytes = shmt_sample_plan_bytes(S);
   torch::Tensor plan = device_bytes(plan_bytes);
-  Readback &rb = readback();
+  const Readback::Slot total = readback().acquire();
   void *stream = current_stream();
   check(shmt_sample_plan(device_address(indptr, "indptr"), pb,
                          map ? gpu_indptr->data_ptr() : nullptr, map ? map->handle() : nullptr,
                          seeds.data_ptr(), static_cast<int>(seeds.element_size()), S, num_picks,
-                         replace, sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, rb.get(),
+                         replace, sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, total.dev,
                          stream));
   // Output size is data dependent. When the bound S*k is modest, sample into a
-  // buffer of that size and read the total once at the end (one host sync per
-  // call); otherwise read the total first and allocate exactly.
+  // buffer of that size and pick up the total afterwards (both kernels are
+  // queued back to back); otherwise wait for the total first and allocate exactly.
   const bool eager = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
   int64_t nnz = -1;
   torch::Tensor sub_indices;
   if (eager) {
     sub_indices = torch::empty({S * num_picks}, indices.options().device(dev));
   } else {
-    nnz = rb.value();
+    nnz = Readback::wait(total);
     sub_indices = torch::empty({nnz}, indices.options().device(dev));
   }
   check(shmt_sample_pick(device_address(indices, "indices"),
@@ -341,7 +379,7 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor &indptr
                          static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
                          static_cast<uint32_t>(stream_id), stream));
   if (eager) {
-    nnz = rb.value();
+    nnz = Readback::wait(total);
     sub_indices = sub_indices.narrow(0, 0, nnz);
   }
   return std::make_tuple(sub_indptr, sub_indices);
@@ -375,12 +413,12 @@ std::tuple<torch::Tensor, torch::Tensor> create_subcsr(torch::Tensor uva_indptr,
   torch::Tensor gpu_indptr = torch::empty({C + 1}, uva_indptr.options().device(torch::kCUDA));
   const int64_t tmp_bytes = shmt_scan_tmp_bytes(C + 1);
   torch::Tensor tmp = device_bytes(tmp_bytes);
-  Readback &rb = readback();
+  const Readback::Slot total = readback().acquire();
   void *stream = current_stream();
   void *indptr_dev = device_address(uva_indptr, "uva_indptr");
   check(shmt_subcsr_plan(indptr_dev, pb, seeds.data_ptr(), static_cast<int>(seeds.element_size()), C,
-                         gpu_indptr.data_ptr(), tmp.data_ptr(), tmp_bytes, rb.get(), stream));
-  const int64_t nnz = rb.value();
+                         gpu_indptr.data_ptr(), tmp.data_ptr(), tmp_bytes, total.dev, stream));
+  const int64_t nnz = Readback::wait(total);
   torch::Tensor gpu_indices = torch::empty({nnz}, uva_indices.options().device(torch::kCUDA));
   check(shmt_subcsr_copy(indptr_dev, device_address(uva_indices, "uva_indices"), pb, ib,
                          seeds.data_ptr(), static_cast<int>(seeds.element_size()), C,
@@ -410,7 +448,7 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
   if (N == 0) return std::make_tuple(unique, labels.split_with_sizes(split_sizes, 0));
   const int64_t scratch_bytes = shmt_relabel_scratch_bytes(N);
   torch::Tensor scratch = device_bytes(scratch_bytes);
-  Readback &rb = readback();
+  const Readback::Slot count = readback().acquire();
   if (tensors.size() <= SHMT_RELABEL_MAX_SEGMENTS) {
     // concatenation fused into the first relabel pass
     std::vector<torch::Tensor> keep;
@@ -426,13 +464,13 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
     torch::Tensor total = torch::empty({N}, options);
     check(shmt_relabel_segments(ptrs, lens, widths, static_cast<int>(tensors.size()), eb,
                                 total.data_ptr(), scratch.data_ptr(), scratch_bytes,
-                                unique.data_ptr(), labels.data_ptr(), rb.get(), current_stream()));
+                                unique.data_ptr(), labels.data_ptr(), count.dev, current_stream()));
   } else {
     torch::Tensor total = torch::cat(tensors, 0).contiguous();
     check(shmt_relabel(total.data_ptr(), N, eb, scratch.data_ptr(), scratch_bytes, unique.data_ptr(),
-                       labels.data_ptr(), rb.get(), current_stream()));
+                       labels.data_ptr(), count.dev, current_stream()));
   }
-  const int64_t U = rb.value();
+  const int64_t U = Readback::wait(count);
   return std::make_tuple(unique.narrow(0, 0, U), labels.split_with_sizes(split_sizes, 0));
 }
 
