@@ -167,3 +167,22 @@ def test_direct_c_abi_fetch(cabi):
     assert lib.shmt_hashmap_create(ctypes.byref(ctypes.c_void_p()), keys.data_ptr(), vals.data_ptr(), 1000, 8, 8,
                                    0.8, table.data_ptr(), 128, None) == -4          # table too small
     lib.shmt_hashmap_destroy(hnd)
+
+
+def test_sliced_tables_and_grid_stride(capi):
+    """Tables whose base pointers are only element-aligned (views into larger
+    tensors) and a query count large enough that every wave loops over tiles."""
+    torch.manual_seed(5)
+    big = torch.randn(4001, 3).pin_memory()
+    data = big[1:]                                  # 12-byte rows starting 12 bytes into the allocation
+    gpu_big = torch.randn(1001, 3).cuda()
+    ids = torch.randperm(4000)[:1000].cuda()
+    gpu_data = gpu_big[1:]
+    gpu_data.copy_(data[ids.cpu()])
+    h = capi.CUCOStaticHashmap(ids, torch.arange(1000).cuda(), 0.5)
+    q = torch.randint(0, 4000, (3_000_001,)).cuda()
+    out = capi.cache_fetch(data, gpu_data, q, h)
+    assert torch.equal(out.cpu(), data[q.cpu()])
+    upd = torch.randn(1000, 3).cuda()
+    capi.cache_set(data, gpu_data, ids, upd, h)     # all hits: only the cache changes
+    assert torch.equal(gpu_big[1:], upd) and torch.equal(capi.uva_fetch(data, ids).cpu(), data[ids.cpu()])
