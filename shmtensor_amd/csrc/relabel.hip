@@ -130,15 +130,19 @@ __global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, u
                                                             void *labels, uint64_t *partials) {
   __shared__ uint64_t lds[kRlBlock / kWave];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kRlTile;
-  int64_t key[kRlItems];
+  int64_t key[kRlItems], idx[kRlItems];
+  bool ok[kRlItems];
   uint32_t pos[kRlItems];
   uint4 slot[kRlItems];
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
-    const int64_t i = base + j * kRlBlock + threadIdx.x;
-    key[j] = i < N ? load_int(total, i, eb) : -1;
-    pos[j] = reduce_range(hash_id(key[j]), cap);
+    idx[j] = base + j * kRlBlock + threadIdx.x;
+    ok[j] = idx[j] < N;
+    key[j] = -1;
   }
+  load_ints<kRlItems>(total, idx, ok, eb, key);
+#pragma unroll
+  for (int j = 0; j < kRlItems; ++j) pos[j] = reduce_range(hash_id(key[j]), cap);
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) slot[j] = *reinterpret_cast<const uint4 *>(&tbl[pos[j]]);
   uint64_t cnt = 0;
@@ -189,14 +193,23 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
   }
   const int64_t first_i = static_cast<int64_t>(blockIdx.x) * kRlTile +
                           static_cast<int64_t>(threadIdx.x) * kRlItems;
-  bool win[kRlItems];
+  bool win[kRlItems], ok[kRlItems];
+  int64_t idx[kRlItems], lab[kRlItems], val[kRlItems];
   uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
-    const int64_t i = first_i + j;
-    win[j] = (i < N) && (load_int(labels, i, eb) == i);
+    idx[j] = first_i + j;
+    ok[j] = idx[j] < N;
+    lab[j] = -1;
+    val[j] = 0;
+  }
+  load_ints<kRlItems>(labels, idx, ok, eb, lab);
+#pragma unroll
+  for (int j = 0; j < kRlItems; ++j) {
+    win[j] = ok[j] && lab[j] == idx[j];
     mine += win[j];
   }
+  load_ints<kRlItems>(total, idx, win, eb, val);
   uint32_t tile_total;
   uint32_t ex = block_exclusive_scan<uint32_t, kRlBlock>(mine, lds, &tile_total);
   uint64_t rank = tile_prefix + ex;
@@ -204,7 +217,7 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
   for (int j = 0; j < kRlItems; ++j) {
     const int64_t i = first_i + j;
     if (win[j]) {
-      store_int(unique_out, static_cast<int64_t>(rank), eb, load_int(total, i, eb));
+      store_int(unique_out, static_cast<int64_t>(rank), eb, val[j]);
       rank_of[i] = static_cast<uint32_t>(rank);
       ++rank;
     }

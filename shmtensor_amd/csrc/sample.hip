@@ -61,14 +61,10 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
   if (MODE == 2) slot = wave_find<kSlot8>(a.map, map_key(a.map, node));
   int64_t cnt = 0;
   if (live) {
+    // both offsets of the row in flight together (cold rows: two host-link reads)
     int64_t begin, end;
-    if (slot >= 0) {
-      begin = load_int(a.cache_indptr, slot, a.ptr_bytes);
-      end = load_int(a.cache_indptr, slot + 1, a.ptr_bytes);
-    } else {
-      begin = load_int(a.indptr, node, a.ptr_bytes);
-      end = load_int(a.indptr, node + 1, a.ptr_bytes);
-    }
+    load_int_pair(slot >= 0 ? a.cache_indptr : a.indptr, slot >= 0 ? slot : node, a.ptr_bytes,
+                  &begin, &end);
     const int64_t deg = end - begin;
     a.plan[i].begin = begin | (slot >= 0 ? kCachedTag : 0);
     a.plan[i].deg = deg;

@@ -37,6 +37,46 @@ __device__ __forceinline__ int64_t load_int(const void *p, int64_t i, int bytes)
                     : static_cast<int64_t>(static_cast<const int32_t *>(p)[i]);
 }
 
+// Several independent loads under ONE width branch. load_int() ends in a
+// join of its two width paths, which makes the compiler wait for each value
+// before the next load is issued; here all N loads of the chosen width are
+// issued back to back. Entries with ok[n] false are skipped (out[n] untouched).
+template <int N>
+__device__ __forceinline__ void load_ints(const void *p, const int64_t (&idx)[N],
+                                          const bool (&ok)[N], int bytes, int64_t (&out)[N]) {
+  if (bytes == 8) {
+    const int64_t *q = static_cast<const int64_t *>(p);
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      if (ok[n]) out[n] = q[idx[n]];
+  } else {
+    const int32_t *q = static_cast<const int32_t *>(p);
+    int32_t tmp[N];
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      if (ok[n]) tmp[n] = q[idx[n]];
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      if (ok[n]) out[n] = static_cast<int64_t>(tmp[n]);
+  }
+}
+
+// p[i] and p[i + 1] (a CSR row's two offsets) in flight together.
+__device__ __forceinline__ void load_int_pair(const void *p, int64_t i, int bytes, int64_t *a,
+                                              int64_t *b) {
+  if (bytes == 8) {
+    const int64_t *q = static_cast<const int64_t *>(p);
+    const int64_t x = q[i], y = q[i + 1];
+    *a = x;
+    *b = y;
+  } else {
+    const int32_t *q = static_cast<const int32_t *>(p);
+    const int32_t x = q[i], y = q[i + 1];
+    *a = x;
+    *b = y;
+  }
+}
+
 __device__ __forceinline__ void store_int(void *p, int64_t i, int bytes, int64_t v) {
   if (bytes == 8)
     static_cast<int64_t *>(p)[i] = v;

@@ -186,3 +186,31 @@ def test_sliced_tables_and_grid_stride(capi):
     upd = torch.randn(1000, 3).cuda()
     capi.cache_set(data, gpu_data, ids, upd, h)     # all hits: only the cache changes
     assert torch.equal(gpu_big[1:], upd) and torch.equal(capi.uva_fetch(data, ids).cpu(), data[ids.cpu()])
+
+
+def test_large_skewed_fetch_scaled(capi):
+    """The large fetch configuration at 1/25 scale: 4,000,000 x 128 fp16 rows pinned, the
+    1,600,000 lowest ids cached, 1,048,576 Zipf(1.1) queries; then a set pass over 262,144
+    cached rows. fp16 compared as raw 16-bit patterns."""
+    from shmtensor_amd.synthetic import zipf_ranks
+    n, c = 4_000_000, 1_600_000
+    g = torch.Generator(device="cuda").manual_seed(2)
+    table_d = torch.randn((n, 128), device="cuda", generator=g).to(torch.float16)
+    table = torch.empty((n, 128), dtype=torch.float16).pin_memory()
+    table.copy_(table_d)
+    cache = table_d[:c].clone()
+    del table_d
+    keys = torch.arange(c, device="cuda")
+    h = capi.CUCOStaticHashmap(keys, keys, 0.8)
+    q = zipf_ranks(1 << 20, n, 1.1, seed=100)
+    hits = float((q < c).float().mean())
+    assert 0.9 < hits < 1.0 and int(q.max()) >= c          # a high hit rate with a miss tail
+    out = capi.cache_fetch(table, cache, q, h)
+    assert torch.equal(out.cpu().view(torch.int16), torch.index_select(table.view(torch.int16), 0, q.cpu()))
+    rows = torch.randperm(c, device="cuda", generator=g)[:262_144].contiguous()
+    upd = torch.randn((262_144, 128), device="cuda", generator=g).to(torch.float16)
+    before = table.clone()
+    capi.cache_set(table, cache, rows, upd, h)
+    assert torch.equal(capi.cache_fetch(table, cache, rows, h).view(torch.int16), upd.view(torch.int16))
+    torch.cuda.synchronize()
+    assert torch.equal(table.view(torch.int16), before.view(torch.int16))      # hits never touch the host copy
