@@ -89,13 +89,26 @@ def build_oracle():
     return ORACLE_LIB
 
 
+NATIVE_TEST = os.path.join(ROOT, "tests", "native", "cabi_smoke.bin")
+
+
+def build_native_test():
+    """Stand-alone C++ program that drives the C ABI without Python or torch
+    (run by tests/test_gpu_native.py on the GPU box)."""
+    _run([hipcc(), "-O2", "-std=c++17", "-I" + INCLUDE, os.path.join(ROOT, "tests", "native", "cabi_smoke.cc"),
+          "-o", NATIVE_TEST, "-L" + LIB_DIR, "-lshmt", "-Wl,-rpath,$ORIGIN/../../shmtensor_amd/lib"])
+    return NATIVE_TEST
+
+
 def build_all():
     build_lib()
     build_module()
     build_oracle()
+    build_native_test()
 
 
 if __name__ == "__main__":
     what = sys.argv[1:] or ["all"]
     for w in what:
-        {"all": build_all, "lib": build_lib, "module": build_module, "oracle": build_oracle}[w]()
+        {"all": build_all, "lib": build_lib, "module": build_module, "oracle": build_oracle,
+         "native": build_native_test}[w]()

@@ -1,0 +1,214 @@
+// Stand-alone check of the C ABI: no Python, no torch. Links libshmt.so and the
+// HIP runtime only, allocates with hipMalloc / hipHostMalloc, and compares the
+// hashmap, fetch, set, scan, relabel and sampling entry points with plain C++
+// loops on the host. Exit status 0 = every check passed.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include <algorithm>
+#include <numeric>
+#include <unordered_map>
+#include <vector>
+
+#include "shmt.h"
+
+#define HIP_OK(x)                                                                 \
+  do {                                                                            \
+    hipError_t e_ = (x);                                                          \
+    if (e_ != hipSuccess) {                                                       \
+      fprintf(stderr, "%s:%d %s: %s\n", __FILE__, __LINE__, #x, hipGetErrorString(e_)); \
+      return 2;                                                                   \
+    }                                                                             \
+  } while (0)
+#define SHMT_OK_(x)                                                          \
+  do {                                                                       \
+    int rc_ = (x);                                                           \
+    if (rc_ != 0) {                                                          \
+      fprintf(stderr, "%s:%d %s -> %d: %s\n", __FILE__, __LINE__, #x, rc_, shmt_last_error()); \
+      return 3;                                                              \
+    }                                                                        \
+  } while (0)
+#define EXPECT(c)                                                  \
+  do {                                                             \
+    if (!(c)) {                                                    \
+      fprintf(stderr, "%s:%d check failed: %s\n", __FILE__, __LINE__, #c); \
+      return 1;                                                    \
+    }                                                              \
+  } while (0)
+
+template <typename T>
+static T *to_device(const std::vector<T> &v) {
+  T *d = nullptr;
+  if (hipMalloc(&d, std::max<size_t>(v.size(), 1) * sizeof(T)) != hipSuccess) return nullptr;
+  if (!v.empty()) (void)hipMemcpy(d, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice);
+  return d;
+}
+template <typename T>
+static std::vector<T> to_host(const T *d, size_t n) {
+  std::vector<T> v(n);
+  if (n) (void)hipMemcpy(v.data(), d, n * sizeof(T), hipMemcpyDeviceToHost);
+  return v;
+}
+
+static uint64_t rng_state = 88172645463325252ull;
+static uint64_t rnd() {
+  rng_state ^= rng_state << 13;
+  rng_state ^= rng_state >> 7;
+  rng_state ^= rng_state << 17;
+  return rng_state;
+}
+
+int main() {
+  EXPECT(shmt_abi_version() == SHMT_ABI_VERSION);
+  hipStream_t stream;
+  HIP_OK(hipStreamCreate(&stream));
+
+  // ---- hashmap: 100,000 distinct int64 keys -> int32 values ----
+  const int64_t n = 100000, nq = 300001;
+  std::vector<int64_t> keys(n);
+  std::vector<int32_t> vals(n);
+  std::unordered_map<int64_t, int32_t> truth;
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t k;
+    do k = static_cast<int64_t>(rnd() % (1ull << 40)); while (truth.count(k));
+    keys[i] = k;
+    vals[i] = static_cast<int32_t>(i);
+    truth[k] = vals[i];
+  }
+  int64_t *d_keys = to_device(keys);
+  int32_t *d_vals = to_device(vals);
+  const int64_t table_bytes = shmt_hashmap_table_bytes(n, 0.8, 8, 4);
+  EXPECT(table_bytes > 0 && shmt_hashmap_capacity(n, 0.8) == 125000);
+  void *d_table = nullptr;
+  HIP_OK(hipMalloc(&d_table, table_bytes));
+  shmt_hashmap_t *map = nullptr;
+  SHMT_OK_(shmt_hashmap_create(&map, d_keys, d_vals, n, 8, 4, 0.8, d_table, table_bytes, stream));
+  std::vector<int64_t> req(nq);
+  for (int64_t i = 0; i < nq; ++i) req[i] = (i % 2) ? keys[rnd() % n] : static_cast<int64_t>(rnd() % (1ull << 40));
+  int64_t *d_req = to_device(req);
+  int32_t *d_res = nullptr;
+  HIP_OK(hipMalloc(&d_res, nq * sizeof(int32_t)));
+  SHMT_OK_(shmt_hashmap_query(map, d_req, 8, nq, d_res, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  std::vector<int32_t> res = to_host(d_res, nq);
+  for (int64_t i = 0; i < nq; ++i) {
+    auto it = truth.find(req[i]);
+    EXPECT(res[i] == (it == truth.end() ? -1 : it->second));
+  }
+
+  // ---- fetch / set: 20,000 x 96-byte rows in pinned host memory, 5,000 cached ----
+  const int64_t rows = 20000, row_bytes = 96, cached = 5000, Q = 70001;
+  char *h_table = nullptr;
+  HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&h_table), rows * row_bytes, hipHostMallocDefault));
+  for (int64_t i = 0; i < rows * row_bytes; ++i) h_table[i] = static_cast<char>(rnd());
+  void *table_alias = nullptr;
+  SHMT_OK_(shmt_host_devptr(h_table, &table_alias));
+  std::vector<int64_t> cache_ids(rows);
+  std::iota(cache_ids.begin(), cache_ids.end(), 0);
+  for (int64_t i = rows - 1; i > 0; --i) std::swap(cache_ids[i], cache_ids[rnd() % (i + 1)]);
+  cache_ids.resize(cached);
+  std::vector<int64_t> slots(cached);
+  std::iota(slots.begin(), slots.end(), 0);
+  std::vector<char> cache_rows(cached * row_bytes);
+  for (int64_t s = 0; s < cached; ++s)
+    for (int64_t b = 0; b < row_bytes; ++b)
+      cache_rows[s * row_bytes + b] = static_cast<char>(h_table[cache_ids[s] * row_bytes + b] ^ 0x5a);  // differs from host
+  char *d_cache = to_device(cache_rows);
+  int64_t *d_cids = to_device(cache_ids), *d_slots = to_device(slots);
+  const int64_t fbytes = shmt_hashmap_table_bytes(cached, 0.5, 8, 8);
+  void *d_ftable = nullptr;
+  HIP_OK(hipMalloc(&d_ftable, fbytes));
+  shmt_hashmap_t *fmap = nullptr;
+  SHMT_OK_(shmt_hashmap_create(&fmap, d_cids, d_slots, cached, 8, 8, 0.5, d_ftable, fbytes, stream));
+  std::vector<int32_t> q(Q);
+  for (auto &x : q) x = static_cast<int32_t>(rnd() % rows);
+  int32_t *d_q = to_device(q);
+  char *d_out = nullptr;
+  HIP_OK(hipMalloc(&d_out, Q * row_bytes));
+  SHMT_OK_(shmt_fetch(table_alias, d_cache, d_q, 4, fmap, nullptr, 0, d_out, Q, row_bytes, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  std::vector<char> out = to_host(d_out, Q * row_bytes);
+  std::unordered_map<int64_t, int64_t> slot_of;
+  for (int64_t s = 0; s < cached; ++s) slot_of[cache_ids[s]] = s;
+  for (int64_t i = 0; i < Q; ++i) {
+    auto it = slot_of.find(q[i]);
+    const char *expect = it == slot_of.end() ? h_table + q[i] * row_bytes : cache_rows.data() + it->second * row_bytes;
+    EXPECT(std::equal(expect, expect + row_bytes, out.begin() + i * row_bytes));
+  }
+  // pageable host memory is refused instead of faulting
+  std::vector<char> pageable(4096);
+  void *alias = nullptr;
+  EXPECT(shmt_host_devptr(pageable.data(), &alias) == SHMT_ENOTPINNED);
+
+  // ---- exclusive scan, int32, 1,000,001 elements ----
+  const int64_t len = 1000001;
+  std::vector<int32_t> a(len);
+  for (auto &x : a) x = static_cast<int32_t>(rnd() % 1000);
+  int32_t *d_a = to_device(a);
+  const int64_t tmp_bytes = shmt_scan_tmp_bytes(len);
+  void *d_tmp = nullptr;
+  HIP_OK(hipMalloc(&d_tmp, std::max<int64_t>(tmp_bytes, 1)));
+  SHMT_OK_(shmt_exclusive_scan(d_a, len, 4, d_tmp, tmp_bytes, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  std::vector<int32_t> scanned = to_host(d_a, len);
+  uint32_t run = 0;
+  for (int64_t i = 0; i < len; ++i) {
+    EXPECT(static_cast<uint32_t>(scanned[i]) == run);
+    run += static_cast<uint32_t>(a[i]);
+  }
+
+  // ---- relabel: 200,000 int64 ids, first-occurrence order ----
+  const int64_t N = 200000;
+  std::vector<int64_t> ids(N);
+  for (auto &x : ids) x = static_cast<int64_t>(rnd() % 50000);
+  int64_t *d_ids = to_device(ids), *d_unique = nullptr, *d_labels = nullptr, *h_count = nullptr;
+  HIP_OK(hipMalloc(&d_unique, N * 8));
+  HIP_OK(hipMalloc(&d_labels, N * 8));
+  HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&h_count), 8, hipHostMallocDefault));
+  const int64_t sbytes = shmt_relabel_scratch_bytes(N);
+  void *d_scratch = nullptr;
+  HIP_OK(hipMalloc(&d_scratch, sbytes));
+  SHMT_OK_(shmt_relabel(d_ids, N, 8, d_scratch, sbytes, d_unique, d_labels, h_count, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  std::unordered_map<int64_t, int64_t> first;
+  std::vector<int64_t> uniq;
+  for (int64_t x : ids)
+    if (first.emplace(x, static_cast<int64_t>(uniq.size())).second) uniq.push_back(x);
+  EXPECT(*h_count == static_cast<int64_t>(uniq.size()));
+  EXPECT(to_host(d_unique, uniq.size()) == uniq);
+  std::vector<int64_t> labels = to_host(d_labels, N);
+  for (int64_t i = 0; i < N; ++i) EXPECT(labels[i] == first[ids[i]]);
+
+  // ---- sampling: 7-row CSR of the reference's unit test, k = 5, no replacement ----
+  std::vector<int64_t> indptr = {0, 0, 4, 9, 15, 100, 101, 107}, indices(107), seeds = {5, 0, 1, 2, 3, 4, 6};
+  std::iota(indices.begin(), indices.end(), 0);
+  int64_t *d_indptr = to_device(indptr), *d_indices = to_device(indices), *d_seeds = to_device(seeds);
+  int64_t *d_sub_indptr = nullptr, *d_sub = nullptr;
+  HIP_OK(hipMalloc(&d_sub_indptr, 8 * 8));
+  HIP_OK(hipMalloc(&d_sub, 7 * 5 * 8));
+  const int64_t pbytes = shmt_sample_plan_bytes(7);
+  void *d_plan = nullptr;
+  HIP_OK(hipMalloc(&d_plan, pbytes));
+  SHMT_OK_(shmt_sample_plan(d_indptr, 8, nullptr, nullptr, d_seeds, 8, 7, 5, 0, d_sub_indptr, d_plan, pbytes,
+                            h_count, stream));
+  SHMT_OK_(shmt_sample_pick(d_indices, nullptr, 8, d_seeds, 8, 7, 5, 0, d_sub_indptr, 8, d_plan, d_sub, 7777, 0,
+                            stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  EXPECT(*h_count == 25);
+  EXPECT((to_host(d_sub_indptr, 8) == std::vector<int64_t>{0, 1, 1, 5, 10, 15, 20, 25}));
+  std::vector<int64_t> sub = to_host(d_sub, 25);
+  EXPECT((std::vector<int64_t>(sub.begin(), sub.begin() + 10) == std::vector<int64_t>{100, 0, 1, 2, 3, 4, 5, 6, 7, 8}));
+  for (int seg = 0; seg < 3; ++seg) {      // rows of degree 6, 85, 6: five distinct neighbours each
+    const int64_t lo[3] = {9, 15, 101}, hi[3] = {15, 100, 107};
+    std::vector<int64_t> s(sub.begin() + 10 + 5 * seg, sub.begin() + 15 + 5 * seg);
+    std::sort(s.begin(), s.end());
+    EXPECT(std::adjacent_find(s.begin(), s.end()) == s.end() && s.front() >= lo[seg] && s.back() < hi[seg]);
+  }
+
+  shmt_hashmap_destroy(map);
+  shmt_hashmap_destroy(fmap);
+  printf("cabi_smoke: all checks passed\n");
+  return 0;
+}
