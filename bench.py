@@ -14,6 +14,8 @@ all-hit / all-miss fetch rates, the cache_set pass, the hashmap microbenchmark
 baseline, and the end-to-end mini-batch of config 5 (per stage and whole batch).
 
 Benchmark configurations referred to by number in this file:
+  1  small fetch: 200,000 x 128 f32 table in pinned host memory, 50,000 random ids cached,
+     65,536 uniform queries (~25 % hits)
   2  static hashmap: 4,194,304 unique int64 keys in [0, 2^40) -> insertion index, load factor 0.5;
      16,777,216 queries, half members, half non-members
   3  cached sampling: R-MAT scale 21, edge factor 30 (a,b,c,d = .57,.19,.19,.05), symmetrised; int64
@@ -206,6 +208,14 @@ def bench_fetch(capi, args, result):
     extra["cache_set_262144"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(a, 1),
                                  "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
 
+    # scatter to the host table over the link (all misses): 262,144 uncached rows
+    sm = torch.randperm(N - C, device="cuda", generator=torch.Generator(device="cuda").manual_seed(10))[:ns] + C
+    t = gpu_time_ms(lambda: capi.cache_set(host, cache, sm, upd, hmap), 10)
+    torch.cuda.synchronize()
+    assert torch.equal(host[sm[:64].cpu()].view(torch.int16), upd[:64].cpu().view(torch.int16))
+    extra["cache_set_all_miss_262144"] = {"ms": round(t["median"], 4),
+                                          "host_link_write_GBs": round(ns * R / t["median"] / 1e6, 2)}
+
     # CPU baseline: the reference's cpu_fetch idiom is data[query.cpu()] (example/test_cache_fetch.py:138);
     # timed here as the oracle's OpenMP gather and as torch.index_select on the same batch
     if not args.no_cpu:
@@ -230,6 +240,44 @@ def bench_fetch(capi, args, result):
                       "OpenMP); torch.index_select with %d threads on the same batch: %.2f GB/s"
                       % (reps, torch.get_num_threads(), Q * R / torch_t / 1e9)}
     del host, cache, hmap
+
+
+# ---------------------------------------------------------------------------
+# config 1: small fetch, as specified (~25 % hits) plus all-hit and all-miss variants
+
+def bench_fetch_small(capi, args, result):
+    import torch
+    torch.manual_seed(0)
+    N, D, C, Q = 200_000, 128, 50_000, 65_536
+    R = D * 4
+    table = torch.randn(N, D).pin_memory()
+    ids = torch.randperm(N)[:C]
+    cache = table[ids].cuda()
+    ids = ids.cuda()
+    hmap = capi.CUCOStaticHashmap(ids, torch.arange(C, device="cuda"), 0.8)
+    q = torch.randint(0, N, (Q,)).cuda()
+    out = capi.cache_fetch(table, cache, q, hmap)
+    assert torch.equal(out.cpu(), torch.index_select(table, 0, q.cpu()))
+    hit = float((hmap.query(q) >= 0).float().mean())
+    q_hit = ids[torch.randint(0, C, (Q,), device="cuda")]
+    cached = torch.zeros(N, dtype=torch.bool, device="cuda")
+    cached[ids] = True
+    cold = torch.nonzero(~cached).flatten()
+    q_miss = cold[torch.randint(0, cold.numel(), (Q,), device="cuda")]
+    res = {"hit_rate": round(hit, 4)}
+    for name, qq in (("as_specified", q), ("all_hit", q_hit), ("all_miss", q_miss)):
+        t = gpu_time_ms(lambda: capi.cache_fetch(table, cache, qq, hmap), 30)
+        res[name] = {"ms": round(t["median"], 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 2),
+                     "algorithmic_GBs": round(Q * (2 * R + 8) / t["median"] / 1e6, 1)}
+    if not args.no_cpu:
+        qc = q.cpu()
+        torch.index_select(table, 0, qc)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            torch.index_select(table, 0, qc)
+        res["cpu_index_select_GBs"] = round(Q * R * 20 / (time.perf_counter() - t0) / 1e9, 2)
+        res["cpu_threads"] = torch.get_num_threads()
+    result["extra"]["fetch_config1"] = res
 
 
 # ---------------------------------------------------------------------------
@@ -470,6 +518,8 @@ def main():
     if "fetch" in todo:
         bench_fetch(capi, args, result)
         torch.cuda.empty_cache()
+    if "fetch" in todo and not args.headline_only:
+        bench_fetch_small(capi, args, result)
     if "hashmap" in todo:
         bench_hashmap(capi, args, result)
         torch.cuda.empty_cache()
