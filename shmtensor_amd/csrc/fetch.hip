@@ -197,7 +197,8 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   int mode = kDirect;
   if (map) {
     mode = map->fmt == kSlot16 ? kMap16 : kMap8;
-    SHMT_REQUIRE(cache != nullptr, "%s: cache table is null", who);
+    // an empty map never yields a slot, so an empty (null) cache table is fine with it
+    SHMT_REQUIRE(cache != nullptr || map->n == 0, "%s: cache table is null", who);
   } else if (mask) {
     mode = kMask;
     SHMT_REQUIRE(width_ok(mask_bytes), "%s: mask can only be int32 or int64", who);

@@ -252,7 +252,11 @@ torch::Tensor fetch_impl(const torch::Tensor &uva_data, const torch::Tensor *gpu
     TORCH_CHECK(m.numel() == numel, "mask and indices must have the same length");
   }
   if (numel == 0 || rs.row_bytes == 0) return output;
-  check(shmt_fetch(device_address(uva_data, "uva_data"), gpu_data ? gpu_data->data_ptr() : nullptr,
+  // an empty cache tensor has no storage; with a mask the C ABI wants a non-null table, and any
+  // addressable pointer will do because no mask entry may point into an empty cache
+  void *cache_ptr = nullptr;
+  if (gpu_data) cache_ptr = gpu_data->numel() > 0 ? gpu_data->data_ptr() : output.data_ptr();
+  check(shmt_fetch(device_address(uva_data, "uva_data"), cache_ptr,
                    indices.data_ptr(), static_cast<int>(indices.element_size()),
                    map ? map->handle() : nullptr, mask ? m.data_ptr() : nullptr,
                    mask ? static_cast<int>(m.element_size()) : 0, output.data_ptr(), numel,
@@ -278,7 +282,9 @@ void set_impl(torch::Tensor &uva_data, torch::Tensor *gpu_data, torch::Tensor in
     TORCH_CHECK(m.numel() == numel, "mask and indices must have the same length");
   }
   if (numel == 0 || rs.row_bytes == 0) return;
-  check(shmt_set(device_address(uva_data, "uva_data"), gpu_data ? gpu_data->data_ptr() : nullptr,
+  void *cache_ptr = nullptr;
+  if (gpu_data) cache_ptr = gpu_data->numel() > 0 ? gpu_data->data_ptr() : update.data_ptr();
+  check(shmt_set(device_address(uva_data, "uva_data"), cache_ptr,
                  indices.data_ptr(), static_cast<int>(indices.element_size()),
                  map ? map->handle() : nullptr, mask ? m.data_ptr() : nullptr,
                  mask ? static_cast<int>(m.element_size()) : 0, update.data_ptr(), numel,
