@@ -40,8 +40,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the config-4 fetch kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/rows_kernel_fetch_config4_pmc.md): 71,373.5 KiB x 2.0 (copy-calibrated) read + 262,144.1 KiB written.
-CONFIG4_TRAFFIC_BYTES = 414_608_592
+# (profiles/rows_kernel_fetch_config4_pmc.md): FETCH_SIZE x 2.0 (calibrated on a copy of known size) + WRITE_SIZE.
+CONFIG4_TRAFFIC_BYTES = 414_600_424
 
 
 def log(*a):
