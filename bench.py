@@ -344,28 +344,39 @@ def bench_sampling(capi, args, result):
     g = torch.Generator(device="cuda").manual_seed(33)
     seed_batches = [torch.randperm(n, device="cuda", generator=g)[:S].contiguous() for _ in range(nbatch)]
 
-    def run_batch(seeds, b):
+    def run_batch(seeds, b, fused=False):
         edges = 0
         for hop, k in enumerate(reversed(fanouts)):       # python/shmtensor/sampling.py:128
-            sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, hmap, seeds, k, False, seed=7777 + b,
-                                             stream_id=hop)
-            uniq, (_, rel) = capi.tensor_relabel([seeds, si])
+            if fused:     # the same two operators queued as one call (one host wait per hop)
+                sp, si, uniq, rel = capi.sample_hop(indptr, indices, gp, gi, hmap, seeds, k, False, seed=7777 + b,
+                                                    stream_id=hop)
+            else:
+                sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, hmap, seeds, k, False, seed=7777 + b,
+                                                 stream_id=hop)
+                uniq, (_, rel) = capi.tensor_relabel([seeds, si])
             edges += si.numel()
             seeds = uniq
         return edges
 
-    for b in range(3):
-        run_batch(seed_batches[b], b)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    edges = sum(run_batch(seed_batches[b], b) for b in range(nbatch))
-    torch.cuda.synchronize()
-    gpu_t = time.perf_counter() - t0
+    def timed(fused):
+        for b in range(3):
+            run_batch(seed_batches[b], b, fused)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        edges = sum(run_batch(seed_batches[b], b, fused) for b in range(nbatch))
+        torch.cuda.synchronize()
+        return edges, time.perf_counter() - t0
+
+    edges, gpu_t = timed(False)
+    edges_fused, gpu_t_fused = timed(True)
+    assert edges_fused == edges, "fused hop sampled a different number of edges"
     res = {"graph": "R-MAT scale %d ef 30 symmetrised: %d nodes, %d edges; top 30 %% by degree cached"
                     % (args.sampling_scale, n, indices.numel()),
            "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
            "edges_per_batch": edges // nbatch, "ms_per_batch": round(gpu_t * 1e3 / nbatch, 4),
-           "sampled_edges_per_s": round(edges / gpu_t, 1)}
+           "sampled_edges_per_s": round(edges / gpu_t, 1),
+           "fused_hop_ms_per_batch": round(gpu_t_fused * 1e3 / nbatch, 4),
+           "fused_hop_sampled_edges_per_s": round(edges / gpu_t_fused, 1)}
     if not args.no_cpu:
         from oracle import oracle as orc
         ip, ix = indptr.numpy(), indices.numpy().astype(np.int64)
@@ -419,13 +430,17 @@ def bench_e2e(capi, args, result):
     gs = torch.Generator(device="cuda").manual_seed(55)
     batches = [torch.randperm(n, device="cuda", generator=gs)[:S].contiguous() for _ in range(nbatch + 1)]
 
-    def one(seeds, b, ev=None):
+    def one(seeds, b, ev=None, fused=False):
         edges = 0
         if ev: ev[0].record()
         for hop, k in enumerate(reversed(fanouts)):
-            sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, adj_map, seeds, k, False, seed=7777 + b,
-                                             stream_id=hop)
-            uniq, (_, rel) = capi.tensor_relabel([seeds, si])
+            if fused:
+                sp, si, uniq, rel = capi.sample_hop(indptr, indices, gp, gi, adj_map, seeds, k, False, seed=7777 + b,
+                                                    stream_id=hop)
+            else:
+                sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, adj_map, seeds, k, False, seed=7777 + b,
+                                                 stream_id=hop)
+                uniq, (_, rel) = capi.tensor_relabel([seeds, si])
             edges += si.numel()
             seeds = uniq
         if ev: ev[1].record()
@@ -451,6 +466,17 @@ def bench_e2e(capi, args, result):
         tot_nodes += inp.numel()
         del x
     wall = time.perf_counter() - w0
+    # the same batches with each hop issued as one fused call
+    _, inp_f, x = one(batches[nbatch], nbatch, fused=True)
+    del x
+    torch.cuda.synchronize()
+    w0 = time.perf_counter()
+    for b in range(nbatch):
+        _, inp_f, x = one(batches[b], b, fused=True)
+        del x
+    torch.cuda.synchronize()
+    wall_fused = time.perf_counter() - w0
+    assert torch.equal(inp_f, inp), "fused hops gave different input nodes"
     result["extra"]["e2e_config5"] = {
         "graph": "R-MAT scale %d ef 16 symmetrised: %d nodes, %d edges; top 20 %% adjacency cached; features %d x %d "
                  "f32 pinned, top-degree 25 %% cached" % (args.e2e_scale, n, indices.numel(), n, D),
@@ -459,6 +485,7 @@ def bench_e2e(capi, args, result):
         "feature_hit_rate": round(hit, 4),
         "sample_relabel_ms": round(t_s / nbatch, 3), "fetch_ms": round(t_f / nbatch, 3),
         "batch_ms_wall": round(wall * 1e3 / nbatch, 3), "batches_per_s": round(nbatch / wall, 2),
+        "fused_hop_batch_ms_wall": round(wall_fused * 1e3 / nbatch, 3),
         "sampled_edges_per_s": round(tot_edges / (t_s * 1e-3), 1),
         "fetch_payload_GBs": round(tot_nodes * D * 4 / (t_f * 1e-3) / 1e9, 2)}
 

@@ -151,13 +151,20 @@ int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
  * segments seg_ptrs[s] of seg_lens[s] ids, seg_bytes[s] in {4,8} wide, are
  * widened to elem_bytes (the width torch::cat would promote to) and written
  * to total_out (N = sum of seg_lens elements), which then plays the role of
- * `total` above. The three arrays are host arrays read during the call.     */
+ * `total` above. The three arrays are host arrays read during the call.
+ * When last_len_dev is not NULL the true length of the LAST segment is read by
+ * the kernels from that device address (an integer last_len_bytes in {4,8}
+ * wide, e.g. sub_indptr[S] written by shmt_sample_plan earlier on the same
+ * stream) and seg_lens[nseg-1] is only its upper bound: launches, scratch,
+ * total_out, unique_out and labels_out are sized for the bound, results cover
+ * the true length. This lets a caller queue sampling and relabel of one hop
+ * without learning nnz on the host in between.                             */
 #define SHMT_RELABEL_MAX_SEGMENTS 8
 int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens,
-                          const int *seg_bytes, int nseg, int elem_bytes,
-                          void *total_out, void *scratch, int64_t scratch_bytes,
-                          void *unique_out, void *labels_out, int64_t *count_out,
-                          void *stream);
+                          const int *seg_bytes, int nseg, const void *last_len_dev,
+                          int last_len_bytes, int elem_bytes, void *total_out,
+                          void *scratch, int64_t scratch_bytes, void *unique_out,
+                          void *labels_out, int64_t *count_out, void *stream);
 
 /* ------------------------------------------------------------------ */
 /* Neighbour sampling: CSRWiseSampling src/cache_graph_sampling.cu:179-220

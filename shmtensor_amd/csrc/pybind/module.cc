@@ -468,7 +468,7 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
       widths[i] = static_cast<int>(keep[i].element_size());
     }
     torch::Tensor total = torch::empty({N}, options);
-    check(shmt_relabel_segments(ptrs, lens, widths, static_cast<int>(tensors.size()), eb,
+    check(shmt_relabel_segments(ptrs, lens, widths, static_cast<int>(tensors.size()), nullptr, 0, eb,
                                 total.data_ptr(), scratch.data_ptr(), scratch_bytes,
                                 unique.data_ptr(), labels.data_ptr(), count.dev, current_stream()));
   } else {
@@ -478,6 +478,83 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
   }
   const int64_t U = Readback::wait(count);
   return std::make_tuple(unique.narrow(0, 0, U), labels.split_with_sizes(split_sizes, 0));
+}
+
+// One hop of mini-batch sampling as the dataloader runs it
+// (python/shmtensor/sampling.py:128-143): sample the seeds, then relabel
+// [seeds, sub_indices]. No counterpart as a single operator in the reference.
+// All kernels of the hop are queued without the host learning nnz in between
+// (the relabel kernels read it from sub_indptr[S] on the device); nnz and the
+// number of unique ids are picked up together at the end. Returns
+// (sub_indptr, sub_indices, unique, relabel_indices): exactly what
+// csr_[cache_]sampling followed by tensor_relabel([seeds, sub_indices]) returns,
+// with relabel_indices = the labels of the sub_indices part.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> sample_hop(
+    torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
+    std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, torch::Tensor seeds,
+    int64_t num_picks, bool replace, std::optional<int64_t> seed, int64_t stream_id) {
+  const bool cached = hashmap != nullptr;
+  TORCH_CHECK(!cached || (gpu_indptr.has_value() && gpu_indices.has_value()),
+              "sample_hop: a hashmap needs gpu_indptr and gpu_indices");
+  seeds = cuda_ids(seeds, "seeds");
+  const int64_t S = seeds.numel();
+  const bool fused = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
+  if (!fused) {  // degenerate or very large bound: the two operators one after the other
+    auto sampled = sample_impl(indptr, indices, cached ? &*gpu_indptr : nullptr,
+                               cached ? &*gpu_indices : nullptr, hashmap, seeds, num_picks, replace,
+                               seed, stream_id);
+    auto relabeled = tensor_relabel({seeds, std::get<1>(sampled)});
+    return std::make_tuple(std::get<0>(sampled), std::get<1>(sampled), std::get<0>(relabeled),
+                           std::get<1>(relabeled)[1]);
+  }
+  const int pb = id_bytes(indptr, "indptr"), ib = id_bytes(indices, "indices");
+  const int sb = static_cast<int>(seeds.element_size());
+  TORCH_CHECK(indptr.is_contiguous() && indices.is_contiguous(), "CSR arrays must be contiguous");
+  if (cached) {
+    TORCH_CHECK(gpu_indptr->is_cuda() && gpu_indices->is_cuda() && gpu_indptr->is_contiguous() &&
+                    gpu_indices->is_contiguous(),
+                "gpu_indptr and gpu_indices must be contiguous CUDA tensors");
+    TORCH_CHECK(gpu_indptr->scalar_type() == indptr.scalar_type() &&
+                    gpu_indices->scalar_type() == indices.scalar_type(),
+                "cached CSR must have the dtypes of the full CSR");
+  }
+  const auto dev = torch::kCUDA;
+  void *stream = current_stream();
+  const int64_t bound = S * num_picks;
+  torch::Tensor sub_indptr = torch::empty({S + 1}, indptr.options().device(dev));
+  torch::Tensor sub_indices = torch::empty({bound}, indices.options().device(dev));
+  const int64_t plan_bytes = shmt_sample_plan_bytes(S);
+  torch::Tensor plan = device_bytes(plan_bytes);
+  const Readback::Slot nnz_slot = readback().acquire();
+  check(shmt_sample_plan(device_address(indptr, "indptr"), pb, cached ? gpu_indptr->data_ptr() : nullptr,
+                         cached ? hashmap->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks,
+                         replace, sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, nnz_slot.dev,
+                         stream));
+  check(shmt_sample_pick(device_address(indices, "indices"), cached ? gpu_indices->data_ptr() : nullptr,
+                         ib, seeds.data_ptr(), sb, S, num_picks, replace, sub_indptr.data_ptr(), pb,
+                         plan.data_ptr(), sub_indices.data_ptr(),
+                         static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
+                         static_cast<uint32_t>(stream_id), stream));
+  // relabel [seeds, sub_indices]; the second length is read from sub_indptr[S] by the kernels
+  const int eb = std::max(sb, ib);
+  const auto id_options = seeds.options().dtype(eb == 8 ? torch::kInt64 : torch::kInt32);
+  const int64_t n_max = S + bound;
+  torch::Tensor total = torch::empty({n_max}, id_options);
+  torch::Tensor unique = torch::empty({n_max}, id_options);
+  torch::Tensor labels = torch::empty({n_max}, id_options);
+  const int64_t scratch_bytes = shmt_relabel_scratch_bytes(n_max);
+  torch::Tensor scratch = device_bytes(scratch_bytes);
+  const void *ptrs[2] = {seeds.data_ptr(), sub_indices.data_ptr()};
+  const int64_t lens[2] = {S, bound};
+  const int widths[2] = {sb, ib};
+  const Readback::Slot count_slot = readback().acquire();
+  check(shmt_relabel_segments(ptrs, lens, widths, 2, static_cast<char *>(sub_indptr.data_ptr()) + S * pb,
+                              pb, eb, total.data_ptr(), scratch.data_ptr(), scratch_bytes,
+                              unique.data_ptr(), labels.data_ptr(), count_slot.dev, stream));
+  const int64_t nnz = Readback::wait(nnz_slot);
+  const int64_t U = Readback::wait(count_slot);
+  return std::make_tuple(sub_indptr, sub_indices.narrow(0, 0, nnz), unique.narrow(0, 0, U),
+                         labels.narrow(0, S, nnz));
 }
 
 }  // namespace
@@ -511,7 +588,10 @@ PYBIND11_MODULE(ShmTensorLib, m) {
            py::arg("seed") = py::none(), py::arg("stream_id") = 0)
       .def("create_subcsr", &create_subcsr, py::arg("uva_indptr"), py::arg("uva_indices"),
            py::arg("seeds"))
-      .def("tensor_relabel", &tensor_relabel, py::arg("tensors"));
+      .def("tensor_relabel", &tensor_relabel, py::arg("tensors"))
+      .def("sample_hop", &sample_hop, py::arg("indptr"), py::arg("indices"), py::arg("gpu_indptr"),
+           py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"),
+           py::arg("replace"), py::arg("seed") = py::none(), py::arg("stream_id") = 0);
 
   py::class_<StaticHashmap>(m, "CUCOStaticHashmap")
       .def(py::init<torch::Tensor, torch::Tensor, double>())

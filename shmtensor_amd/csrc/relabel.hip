@@ -26,6 +26,24 @@ constexpr int kRlItems = 8;
 constexpr int kRlTile = kRlBlock * kRlItems;
 constexpr int64_t kRlSelfPrefixTiles = 2048;  // up to 4 M ids the unique pass sums the tile counts itself
 
+// Number of input ids: a host-known part plus, optionally, a part that only
+// the device knows (the length of the last segment, e.g. the nnz a sampling
+// kernel produced earlier on the same stream).
+struct RlCount {
+  int64_t fixed;
+  const void *extra;  // device address of the extra length, or null
+  int extra_bytes;    // its width, 4 or 8
+  int64_t limit;      // what launches and buffers were sized for; the count is clamped to it
+};
+
+__device__ __forceinline__ int64_t rl_count(const RlCount &n) {
+  if (!n.extra) return n.fixed;
+  int64_t extra = load_int(n.extra, 0, n.extra_bytes);
+  if (extra < 0) extra = 0;
+  const int64_t N = n.fixed + extra;
+  return N < n.limit ? N : n.limit;
+}
+
 struct RlSlot {
   int64_t key;
   uint32_t first;
@@ -86,10 +104,11 @@ constexpr int kRlLdsSlots = 2 * kRlInsertTile;   // per-workgroup staging table,
 // Insert pass. Ids of hub nodes repeat thousands of times in a sampled batch,
 // and atomics on one address serialise in L2, so every workgroup first
 // de-duplicates its 256 ids in an LDS table (key -> smallest index among
-// them) and sends one global insert per distinct id; each thread then has at
-// most a couple of dependent global probe chains.
+// them) and sends one global insert per distinct id, issued by the thread that
+// holds the id's smallest index: at most one global probe chain per thread.
 __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32_t cap,
-                                                             const void *total, int eb, int64_t N) {
+                                                             const void *total, int eb, RlCount n) {
+  const int64_t N = rl_count(n);
   __shared__ unsigned long long lkey[kRlLdsSlots];
   __shared__ uint32_t lfirst[kRlLdsSlots];
   const int64_t ntiles = (N + kRlInsertTile - 1) / kRlInsertTile;
@@ -100,9 +119,12 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
     }
     __syncthreads();
     const int64_t i = tile * kRlInsertTile + threadIdx.x;
+    int64_t key = 0;
+    uint32_t pos = 0;
     if (i < N) {
-      const int64_t key = load_int(total, i, eb);
-      uint32_t pos = hash_id(key) & (kRlLdsSlots - 1);
+      key = load_int(total, i, eb);
+      pos = hash_id(key) & (kRlLdsSlots - 1);
+      // the staging table has twice as many slots as the tile has ids: a free slot always turns up
       for (int probes = 0; probes < kRlLdsSlots; ++probes) {
         const unsigned long long prev =
             atomicCAS(&lkey[pos], ~0ull, static_cast<unsigned long long>(key));
@@ -114,10 +136,10 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
       }
     }
     __syncthreads();
-    for (int t = threadIdx.x; t < kRlLdsSlots; t += kRlBlock) {
-      const unsigned long long k = lkey[t];
-      if (k != ~0ull) rl_global_insert(tbl, cap, static_cast<int64_t>(k), lfirst[t]);
-    }
+    // the thread holding the smallest index of an id inserts it for the whole tile:
+    // one global probe chain per thread at most
+    if (i < N && lfirst[pos] == static_cast<uint32_t>(i))
+      rl_global_insert(tbl, cap, key, static_cast<uint32_t>(i));
     __syncthreads();
   }
 }
@@ -126,8 +148,9 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
 // thread's eight elements are issued together; only the rare longer probe
 // chains continue one by one.
 __global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
-                                                            const void *total, int eb, int64_t N,
+                                                            const void *total, int eb, RlCount n,
                                                             void *labels, uint64_t *partials) {
+  const int64_t N = rl_count(n);
   __shared__ uint64_t lds[kRlBlock / kWave];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kRlTile;
   int64_t key[kRlItems], idx[kRlItems];
@@ -172,11 +195,12 @@ __global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, u
   if (threadIdx.x == 0) partials[blockIdx.x] = tile_total;
 }
 
-__global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, int eb, int64_t N,
+__global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, int eb, RlCount n,
                                                              const void *labels,
                                                              const uint64_t *partials,
                                                              void *unique_out, uint32_t *rank_of,
                                                              int64_t *count_out, int scanned) {
+  const int64_t N = rl_count(n);
   __shared__ uint32_t lds[kRlBlock / kWave];
   __shared__ uint64_t lds64[kRlBlock / kWave];
   // Tile prefix: either already scanned by a separate launch, or (few tiles)
@@ -222,14 +246,17 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
       ++rank;
     }
   }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+  // the workgroup holding the last id reports the number of distinct ids
+  const int64_t last_tile = N > 0 ? (N - 1) / kRlTile : 0;
+  if (static_cast<int64_t>(blockIdx.x) == last_tile && threadIdx.x == 0) {
     *count_out = static_cast<int64_t>(tile_prefix + tile_total);
     __threadfence_system();
   }
 }
 
-__global__ __launch_bounds__(256) void rl_labels_kernel(void *labels, int eb, int64_t N,
+__global__ __launch_bounds__(256) void rl_labels_kernel(void *labels, int eb, RlCount n,
                                                         const uint32_t *rank_of) {
+  const int64_t N = rl_count(n);
   int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (; i < N; i += stride) {
@@ -248,7 +275,8 @@ struct RlSegments {
 // First pass when the input arrives as segments: empties the table and writes
 // the concatenated, widened ids in one sweep (both are streaming stores).
 __global__ __launch_bounds__(256) void rl_fill_concat_kernel(uint4 *tbl16, int64_t cap, RlSegments segs,
-                                                             void *total, int eb, int64_t N) {
+                                                             void *total, int eb, RlCount n) {
+  const int64_t N = rl_count(n);
   int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   const int64_t span = cap > N ? cap : N;
@@ -279,9 +307,12 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
   return rl_layout(N).total;
 }
 
-static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, int elem_bytes,
-                        void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
-                        int64_t *count_out, void *stream) {
+// N is the host-known number of ids, or an upper bound of it when `n.extra`
+// names a device-side length: launches and scratch are sized for N, the
+// kernels work on the true count.
+static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
+                        int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
+                        void *labels_out, int64_t *count_out, void *stream) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
@@ -313,17 +344,17 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, in
     const int64_t span = l.cap > N ? l.cap : N;
     hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(span, 256 * 4)), dim3(256), 0, s,
                        reinterpret_cast<uint4 *>(tbl), l.cap, *segs, const_cast<void *>(total),
-                       elem_bytes, N);
+                       elem_bytes, n);
     SHMT_LAUNCH_CHECK();
   } else {
     rc = launch_fill_ones(tbl, l.cap, s);
     if (rc) return rc;
   }
   hipLaunchKernelGGL(rl_insert_kernel, dim3(grid_for(N, kRlInsertTile, 256 * 32)), dim3(kRlBlock), 0,
-                     s, tbl, cap, total, elem_bytes, N);
+                     s, tbl, cap, total, elem_bytes, n);
   SHMT_LAUNCH_CHECK();
   hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, tbl,
-                     cap, total, elem_bytes, N, labels_out, partials);
+                     cap, total, elem_bytes, n, labels_out, partials);
   SHMT_LAUNCH_CHECK();
   const int scanned = nb > kRlSelfPrefixTiles;
   if (scanned) {
@@ -331,11 +362,11 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, in
     if (rc) return rc;
   }
   hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s,
-                     total, elem_bytes, N, labels_out, partials, unique_out, rank_of, count_out,
+                     total, elem_bytes, n, labels_out, partials, unique_out, rank_of, count_out,
                      scanned);
   SHMT_LAUNCH_CHECK();
   hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, labels_out,
-                     elem_bytes, N, rank_of);
+                     elem_bytes, n, rank_of);
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;
 }
@@ -343,17 +374,19 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, in
 int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
                  void *stream) {
-  return relabel_impl(total, nullptr, N, elem_bytes, scratch, scratch_bytes, unique_out, labels_out,
-                      count_out, stream);
+  return relabel_impl(total, nullptr, N, RlCount{N, nullptr, 8, N}, elem_bytes, scratch, scratch_bytes,
+                      unique_out, labels_out, count_out, stream);
 }
 
 int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, const int *seg_bytes,
-                          int nseg, int elem_bytes, void *total_out, void *scratch,
-                          int64_t scratch_bytes, void *unique_out, void *labels_out,
-                          int64_t *count_out, void *stream) {
+                          int nseg, const void *last_len_dev, int last_len_bytes, int elem_bytes,
+                          void *total_out, void *scratch, int64_t scratch_bytes, void *unique_out,
+                          void *labels_out, int64_t *count_out, void *stream) {
   SHMT_REQUIRE(nseg >= 1 && nseg <= SHMT_RELABEL_MAX_SEGMENTS,
                "shmt_relabel_segments: between 1 and %d segments", SHMT_RELABEL_MAX_SEGMENTS);
   SHMT_REQUIRE(seg_ptrs && seg_lens && seg_bytes, "shmt_relabel_segments: null segment arrays");
+  SHMT_REQUIRE(last_len_dev == nullptr || width_ok(last_len_bytes),
+               "shmt_relabel_segments: last_len_bytes must be 4 or 8");
   RlSegments segs;
   segs.n = nseg;
   int64_t N = 0;
@@ -373,7 +406,14 @@ int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, 
     segs.bytes[i] = 8;
   }
   SHMT_REQUIRE(N == 0 || total_out != nullptr, "shmt_relabel_segments: total_out is null");
-  return relabel_impl(total_out, &segs, N, elem_bytes, scratch, scratch_bytes, unique_out,
+  RlCount n{N, nullptr, 8, N};
+  if (last_len_dev) {
+    // the last segment's true length lives on the device; N stays the bound
+    n.fixed = N - seg_lens[nseg - 1];
+    n.extra = last_len_dev;
+    n.extra_bytes = last_len_bytes;
+  }
+  return relabel_impl(total_out, &segs, N, n, elem_bytes, scratch, scratch_bytes, unique_out,
                       labels_out, count_out, stream);
 }
 

@@ -2,7 +2,8 @@
 ShmTensorLib operators. Same constructor, iteration protocol, cache
 management and return values as python/shmtensor/sampling.py:30-237 in the
 reference; the per-hop work is `csr_sampling` / `csr_cache_sampling` followed
-by `tensor_relabel([seeds, sub_indices])`.
+by `tensor_relabel([seeds, sub_indices])`, issued through the fused
+`sample_hop` operator (same results, one host wait per hop instead of two).
 
 Without DGL installed a block is a `CSCBlock` tuple (indptr, indices,
 num_src, num_dst); with DGL it is the DGLBlock the reference builds
@@ -120,6 +121,17 @@ class GPUSamplingDataloader:
                                            self.hashmap, seeds, num_pick, self.replace, **extra)
         return capi.csr_sampling(self.indptr, self.indices, seeds, num_pick, self.replace, **extra)
 
+    def _hop(self, seeds, num_pick, hop):
+        """Sampling and relabel of one hop as one operator: all its kernels are
+        queued before the host waits for either data-dependent size."""
+        extra = {}
+        if self.rng_seed is not None:
+            extra = {"seed": int(self.rng_seed) + self._batches_drawn, "stream_id": hop}
+        cached = self.has_cache
+        return capi.sample_hop(self.indptr, self.indices, self.gpu_indptr if cached else None,
+                               self.gpu_indices if cached else None, self.hashmap if cached else None,
+                               seeds, num_pick, self.replace, **extra)
+
     def __next__(self):
         if self.curr >= self.len:
             raise StopIteration
@@ -130,8 +142,7 @@ class GPUSamplingDataloader:
         blocks = []
         # the last fanout is applied to the seed layer (sampling.py:128)
         for hop, num_pick in enumerate(reversed(self.num_picks)):
-            sub_indptr, sub_indices = self._sample(seeds, num_pick, hop)
-            unique_tensor, (_, relabel_indices) = capi.tensor_relabel([seeds, sub_indices])
+            sub_indptr, _, unique_tensor, relabel_indices = self._hop(seeds, num_pick, hop)
             blocks.insert(0, create_block_from_csc(sub_indptr, relabel_indices, torch.Tensor(),
                                                    unique_tensor.numel(), seeds.numel()))
             seeds = unique_tensor

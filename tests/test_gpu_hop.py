@@ -1,0 +1,167 @@
+"""One fused hop (sample + relabel queued without a host wait between them)
+against the two separate operators it replaces, and the device-side segment
+length of shmt_relabel_segments against the oracle. Bit-exact throughout."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from shmtensor_amd.synthetic import rmat_csr
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(scale=14, edge_factor=12, seed=3, ptr_dt=torch.int64, idx_dt=torch.int64):
+    indptr, indices = rmat_csr(scale, edge_factor, seed)
+    return indptr.to(ptr_dt), indices.to(idx_dt)
+
+
+def _two_step(capi, indptr, indices, cache, seeds, k, replace, **kw):
+    if cache is None:
+        sp, si = capi.csr_sampling(indptr, indices, seeds, k, replace, **kw)
+    else:
+        gp, gi, h = cache
+        sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, h, seeds, k, replace, **kw)
+    uniq, (_, lab) = capi.tensor_relabel([seeds, si])
+    return sp, si, uniq, lab
+
+
+def _hop(capi, indptr, indices, cache, seeds, k, replace, **kw):
+    gp, gi, h = cache if cache is not None else (None, None, None)
+    return capi.sample_hop(indptr, indices, gp, gi, h, seeds, k, replace, **kw)
+
+
+def _same(a, b):
+    assert len(a) == len(b)
+    for x, y in zip(a, b):
+        assert x.dtype == y.dtype and x.shape == y.shape and x.device == y.device
+        assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("replace", [False, True])
+@pytest.mark.parametrize("k", [1, 5, 25, 64, 100])
+@pytest.mark.parametrize("seed_dt", [torch.int32, torch.int64])
+def test_hop_equals_sampling_then_relabel_device_graph(capi, replace, k, seed_dt):
+    indptr, indices = _graph()
+    indptr, indices = indptr.cuda(), indices.cuda()
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(k)
+    for S in (1, 7, 1024, 1025, 6000):
+        seeds = torch.randint(0, n, (S,), generator=g).to(seed_dt).cuda()   # with repeats
+        _same(_hop(capi, indptr, indices, None, seeds, k, replace),
+              _two_step(capi, indptr, indices, None, seeds, k, replace))
+
+
+@pytest.mark.parametrize("ptr_dt,idx_dt", [(torch.int64, torch.int32), (torch.int32, torch.int32),
+                                           (torch.int64, torch.int64)])
+def test_hop_cached_pinned_graph(capi, ptr_dt, idx_dt):
+    indptr, indices = _graph(ptr_dt=ptr_dt, idx_dt=idx_dt)
+    indptr, indices = indptr.cpu().pin_memory(), indices.cpu().pin_memory()
+    n = indptr.numel() - 1
+    hot = torch.randperm(n, generator=torch.Generator().manual_seed(1))[: n // 4].cuda()
+    gp, gi = capi.create_subcsr(indptr, indices, hot)
+    h = capi.CUCOStaticHashmap(hot.int(), torch.arange(hot.numel(), dtype=torch.int32).cuda(), 0.8)
+    cache = (gp, gi, h)
+    seeds = torch.randperm(n, generator=torch.Generator().manual_seed(2))[:3000].int().cuda()
+    for replace in (False, True):
+        for kw in ({}, {"seed": 99, "stream_id": 3}):
+            got = _hop(capi, indptr, indices, cache, seeds, 10, replace, **kw)
+            _same(got, _two_step(capi, indptr, indices, cache, seeds, 10, replace, **kw))
+            _same(got, _hop(capi, indptr, indices, None, seeds, 10, replace, **kw))   # cache is transparent
+
+
+def test_hop_degenerate_inputs(capi):
+    # node 0: 3 neighbours, node 1: none, node 2: 1 neighbour
+    indptr = torch.tensor([0, 3, 3, 4]).cuda()
+    indices = torch.tensor([2, 1, 0, 2]).cuda()
+    empty = torch.empty(0, dtype=torch.int64).cuda()
+    sp, si, uniq, lab = capi.sample_hop(indptr, indices, None, None, None, empty, 5, False)
+    assert sp.tolist() == [0] and si.numel() == 0 and uniq.numel() == 0 and lab.numel() == 0
+    only_isolated = torch.tensor([1, 1]).cuda()
+    sp, si, uniq, lab = capi.sample_hop(indptr, indices, None, None, None, only_isolated, 5, False)
+    assert sp.tolist() == [0, 0, 0] and si.numel() == 0 and uniq.tolist() == [1] and lab.numel() == 0
+    seeds = torch.tensor([2, 1, 0]).cuda()
+    sp, si, uniq, lab = capi.sample_hop(indptr, indices, None, None, None, seeds, 5, False)
+    assert sp.tolist() == [0, 1, 1, 4] and si[0].item() == 2 and sorted(si[1:].tolist()) == [0, 1, 2]
+    assert uniq.tolist() == [2, 1, 0] and torch.equal(uniq[lab], si)
+    sp0, si0, uniq0, lab0 = capi.sample_hop(indptr, indices, None, None, None, seeds, 0, False)
+    assert sp0.tolist() == [0, 0, 0, 0] and si0.numel() == 0 and uniq0.tolist() == [2, 1, 0]
+    with pytest.raises(RuntimeError):
+        capi.sample_hop(indptr, indices, None, None, None, seeds.float(), 5, False)
+
+
+def test_hop_chain_matches_dataloader_protocol(capi):
+    """Three hops chained as the dataloader does (python/shmtensor/sampling.py:128-143):
+    the unique ids of one hop seed the next; seeds stay a prefix of unique."""
+    indptr, indices = _graph(scale=15)
+    indptr, indices = indptr.cuda(), indices.cuda()
+    seeds = torch.randperm(indptr.numel() - 1, generator=torch.Generator().manual_seed(5))[:1000].cuda()
+    a = b = seeds
+    for hop, k in enumerate([10, 10, 5]):
+        got = _hop(capi, indptr, indices, None, a, k, False, seed=11, stream_id=hop)
+        want = _two_step(capi, indptr, indices, None, b, k, False, seed=11, stream_id=hop)
+        _same(got, want)
+        assert torch.equal(got[2][: a.numel()], a)
+        assert torch.equal(got[2][got[3]], got[1])
+        a, b = got[2], want[2]
+
+
+@pytest.mark.parametrize("len_bytes", [4, 8])
+@pytest.mark.parametrize("true_len", [0, 1, 2047, 2048, 5000, 20000])
+def test_relabel_segments_device_length(cabi, oracle, len_bytes, true_len):
+    """The last segment's length read on the device: buffers and launches sized
+    for the bound, results those of the true length."""
+    lib = cabi.load()
+    rng = np.random.default_rng(true_len + len_bytes)
+    head = rng.integers(0, 3000, size=700).astype(np.int32)
+    bound = 20000
+    tail = rng.integers(0, 3000, size=bound).astype(np.int64)      # entries past true_len must be ignored
+    exp_unique, exp_parts = oracle.relabel([head, tail[:true_len]])
+    exp_labels = np.concatenate(exp_parts)
+    d_head, d_tail = torch.from_numpy(head).cuda(), torch.from_numpy(tail).cuda()
+    d_len = torch.tensor([true_len], dtype=torch.int32 if len_bytes == 4 else torch.int64).cuda()
+    n_max = head.size + bound
+    total = torch.empty(n_max, dtype=torch.int64).cuda()
+    unique = torch.empty(n_max, dtype=torch.int64).cuda()
+    labels = torch.empty(n_max, dtype=torch.int64).cuda()
+    sbytes = lib.shmt_relabel_scratch_bytes(n_max)
+    scratch = torch.empty(sbytes, dtype=torch.uint8).cuda()
+    count = torch.full((1,), -5, dtype=torch.int64).cuda()
+    vp = ctypes.c_void_p
+    ptrs = (vp * 2)(d_head.data_ptr(), d_tail.data_ptr())
+    lens = (ctypes.c_int64 * 2)(head.size, bound)
+    widths = (ctypes.c_int * 2)(4, 8)
+    cabi.check(lib.shmt_relabel_segments(ptrs, lens, widths, 2, d_len.data_ptr(), len_bytes, 8,
+                                         total.data_ptr(), scratch.data_ptr(), sbytes, unique.data_ptr(),
+                                         labels.data_ptr(), count.data_ptr(), cabi.current_stream()))
+    torch.cuda.synchronize()
+    n = head.size + true_len
+    u = int(count.item())
+    assert u == exp_unique.size
+    assert np.array_equal(unique[:u].cpu().numpy(), exp_unique)
+    assert np.array_equal(labels[:n].cpu().numpy(), exp_labels)
+    assert np.array_equal(total[:n].cpu().numpy(), np.concatenate([head.astype(np.int64), tail[:true_len]]))
+
+
+def test_relabel_segments_device_length_clamped_and_rejected(cabi):
+    lib = cabi.load()
+    head = torch.arange(10, dtype=torch.int64).cuda()
+    tail = torch.arange(5, 15, dtype=torch.int64).cuda()
+    too_long = torch.tensor([1000], dtype=torch.int64).cuda()       # beyond the bound: clamped to it
+    total, unique, labels = (torch.empty(20, dtype=torch.int64).cuda() for _ in range(3))
+    sbytes = lib.shmt_relabel_scratch_bytes(20)
+    scratch = torch.empty(sbytes, dtype=torch.uint8).cuda()
+    count = torch.zeros(1, dtype=torch.int64).cuda()
+    vp = ctypes.c_void_p
+    ptrs = (vp * 2)(head.data_ptr(), tail.data_ptr())
+    lens = (ctypes.c_int64 * 2)(10, 10)
+    widths = (ctypes.c_int * 2)(8, 8)
+    args = (total.data_ptr(), scratch.data_ptr(), sbytes, unique.data_ptr(), labels.data_ptr(), count.data_ptr(),
+            cabi.current_stream())
+    cabi.check(lib.shmt_relabel_segments(ptrs, lens, widths, 2, too_long.data_ptr(), 8, 8, *args))
+    torch.cuda.synchronize()
+    assert count.item() == 15 and unique[:15].tolist() == list(range(15))
+    assert labels.tolist() == list(range(10)) + list(range(5, 15))
+    assert lib.shmt_relabel_segments(ptrs, lens, widths, 2, too_long.data_ptr(), 3, 8, *args) == -1
+    assert b"last_len_bytes" in lib.shmt_last_error()
