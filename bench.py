@@ -367,16 +367,39 @@ def bench_sampling(capi, args, result):
         torch.cuda.synchronize()
         return edges, time.perf_counter() - t0
 
+    picks = list(reversed(fanouts))
+
+    def timed_in_flight(in_flight):
+        """All batches through sample_blocks: up to `in_flight` of them advance concurrently."""
+        rng = [7777 + b for b in range(nbatch)]
+        for _ in range(2):
+            capi.sample_blocks(indptr, indices, gp, gi, hmap, seed_batches, picks, False, seeds_rng=rng,
+                               max_in_flight=in_flight)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        res = capi.sample_blocks(indptr, indices, gp, gi, hmap, seed_batches, picks, False, seeds_rng=rng,
+                                 max_in_flight=in_flight)
+        torch.cuda.synchronize()
+        t = time.perf_counter() - t0
+        return sum(hop[1].numel() for chain in res for hop in chain), t
+
     edges, gpu_t = timed(False)
     edges_fused, gpu_t_fused = timed(True)
     assert edges_fused == edges, "fused hop sampled a different number of edges"
+    overlapped = {}
+    for in_flight in (1, 2, 4, 8, 16):
+        e, t = timed_in_flight(in_flight)
+        assert e == edges, "batched hops sampled a different number of edges"
+        overlapped["%d_batches_in_flight" % in_flight] = {"ms_per_batch": round(t * 1e3 / nbatch, 4),
+                                                          "sampled_edges_per_s": round(e / t, 1)}
     res = {"graph": "R-MAT scale %d ef 30 symmetrised: %d nodes, %d edges; top 30 %% by degree cached"
                     % (args.sampling_scale, n, indices.numel()),
            "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
            "edges_per_batch": edges // nbatch, "ms_per_batch": round(gpu_t * 1e3 / nbatch, 4),
            "sampled_edges_per_s": round(edges / gpu_t, 1),
            "fused_hop_ms_per_batch": round(gpu_t_fused * 1e3 / nbatch, 4),
-           "fused_hop_sampled_edges_per_s": round(edges / gpu_t_fused, 1)}
+           "fused_hop_sampled_edges_per_s": round(edges / gpu_t_fused, 1),
+           "sample_blocks_batches_in_flight": overlapped}
     if not args.no_cpu:
         from oracle import oracle as orc
         ip, ix = indptr.numpy(), indices.numpy().astype(np.int64)
@@ -477,6 +500,40 @@ def bench_e2e(capi, args, result):
     torch.cuda.synchronize()
     wall_fused = time.perf_counter() - w0
     assert torch.equal(inp_f, inp), "fused hops gave different input nodes"
+    # sampling + relabel only, several batches advancing concurrently
+    in_flight_ms = {}
+    for k_in_flight in (1, 4, 8):
+        rng = [7777 + b for b in range(nbatch)]
+        capi.sample_blocks(indptr, indices, gp, gi, adj_map, batches[:nbatch], list(reversed(fanouts)), False,
+                           seeds_rng=rng, max_in_flight=k_in_flight)
+        torch.cuda.synchronize()
+        w0 = time.perf_counter()
+        chains = capi.sample_blocks(indptr, indices, gp, gi, adj_map, batches[:nbatch], list(reversed(fanouts)), False,
+                                    seeds_rng=rng, max_in_flight=k_in_flight)
+        torch.cuda.synchronize()
+        in_flight_ms[str(k_in_flight)] = round((time.perf_counter() - w0) * 1e3 / nbatch, 3)
+        assert torch.equal(chains[nbatch - 1][-1][2], inp), "sample_blocks gave different input nodes"
+        del chains
+    # the dataloader sampling ahead on a background thread (4 batches in flight) while this thread fetches
+    import shmtensor
+    dl = shmtensor.GPUSamplingDataloader(indptr, indices, torch.cat(batches[:nbatch]), S, fanouts, shuffle=False,
+                                         rng_seed=7777, prefetch=4, background=True)
+    dl.gpu_indptr, dl.gpu_indices, dl.hashmap, dl.has_cache = gp, gi, adj_map, True
+
+    def epoch():
+        last = None
+        for input_nodes, _, _ in dl:
+            x = capi.cache_fetch(feats, feat_cache, input_nodes, feat_map)
+            last = input_nodes
+            del x
+        torch.cuda.synchronize()
+        return last
+
+    # first epoch: batch b draws from seed 7777 + b like the loops above (later epochs continue the count)
+    assert torch.equal(epoch(), inp), "prefetching dataloader gave different input nodes"
+    w0 = time.perf_counter()
+    epoch()
+    wall_pipe = time.perf_counter() - w0
     result["extra"]["e2e_config5"] = {
         "graph": "R-MAT scale %d ef 16 symmetrised: %d nodes, %d edges; top 20 %% adjacency cached; features %d x %d "
                  "f32 pinned, top-degree 25 %% cached" % (args.e2e_scale, n, indices.numel(), n, D),
@@ -486,6 +543,8 @@ def bench_e2e(capi, args, result):
         "sample_relabel_ms": round(t_s / nbatch, 3), "fetch_ms": round(t_f / nbatch, 3),
         "batch_ms_wall": round(wall * 1e3 / nbatch, 3), "batches_per_s": round(nbatch / wall, 2),
         "fused_hop_batch_ms_wall": round(wall_fused * 1e3 / nbatch, 3),
+        "background_prefetch_batch_ms_wall": round(wall_pipe * 1e3 / nbatch, 3),
+        "sample_blocks_ms_per_batch_by_batches_in_flight": in_flight_ms,
         "sampled_edges_per_s": round(tot_edges / (t_s * 1e-3), 1),
         "fetch_payload_GBs": round(tot_nodes * D * 4 / (t_f * 1e-3) / 1e9, 2)}
 

@@ -4,6 +4,9 @@
 // operator validates its tensors, allocates outputs and scratch from torch's
 // caching allocator and calls the C ABI of libshmt.so (include/shmt.h) on
 // torch's current HIP stream. Failures raise RuntimeError; nothing exits.
+#include <ATen/hip/HIPEvent.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
@@ -11,7 +14,9 @@
 #include <chrono>
 #include <cstdint>
 #include <mutex>
+#include <exception>
 #include <optional>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -73,6 +78,7 @@ class Readback {
   };
 
   Slot acquire() {
+    std::lock_guard<std::mutex> lock(mutex_);
     if (!host_.defined()) {
       host_ = torch::zeros({kSlots}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
       void *d = nullptr;
@@ -103,9 +109,10 @@ class Readback {
   }
 
  private:
-  static constexpr int kSlots = 16;
+  static constexpr int kSlots = 256;  // more than any operator keeps pending at once
   static constexpr int64_t kPending = INT64_MIN;
   static constexpr int kSpinBudgetMs = 200;
+  std::mutex mutex_;  // operators may run on several host threads (sample_blocks)
   torch::Tensor host_;
   int64_t *dev_ = nullptr;
   int next_ = 0;
@@ -485,76 +492,247 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
 // [seeds, sub_indices]. No counterpart as a single operator in the reference.
 // All kernels of the hop are queued without the host learning nnz in between
 // (the relabel kernels read it from sub_indptr[S] on the device); nnz and the
-// number of unique ids are picked up together at the end. Returns
+// number of unique ids are picked up together at the end. The result is
 // (sub_indptr, sub_indices, unique, relabel_indices): exactly what
 // csr_[cache_]sampling followed by tensor_relabel([seeds, sub_indices]) returns,
 // with relabel_indices = the labels of the sub_indices part.
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> sample_hop(
-    torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
-    std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, torch::Tensor seeds,
-    int64_t num_picks, bool replace, std::optional<int64_t> seed, int64_t stream_id) {
-  const bool cached = hashmap != nullptr;
-  TORCH_CHECK(!cached || (gpu_indptr.has_value() && gpu_indices.has_value()),
+using HopResult = std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>;
+
+struct CsrArgs {
+  torch::Tensor indptr, indices;
+  std::optional<torch::Tensor> gpu_indptr, gpu_indices;
+  StaticHashmap *hashmap;
+  bool cached() const { return hashmap != nullptr; }
+};
+
+void check_csr(const CsrArgs &g) {
+  TORCH_CHECK(!g.cached() || (g.gpu_indptr.has_value() && g.gpu_indices.has_value()),
               "sample_hop: a hashmap needs gpu_indptr and gpu_indices");
+  id_bytes(g.indptr, "indptr");
+  id_bytes(g.indices, "indices");
+  TORCH_CHECK(g.indptr.is_contiguous() && g.indices.is_contiguous(), "CSR arrays must be contiguous");
+  if (g.cached()) {
+    TORCH_CHECK(g.gpu_indptr->is_cuda() && g.gpu_indices->is_cuda() && g.gpu_indptr->is_contiguous() &&
+                    g.gpu_indices->is_contiguous(),
+                "gpu_indptr and gpu_indices must be contiguous CUDA tensors");
+    TORCH_CHECK(g.gpu_indptr->scalar_type() == g.indptr.scalar_type() &&
+                    g.gpu_indices->scalar_type() == g.indices.scalar_type(),
+                "cached CSR must have the dtypes of the full CSR");
+  }
+}
+
+// A hop whose kernels are queued on the stream that was current when it was
+// issued and whose two data-dependent sizes have not been read yet.
+struct PendingHop {
+  bool finished = false;
+  HopResult result;                       // valid when finished
+  int64_t S = 0;
+  torch::Tensor sub_indptr, sub_indices, unique, labels;
+  torch::Tensor plan, total, scratch;     // kept until the sizes are in
+  Readback::Slot nnz_slot{}, count_slot{};
+};
+
+PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, bool replace,
+                     std::optional<int64_t> seed, int64_t stream_id) {
+  PendingHop h;
   seeds = cuda_ids(seeds, "seeds");
+  TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0");
   const int64_t S = seeds.numel();
   const bool fused = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
   if (!fused) {  // degenerate or very large bound: the two operators one after the other
-    auto sampled = sample_impl(indptr, indices, cached ? &*gpu_indptr : nullptr,
-                               cached ? &*gpu_indices : nullptr, hashmap, seeds, num_picks, replace,
-                               seed, stream_id);
+    auto sampled = sample_impl(g.indptr, g.indices, g.cached() ? &*g.gpu_indptr : nullptr,
+                               g.cached() ? &*g.gpu_indices : nullptr, g.hashmap, seeds, num_picks,
+                               replace, seed, stream_id);
     auto relabeled = tensor_relabel({seeds, std::get<1>(sampled)});
-    return std::make_tuple(std::get<0>(sampled), std::get<1>(sampled), std::get<0>(relabeled),
-                           std::get<1>(relabeled)[1]);
+    h.result = std::make_tuple(std::get<0>(sampled), std::get<1>(sampled), std::get<0>(relabeled),
+                               std::get<1>(relabeled)[1]);
+    h.finished = true;
+    return h;
   }
-  const int pb = id_bytes(indptr, "indptr"), ib = id_bytes(indices, "indices");
+  const int pb = static_cast<int>(g.indptr.element_size());
+  const int ib = static_cast<int>(g.indices.element_size());
   const int sb = static_cast<int>(seeds.element_size());
-  TORCH_CHECK(indptr.is_contiguous() && indices.is_contiguous(), "CSR arrays must be contiguous");
-  if (cached) {
-    TORCH_CHECK(gpu_indptr->is_cuda() && gpu_indices->is_cuda() && gpu_indptr->is_contiguous() &&
-                    gpu_indices->is_contiguous(),
-                "gpu_indptr and gpu_indices must be contiguous CUDA tensors");
-    TORCH_CHECK(gpu_indptr->scalar_type() == indptr.scalar_type() &&
-                    gpu_indices->scalar_type() == indices.scalar_type(),
-                "cached CSR must have the dtypes of the full CSR");
-  }
   const auto dev = torch::kCUDA;
   void *stream = current_stream();
   const int64_t bound = S * num_picks;
-  torch::Tensor sub_indptr = torch::empty({S + 1}, indptr.options().device(dev));
-  torch::Tensor sub_indices = torch::empty({bound}, indices.options().device(dev));
+  h.S = S;
+  h.sub_indptr = torch::empty({S + 1}, g.indptr.options().device(dev));
+  h.sub_indices = torch::empty({bound}, g.indices.options().device(dev));
   const int64_t plan_bytes = shmt_sample_plan_bytes(S);
-  torch::Tensor plan = device_bytes(plan_bytes);
-  const Readback::Slot nnz_slot = readback().acquire();
-  check(shmt_sample_plan(device_address(indptr, "indptr"), pb, cached ? gpu_indptr->data_ptr() : nullptr,
-                         cached ? hashmap->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks,
-                         replace, sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, nnz_slot.dev,
-                         stream));
-  check(shmt_sample_pick(device_address(indices, "indices"), cached ? gpu_indices->data_ptr() : nullptr,
-                         ib, seeds.data_ptr(), sb, S, num_picks, replace, sub_indptr.data_ptr(), pb,
-                         plan.data_ptr(), sub_indices.data_ptr(),
-                         static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
+  h.plan = device_bytes(plan_bytes);
+  h.nnz_slot = readback().acquire();
+  check(shmt_sample_plan(device_address(g.indptr, "indptr"), pb,
+                         g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
+                         g.cached() ? g.hashmap->handle() : nullptr, seeds.data_ptr(), sb, S,
+                         num_picks, replace, h.sub_indptr.data_ptr(), h.plan.data_ptr(), plan_bytes,
+                         h.nnz_slot.dev, stream));
+  check(shmt_sample_pick(device_address(g.indices, "indices"),
+                         g.cached() ? g.gpu_indices->data_ptr() : nullptr, ib, seeds.data_ptr(), sb, S,
+                         num_picks, replace, h.sub_indptr.data_ptr(), pb, h.plan.data_ptr(),
+                         h.sub_indices.data_ptr(), static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
                          static_cast<uint32_t>(stream_id), stream));
   // relabel [seeds, sub_indices]; the second length is read from sub_indptr[S] by the kernels
   const int eb = std::max(sb, ib);
   const auto id_options = seeds.options().dtype(eb == 8 ? torch::kInt64 : torch::kInt32);
   const int64_t n_max = S + bound;
-  torch::Tensor total = torch::empty({n_max}, id_options);
-  torch::Tensor unique = torch::empty({n_max}, id_options);
-  torch::Tensor labels = torch::empty({n_max}, id_options);
+  h.total = torch::empty({n_max}, id_options);
+  h.unique = torch::empty({n_max}, id_options);
+  h.labels = torch::empty({n_max}, id_options);
   const int64_t scratch_bytes = shmt_relabel_scratch_bytes(n_max);
-  torch::Tensor scratch = device_bytes(scratch_bytes);
-  const void *ptrs[2] = {seeds.data_ptr(), sub_indices.data_ptr()};
+  h.scratch = device_bytes(scratch_bytes);
+  const void *ptrs[2] = {seeds.data_ptr(), h.sub_indices.data_ptr()};
   const int64_t lens[2] = {S, bound};
   const int widths[2] = {sb, ib};
-  const Readback::Slot count_slot = readback().acquire();
-  check(shmt_relabel_segments(ptrs, lens, widths, 2, static_cast<char *>(sub_indptr.data_ptr()) + S * pb,
-                              pb, eb, total.data_ptr(), scratch.data_ptr(), scratch_bytes,
-                              unique.data_ptr(), labels.data_ptr(), count_slot.dev, stream));
-  const int64_t nnz = Readback::wait(nnz_slot);
-  const int64_t U = Readback::wait(count_slot);
-  return std::make_tuple(sub_indptr, sub_indices.narrow(0, 0, nnz), unique.narrow(0, 0, U),
-                         labels.narrow(0, S, nnz));
+  h.count_slot = readback().acquire();
+  check(shmt_relabel_segments(ptrs, lens, widths, 2,
+                              static_cast<char *>(h.sub_indptr.data_ptr()) + S * pb, pb, eb,
+                              h.total.data_ptr(), h.scratch.data_ptr(), scratch_bytes,
+                              h.unique.data_ptr(), h.labels.data_ptr(), h.count_slot.dev, stream));
+  return h;
+}
+
+// Must run with the stream of hop_issue current (the wait falls back to
+// synchronising the current stream).
+HopResult hop_finish(PendingHop &h) {
+  if (!h.finished) {
+    const int64_t nnz = Readback::wait(h.nnz_slot);
+    const int64_t U = Readback::wait(h.count_slot);
+    h.result = std::make_tuple(h.sub_indptr, h.sub_indices.narrow(0, 0, nnz), h.unique.narrow(0, 0, U),
+                               h.labels.narrow(0, h.S, nnz));
+    h.finished = true;
+    // scratch goes back to the allocator of its stream; work queued later on
+    // that stream is ordered after the kernels that still read it
+    h.plan = h.total = h.scratch = torch::Tensor();
+  }
+  return h.result;
+}
+
+HopResult sample_hop(torch::Tensor indptr, torch::Tensor indices,
+                     std::optional<torch::Tensor> gpu_indptr, std::optional<torch::Tensor> gpu_indices,
+                     StaticHashmap *hashmap, torch::Tensor seeds, int64_t num_picks, bool replace,
+                     std::optional<int64_t> seed, int64_t stream_id) {
+  const CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+  check_csr(g);
+  PendingHop h = hop_issue(g, seeds, num_picks, replace, seed, stream_id);
+  return hop_finish(h);
+}
+
+// RAII: make `s` torch's current stream, restore the previous one on exit.
+class CurrentStreamScope {
+ public:
+  explicit CurrentStreamScope(c10::hip::HIPStreamMasqueradingAsCUDA s)
+      : prev_(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA()) {
+    c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(s);
+  }
+  ~CurrentStreamScope() { c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(prev_); }
+  CurrentStreamScope(const CurrentStreamScope &) = delete;
+  CurrentStreamScope &operator=(const CurrentStreamScope &) = delete;
+
+ private:
+  c10::hip::HIPStreamMasqueradingAsCUDA prev_;
+};
+
+constexpr int64_t kMaxBatchesInFlight = 32;
+
+// All hops of one batch on the current stream: hop h samples `num_picks[h]`
+// neighbours of the previous hop's unique ids (RNG stream h when a seed is
+// given), as the dataloader's loop does (python/shmtensor/sampling.py:128-143; `num_picks` is
+// already in call order, i.e. the reversed fanout list).
+std::vector<HopResult> run_hops(const CsrArgs &g, torch::Tensor seeds,
+                                const std::vector<int64_t> &num_picks, bool replace,
+                                std::optional<int64_t> seed) {
+  std::vector<HopResult> hops;
+  hops.reserve(num_picks.size());
+  for (size_t hop = 0; hop < num_picks.size(); ++hop) {
+    // without an RNG seed every call draws from the fixed default seed, stream 0,
+    // as every call of the reference does (src/cache_graph_sampling.cu:204,407)
+    const int64_t rng_stream = seed.has_value() ? static_cast<int64_t>(hop) : 0;
+    PendingHop pending = hop_issue(g, seeds, num_picks[hop], replace, seed, rng_stream);
+    hops.push_back(hop_finish(pending));
+    seeds = std::get<2>(hops.back());
+  }
+  return hops;
+}
+
+// Multi-hop sampling of several independent seed batches. Every batch is a
+// chain of short, latency-bound kernels with two host reads of a size per hop,
+// so one batch alone leaves most of the GPU idle. Here up to `max_in_flight`
+// batches advance at the same time: each is driven by its own host thread on
+// its own stream (default priority, the same streams every call), so both the
+// launches and the kernels of different batches overlap. Results are those of
+// sample_hop called hop by hop, batch by batch (`seeds_rng[b]` is the RNG seed
+// of batch b, RNG stream = hop number; without seeds_rng every hop uses the
+// default seed and stream 0); they are ordered after the calling
+// stream's earlier work and before its later work, and their memory is
+// registered with the calling stream.
+std::vector<std::vector<HopResult>> sample_blocks(
+    torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
+    std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, std::vector<torch::Tensor> seeds,
+    std::vector<int64_t> num_picks, bool replace, std::optional<std::vector<int64_t>> seeds_rng,
+    int64_t max_in_flight) {
+  const CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+  check_csr(g);
+  const int64_t B = static_cast<int64_t>(seeds.size());
+  TORCH_CHECK(!seeds_rng.has_value() || static_cast<int64_t>(seeds_rng->size()) == B,
+              "seeds_rng must have one entry per batch");
+  TORCH_CHECK(max_in_flight >= 1, "max_in_flight must be >= 1");
+  for (const torch::Tensor &t : seeds) cuda_ids(t, "seeds");
+  for (int64_t k : num_picks) TORCH_CHECK(k >= 0, "num_picks must be >= 0");
+  auto rng_of = [&](int64_t b) {
+    return seeds_rng ? std::optional<int64_t>((*seeds_rng)[b]) : std::nullopt;
+  };
+  std::vector<std::vector<HopResult>> out(B);
+  const int64_t K = std::min<int64_t>({max_in_flight, kMaxBatchesInFlight, B});
+  if (K <= 1) {
+    py::gil_scoped_release no_gil;  // lets a Python thread that prefetches batches run beside the caller
+    for (int64_t b = 0; b < B; ++b) out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b));
+    return out;
+  }
+  const auto caller = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  const c10::DeviceIndex device = caller.device_index();
+  at::cuda::CUDAEvent inputs_ready;
+  inputs_ready.record(caller);
+  // the same lanes every call: torch's allocator caches blocks per stream
+  static std::vector<c10::hip::HIPStreamMasqueradingAsCUDA> lane_pool;
+  while (static_cast<int64_t>(lane_pool.size()) < K)
+    lane_pool.push_back(c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, device));
+  const std::vector<c10::hip::HIPStreamMasqueradingAsCUDA> lanes(lane_pool.begin(), lane_pool.begin() + K);
+  for (auto &lane : lanes) inputs_ready.block(lane);
+
+  std::atomic<int64_t> next_batch{0};
+  std::vector<std::exception_ptr> failures(K);
+  {
+    py::gil_scoped_release no_gil;  // the workers touch tensors, never Python objects
+    std::vector<std::thread> workers;
+    workers.reserve(K);
+    for (int64_t j = 0; j < K; ++j) {
+      workers.emplace_back([&, j] {
+        try {
+          c10::hip::set_device(device);
+          CurrentStreamScope scope(lanes[j]);  // torch's current stream is per thread
+          for (int64_t b = next_batch++; b < B; b = next_batch++)
+            out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b));
+        } catch (...) {
+          failures[j] = std::current_exception();
+        }
+      });
+    }
+    for (auto &w : workers) w.join();
+  }
+  // later work of the caller's stream sees the results; their memory must not be
+  // reused by the lanes while the caller's stream may still read it
+  for (auto &lane : lanes) {
+    at::cuda::CUDAEvent done;
+    done.record(lane);
+    done.block(caller);
+  }
+  for (auto &f : failures)
+    if (f) std::rethrow_exception(f);
+  for (auto &hops : out)
+    for (auto &r : hops)
+      for (const torch::Tensor &t : {std::get<0>(r), std::get<1>(r), std::get<2>(r), std::get<3>(r)})
+        if (t.defined() && t.is_cuda() && t.numel() > 0) t.record_stream(caller.unwrap());
+  return out;
 }
 
 }  // namespace
@@ -591,7 +769,10 @@ PYBIND11_MODULE(ShmTensorLib, m) {
       .def("tensor_relabel", &tensor_relabel, py::arg("tensors"))
       .def("sample_hop", &sample_hop, py::arg("indptr"), py::arg("indices"), py::arg("gpu_indptr"),
            py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"),
-           py::arg("replace"), py::arg("seed") = py::none(), py::arg("stream_id") = 0);
+           py::arg("replace"), py::arg("seed") = py::none(), py::arg("stream_id") = 0)
+      .def("sample_blocks", &sample_blocks, py::arg("indptr"), py::arg("indices"), py::arg("gpu_indptr"),
+           py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"),
+           py::arg("replace"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4);
 
   py::class_<StaticHashmap>(m, "CUCOStaticHashmap")
       .def(py::init<torch::Tensor, torch::Tensor, double>())

@@ -3,12 +3,15 @@ ShmTensorLib operators. Same constructor, iteration protocol, cache
 management and return values as python/shmtensor/sampling.py:30-237 in the
 reference; the per-hop work is `csr_sampling` / `csr_cache_sampling` followed
 by `tensor_relabel([seeds, sub_indices])`, issued through the fused
-`sample_hop` operator (same results, one host wait per hop instead of two).
+`sample_blocks` operator (same results; one host wait per hop instead of two,
+and optionally several batches in flight at once).
 
 Without DGL installed a block is a `CSCBlock` tuple (indptr, indices,
 num_src, num_dst); with DGL it is the DGLBlock the reference builds
 (python/shmtensor/sampling.py:9-18)."""
 import collections
+import queue
+import threading
 import weakref
 
 import torch
@@ -46,7 +49,7 @@ def _unpin(tensor):
 class GPUSamplingDataloader:
 
     def __init__(self, indptr, indices, seeds, batchsize, num_picks, replace=False, use_ddp=False,
-                 shuffle=True, drop_last=False, rng_seed=None):
+                 shuffle=True, drop_last=False, rng_seed=None, prefetch=1, background=False):
         self.indptr = indptr
         self.indices = indices
         self.seeds = seeds
@@ -61,6 +64,14 @@ class GPUSamplingDataloader:
         # (rng_seed + b, stream h), so epochs and batches differ reproducibly.
         self.rng_seed = rng_seed
         self._batches_drawn = 0
+        # prefetch > 1: that many consecutive batches are sampled together, their
+        # kernels overlapping on separate streams (same batches, same order, same
+        # results). background=True: a host thread samples ahead on a side stream
+        # while the caller consumes the previous batches (feature fetch, training).
+        self.prefetch = max(1, int(prefetch))
+        self.background = bool(background)
+        self._ready = collections.deque()
+        self._producer = None
 
         self.has_cache = False
         self.gpu_indptr = None
@@ -96,12 +107,24 @@ class GPUSamplingDataloader:
         return self.len
 
     def __iter__(self):
+        self._stop_producer()
+        self._ready.clear()
         if self.shuffle:
             self.seeds = self.seeds[torch.randperm(self.seeds.numel(), device=self.seeds.device)]
         self.curr = 0
         return self
 
+    def _discard_prefetched(self):
+        """Batches sampled ahead belong to the old parameters / cache: drop them."""
+        self._stop_producer()
+        self._ready.clear()
+
+    def close(self):
+        """Stop the background thread (it otherwise ends with the epoch)."""
+        self._discard_prefetched()
+
     def update_params(self, **kwargs):
+        self._discard_prefetched()
         for k, v in kwargs.items():
             setattr(self, k, v)
         if "seeds" in kwargs or "use_ddp" in kwargs:
@@ -121,33 +144,97 @@ class GPUSamplingDataloader:
                                            self.hashmap, seeds, num_pick, self.replace, **extra)
         return capi.csr_sampling(self.indptr, self.indices, seeds, num_pick, self.replace, **extra)
 
-    def _hop(self, seeds, num_pick, hop):
-        """Sampling and relabel of one hop as one operator: all its kernels are
-        queued before the host waits for either data-dependent size."""
-        extra = {}
+    def _sample_group(self, first_batch, count, batches_drawn):
+        """Sample `count` consecutive batches starting at batch `first_batch`; returns one
+        (input_nodes, output_nodes, blocks) per batch."""
+        groups = [self.seeds[b * self.batchsize:(b + 1) * self.batchsize]
+                  for b in range(first_batch, first_batch + count)]
+        rng = None
         if self.rng_seed is not None:
-            extra = {"seed": int(self.rng_seed) + self._batches_drawn, "stream_id": hop}
+            rng = [int(self.rng_seed) + batches_drawn + j for j in range(count)]
         cached = self.has_cache
-        return capi.sample_hop(self.indptr, self.indices, self.gpu_indptr if cached else None,
-                               self.gpu_indices if cached else None, self.hashmap if cached else None,
-                               seeds, num_pick, self.replace, **extra)
+        # the last fanout is applied to the seed layer (sampling.py:128)
+        chains = capi.sample_blocks(self.indptr, self.indices, self.gpu_indptr if cached else None,
+                                    self.gpu_indices if cached else None, self.hashmap if cached else None,
+                                    groups, list(reversed(self.num_picks)), self.replace, seeds_rng=rng,
+                                    max_in_flight=self.prefetch)
+        out = []
+        for seeds, chain in zip(groups, chains):
+            blocks, dst = [], seeds
+            for sub_indptr, _, unique_tensor, relabel_indices in chain:
+                blocks.insert(0, create_block_from_csc(sub_indptr, relabel_indices, torch.Tensor(),
+                                                       unique_tensor.numel(), dst.numel()))
+                dst = unique_tensor
+            out.append((dst, seeds, blocks))
+        return out
+
+    def _produce(self, first_batch, batches_drawn, out_queue, stop):
+        """Body of the background thread: groups of batches, each handed over with the
+        event that marks its results complete on the producer's stream."""
+        try:
+            torch.cuda.set_device(self.seeds.device)
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                b = first_batch
+                while b < self.len and not stop.is_set():
+                    count = min(self.prefetch, self.len - b)
+                    group = self._sample_group(b, count, batches_drawn)
+                    done = torch.cuda.Event()
+                    done.record(side)
+                    out_queue.put((group, done))
+                    b += count
+                    batches_drawn += count
+            out_queue.put(None)
+        except BaseException as exc:       # surfaces in the consumer's __next__
+            out_queue.put(exc)
+
+    def _stop_producer(self):
+        if self._producer is not None:
+            thread, out_queue, stop = self._producer
+            stop.set()
+            while thread.is_alive():
+                try:
+                    out_queue.get(timeout=0.05)
+                except queue.Empty:
+                    pass
+            thread.join()
+            self._producer = None
+
+    def _refill(self):
+        if not self.background:
+            count = min(self.prefetch, self.len - self.curr)
+            self._ready.extend(self._sample_group(self.curr, count, self._batches_drawn))
+            return
+        if self._producer is None:
+            out_queue, stop = queue.Queue(maxsize=2), threading.Event()
+            thread = threading.Thread(target=self._produce, daemon=True,
+                                      args=(self.curr, self._batches_drawn, out_queue, stop))
+            self._producer = (thread, out_queue, stop)
+            thread.start()
+        item = self._producer[1].get()
+        if isinstance(item, BaseException):
+            self._stop_producer()
+            raise item
+        if item is None:
+            raise StopIteration
+        group, done = item
+        current = torch.cuda.current_stream()
+        current.wait_event(done)
+        for dst, _, blocks in group:       # produced on other streams, consumed on this one
+            for t in (dst,) + tuple(x for blk in blocks if isinstance(blk, CSCBlock) for x in blk[:2]):
+                if t.numel() > 0:
+                    t.record_stream(current)
+        self._ready.extend(group)
 
     def __next__(self):
         if self.curr >= self.len:
+            self._stop_producer()
             raise StopIteration
-        seeds = self.seeds[self.curr * self.batchsize:(self.curr + 1) * self.batchsize]
+        if not self._ready:
+            self._refill()
+        input_nodes, output_nodes, blocks = self._ready.popleft()
         self.curr += 1
-
-        output_nodes = seeds
-        blocks = []
-        # the last fanout is applied to the seed layer (sampling.py:128)
-        for hop, num_pick in enumerate(reversed(self.num_picks)):
-            sub_indptr, _, unique_tensor, relabel_indices = self._hop(seeds, num_pick, hop)
-            blocks.insert(0, create_block_from_csc(sub_indptr, relabel_indices, torch.Tensor(),
-                                                   unique_tensor.numel(), seeds.numel()))
-            seeds = unique_tensor
         self._batches_drawn += 1
-        input_nodes = seeds
         return input_nodes, output_nodes, blocks
 
     # ---- cache ---------------------------------------------------------------------
@@ -158,6 +245,7 @@ class GPUSamplingDataloader:
         entry + 10 bytes of hashmap (int32 key and value at load factor 0.8)."""
         if cache_capacity <= 0:
             return
+        self._discard_prefetched()
         full_size = self.indptr.nbytes + self.indices.nbytes
         if full_size <= cache_capacity:      # everything fits: plain GPU sampling
             self.has_cache = False
@@ -182,6 +270,7 @@ class GPUSamplingDataloader:
             print("create cache success")
 
     def clear_cache(self):
+        self._discard_prefetched()
         self.has_cache = False
         self.gpu_indptr = None
         self.gpu_indices = None

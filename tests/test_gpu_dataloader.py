@@ -115,3 +115,47 @@ def test_pin_memory_makes_a_plain_tensor_fetchable(capi):
     assert torch.equal(data[[0, 999, 17]], upd.cpu())               # GPU writes land in the same tensor
     capi.unpin_memory(data)
     capi.pin_memory(torch.zeros(0))                                  # empty tensors are a no-op
+
+
+def _collect(dl):
+    return [(i.clone(), o.clone(), [(b.indptr.clone(), b.indices.clone(), b.num_src, b.num_dst) for b in blocks])
+            for i, o, blocks in dl]
+
+
+def _same_epoch(a, b):
+    assert len(a) == len(b)
+    for (ai, ao, ab), (bi, bo, bb) in zip(a, b):
+        assert torch.equal(ai, bi) and torch.equal(ao, bo) and len(ab) == len(bb)
+        for (p, x, s, d), (q, y, t, e) in zip(ab, bb):
+            assert torch.equal(p, q) and torch.equal(x, y) and (s, d) == (t, e)
+
+
+@pytest.mark.parametrize("rng_seed", [None, 17])
+def test_prefetch_and_background_give_the_same_batches(capi, graph, rng_seed):
+    """Sampling several batches at once, or ahead on a background thread, changes
+    neither the batches nor their order."""
+    base = _collect(_loader(graph, batchsize=100, num_picks=[6, 4, 3], rng_seed=rng_seed))
+    assert len(base) == 10
+    for kw in (dict(prefetch=3), dict(prefetch=4, background=True), dict(prefetch=1, background=True),
+               dict(prefetch=16)):
+        dl = _loader(graph, batchsize=100, num_picks=[6, 4, 3], rng_seed=rng_seed, **kw)
+        _same_epoch(_collect(dl), base)
+        if rng_seed is None:                       # a second epoch over the same loader
+            _same_epoch(_collect(dl), base)
+        assert dl._producer is None
+
+
+def test_background_producer_stops_early_and_reports_errors(capi, graph):
+    dl = _loader(graph, batchsize=50, prefetch=2, background=True)
+    it = iter(dl)
+    first = next(it)
+    dl.close()                                     # mid-epoch: thread ends, prefetched batches dropped
+    assert dl._producer is None and not dl._ready
+    again = next(iter(dl))
+    assert torch.equal(first[0], again[0])
+    dl.close()
+    bad = _loader(graph, batchsize=50, prefetch=2, background=True)
+    bad.num_picks = [-1]                           # rejected by the operator on the producer thread
+    with pytest.raises(RuntimeError):
+        next(iter(bad))
+    assert bad._producer is None

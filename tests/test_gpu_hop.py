@@ -165,3 +165,58 @@ def test_relabel_segments_device_length_clamped_and_rejected(cabi):
     assert labels.tolist() == list(range(10)) + list(range(5, 15))
     assert lib.shmt_relabel_segments(ptrs, lens, widths, 2, too_long.data_ptr(), 3, 8, *args) == -1
     assert b"last_len_bytes" in lib.shmt_last_error()
+
+
+@pytest.mark.parametrize("in_flight", [1, 3, 8])
+def test_sample_blocks_equals_hop_by_hop(capi, in_flight):
+    """Several batches driven concurrently (host threads + side streams): the
+    same results as one sample_hop call per hop and batch."""
+    indptr, indices = _graph(scale=15)
+    indptr_h, indices_h = indptr.cpu().pin_memory(), indices.cpu().pin_memory()
+    n = indptr.numel() - 1
+    hot = torch.randperm(n, generator=torch.Generator().manual_seed(1))[: n // 3].cuda()
+    gp, gi = capi.create_subcsr(indptr_h, indices_h, hot)
+    h = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel()).cuda(), 0.8)
+    g = torch.Generator().manual_seed(9)
+    sizes = [1000, 1, 0, 257, 4000, 33, 1024, 2048, 5, 700, 1500]
+    batches = [torch.randperm(n, generator=g)[:s].cuda() for s in sizes]
+    rng = [100 + b for b in range(len(batches))]
+    picks = [7, 12, 3]
+    for repeat in range(3):              # also exercises reuse of the side streams' cached memory
+        got = capi.sample_blocks(indptr_h, indices_h, gp, gi, h, batches, picks, False, seeds_rng=rng,
+                                 max_in_flight=in_flight)
+        assert len(got) == len(batches)
+        for b, seeds in enumerate(batches):
+            assert len(got[b]) == len(picks)
+            for hop, k in enumerate(picks):
+                want = capi.sample_hop(indptr_h, indices_h, gp, gi, h, seeds, k, False, seed=rng[b], stream_id=hop)
+                _same(got[b][hop], want)
+                seeds = want[2]
+            # results are usable on the calling stream right away
+            assert got[b][-1][2].sum().item() == seeds.sum().item()
+
+
+def test_sample_blocks_arguments(capi):
+    indptr = torch.tensor([0, 3, 3, 4]).cuda()
+    indices = torch.tensor([2, 1, 0, 2]).cuda()
+    assert capi.sample_blocks(indptr, indices, None, None, None, [], [5], False) == []
+    seeds = [torch.tensor([0, 2]).cuda(), torch.tensor([1]).cuda()]
+    a = capi.sample_blocks(indptr, indices, None, None, None, seeds, [5, 2], False)       # default RNG seed
+    for b in range(2):
+        first = capi.sample_hop(indptr, indices, None, None, None, seeds[b], 5, False)
+        _same(a[b][0], first)
+        _same(a[b][1], capi.sample_hop(indptr, indices, None, None, None, first[2], 2, False))
+    assert capi.sample_blocks(indptr, indices, None, None, None, seeds, [], False) == [[], []]
+    with pytest.raises(RuntimeError):
+        capi.sample_blocks(indptr, indices, None, None, None, seeds, [5], False, seeds_rng=[1])
+    with pytest.raises(RuntimeError):
+        capi.sample_blocks(indptr, indices, None, None, None, seeds, [5], False, max_in_flight=0)
+    with pytest.raises(RuntimeError):    # an error raised on a worker thread reaches the caller
+        capi.sample_blocks(indptr.cpu(), indices, None, None, None, seeds, [5], False, max_in_flight=2)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):          # called with a non-default current stream
+        b = capi.sample_blocks(indptr, indices, None, None, None, seeds, [5, 2], False, max_in_flight=2)
+    side.synchronize()
+    for x, y in zip(a, b):
+        for hx, hy in zip(x, y):
+            _same(hx, hy)
