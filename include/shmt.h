@@ -200,6 +200,38 @@ int shmt_sample_pick(const void *indices, const void *cache_indices,
                      int ptr_bytes, const void *plan, void *sub_indices,
                      uint64_t rng_seed, uint32_t rng_stream, void *stream);
 
+/* One hop of mini-batch sampling as one launch sequence: the body of the
+ * dataloader's loop, python/shmtensor/sampling.py:128-143, i.e.
+ * CSRWise[Cache]Sampling (src/cache_graph_sampling.cu:179-220, :382-426)
+ * followed by TensorRelabel({seeds, sub_indices}) (src/tensor_relabel.cu:125-209).
+ * No single operator of the reference corresponds to it. Results are exactly
+ * those of shmt_sample_plan + shmt_sample_pick + shmt_relabel_segments on
+ * {seeds, sub_indices}; the kernels are arranged so that the host need not
+ * learn nnz before the relabel is queued and so that no separate
+ * concatenation, table-fill or offset pass is launched: the plan kernel also
+ * writes the seeds to total_out[0..S), the pick kernel also writes every
+ * sampled id to total_out[S + offset], adds the tile offsets and empties the
+ * relabel table, and the relabel passes read the sampled count from
+ * sub_indptr[S] on the device.
+ * Requires S >= 1, k >= 1 and S * (k + 1) < 2^31. Buffers: sub_indptr S + 1
+ * entries (ptr_bytes); sub_indices S * k entries (idx_bytes; the first nnz are
+ * the result); plan >= shmt_sample_plan_bytes(S); total_out, unique_out,
+ * labels_out S + S * k entries of elem_bytes = max(seed_bytes, idx_bytes);
+ * scratch >= shmt_relabel_scratch_bytes(S + S * k), 16-byte aligned.
+ * *nnz_out and *count_out (int64, device-accessible) receive the number of
+ * sampled ids and of distinct ids; labels_out[S .. S + nnz) are the labels of
+ * the sampled ids, unique_out[0 .. count) the distinct ids, seeds first.    */
+int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices,
+                    int idx_bytes, const void *cache_indptr,
+                    const void *cache_indices, const shmt_hashmap_t *map,
+                    const void *seeds, int seed_bytes, int64_t S, int64_t k,
+                    int replace, uint64_t rng_seed, uint32_t rng_stream,
+                    void *sub_indptr, void *sub_indices, void *plan,
+                    int64_t plan_bytes, int elem_bytes, void *total_out,
+                    void *scratch, int64_t scratch_bytes, void *unique_out,
+                    void *labels_out, int64_t *nnz_out, int64_t *count_out,
+                    void *stream);
+
 /* Cached sub-CSR: CreateCacheCSR, src/cache_graph_sampling.cu:455-492
  * (CSRIndicesCopyKernel :428-453). Step 1 writes
  * cache_indptr[0..C] = exclusive scan of deg(seeds[i]) (width ptr_bytes) and

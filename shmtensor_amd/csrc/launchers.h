@@ -12,4 +12,18 @@ int launch_fill_ones(void *p, int64_t n16, hipStream_t s);
 // In-place exclusive scan of nb 64-bit tile totals by one workgroup.
 int launch_scan_partials(uint64_t *partials, int64_t nb, hipStream_t s);
 
+// Relabel as the tail of a fused launch sequence. relabel_table() names the
+// hash-table part of a relabel scratch buffer sized for N ids (n16 16-byte
+// words that must be all ones when the passes start); launch_relabel_passes()
+// runs insert -> first -> unique -> labels on `total`, which earlier kernels of
+// the same stream have filled, for n_fixed + *n_extra_dev ids (at most n_bound).
+struct RelabelTable {
+  void *slots;
+  int64_t n16;
+};
+int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable *out);
+int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const void *n_extra_dev,
+                          int n_extra_bytes, int elem_bytes, void *scratch, int64_t scratch_bytes,
+                          void *unique_out, void *labels_out, int64_t *count_out, hipStream_t stream);
+
 }  // namespace shmt

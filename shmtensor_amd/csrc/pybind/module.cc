@@ -560,18 +560,6 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   h.sub_indices = torch::empty({bound}, g.indices.options().device(dev));
   const int64_t plan_bytes = shmt_sample_plan_bytes(S);
   h.plan = device_bytes(plan_bytes);
-  h.nnz_slot = readback().acquire();
-  check(shmt_sample_plan(device_address(g.indptr, "indptr"), pb,
-                         g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
-                         g.cached() ? g.hashmap->handle() : nullptr, seeds.data_ptr(), sb, S,
-                         num_picks, replace, h.sub_indptr.data_ptr(), h.plan.data_ptr(), plan_bytes,
-                         h.nnz_slot.dev, stream));
-  check(shmt_sample_pick(device_address(g.indices, "indices"),
-                         g.cached() ? g.gpu_indices->data_ptr() : nullptr, ib, seeds.data_ptr(), sb, S,
-                         num_picks, replace, h.sub_indptr.data_ptr(), pb, h.plan.data_ptr(),
-                         h.sub_indices.data_ptr(), static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
-                         static_cast<uint32_t>(stream_id), stream));
-  // relabel [seeds, sub_indices]; the second length is read from sub_indptr[S] by the kernels
   const int eb = std::max(sb, ib);
   const auto id_options = seeds.options().dtype(eb == 8 ? torch::kInt64 : torch::kInt32);
   const int64_t n_max = S + bound;
@@ -580,14 +568,17 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   h.labels = torch::empty({n_max}, id_options);
   const int64_t scratch_bytes = shmt_relabel_scratch_bytes(n_max);
   h.scratch = device_bytes(scratch_bytes);
-  const void *ptrs[2] = {seeds.data_ptr(), h.sub_indices.data_ptr()};
-  const int64_t lens[2] = {S, bound};
-  const int widths[2] = {sb, ib};
+  h.nnz_slot = readback().acquire();
   h.count_slot = readback().acquire();
-  check(shmt_relabel_segments(ptrs, lens, widths, 2,
-                              static_cast<char *>(h.sub_indptr.data_ptr()) + S * pb, pb, eb,
-                              h.total.data_ptr(), h.scratch.data_ptr(), scratch_bytes,
-                              h.unique.data_ptr(), h.labels.data_ptr(), h.count_slot.dev, stream));
+  check(shmt_sample_hop(device_address(g.indptr, "indptr"), pb, device_address(g.indices, "indices"), ib,
+                        g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
+                        g.cached() ? g.gpu_indices->data_ptr() : nullptr,
+                        g.cached() ? g.hashmap->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks,
+                        replace, static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
+                        static_cast<uint32_t>(stream_id), h.sub_indptr.data_ptr(), h.sub_indices.data_ptr(),
+                        h.plan.data_ptr(), plan_bytes, eb, h.total.data_ptr(), h.scratch.data_ptr(),
+                        scratch_bytes, h.unique.data_ptr(), h.labels.data_ptr(), h.nnz_slot.dev,
+                        h.count_slot.dev, stream));
   return h;
 }
 

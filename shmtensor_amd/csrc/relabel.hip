@@ -312,7 +312,7 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
 // kernels work on the true count.
 static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
                         int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
-                        void *labels_out, int64_t *count_out, void *stream) {
+                        void *labels_out, int64_t *count_out, void *stream, bool prepared = false) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
@@ -340,7 +340,9 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   const uint32_t cap = static_cast<uint32_t>(l.cap);
 
   int rc = SHMT_OK;
-  if (segs) {
+  if (prepared) {
+    // the caller's earlier kernels on this stream emptied the table and wrote `total`
+  } else if (segs) {
     const int64_t span = l.cap > N ? l.cap : N;
     hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(span, 256 * 4)), dim3(256), 0, s,
                        reinterpret_cast<uint4 *>(tbl), l.cap, *segs, const_cast<void *>(total),
@@ -370,6 +372,35 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;
 }
+
+}  // extern "C"
+
+namespace shmt {
+
+int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable *out) {
+  SHMT_REQUIRE(N >= 1 && N < (1ll << 31), "relabel: N must be in [1, 2^31)");
+  const RlLayout l = rl_layout(N);
+  if (scratch == nullptr || scratch_bytes < l.total) {
+    set_error("relabel: scratch too small (%lld < %lld bytes)", static_cast<long long>(scratch_bytes),
+              static_cast<long long>(l.total));
+    return SHMT_ENOMEM;
+  }
+  SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "relabel: scratch must be 16-byte aligned");
+  out->slots = static_cast<char *>(scratch) + l.table_off;
+  out->n16 = l.cap;
+  return SHMT_OK;
+}
+
+int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const void *n_extra_dev,
+                          int n_extra_bytes, int elem_bytes, void *scratch, int64_t scratch_bytes,
+                          void *unique_out, void *labels_out, int64_t *count_out, hipStream_t stream) {
+  return relabel_impl(total, nullptr, n_bound, RlCount{n_fixed, n_extra_dev, n_extra_bytes, n_bound},
+                      elem_bytes, scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true);
+}
+
+}  // namespace shmt
+
+extern "C" {
 
 int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,

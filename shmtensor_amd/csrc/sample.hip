@@ -48,6 +48,8 @@ struct PlanArgs {
   int ptr_bytes;
   int seed_bytes;
   int replace;
+  void *seed_copy;      // optional: seeds widened to seed_copy_bytes (head of a relabel input)
+  int seed_copy_bytes;
 };
 
 // MODE 0: no cache; 1: wide map; 2: narrow map.
@@ -56,6 +58,7 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
   // called by whole waves; lanes past S use a harmless key and produce cnt 0
   const bool live = i < a.S;
   int64_t node = live ? load_int(a.seeds, i, a.seed_bytes) : -1;
+  if (live && a.seed_copy) store_int(a.seed_copy, i, a.seed_copy_bytes, node);
   int64_t slot = -1;
   if (MODE == 1) slot = wave_find<kSlot16>(a.map, map_key(a.map, node));
   if (MODE == 2) slot = wave_find<kSlot8>(a.map, map_key(a.map, node));
@@ -129,6 +132,30 @@ __global__ __launch_bounds__(256) void add_tile_offsets_kernel(void *data, int e
   }
 }
 
+// Fused-hop form of the two kernels above: scans the nb tile totals in place
+// (partials[nb] becomes the grand total) and publishes the total; the tile
+// offsets themselves are added by the pick kernel.
+__global__ __launch_bounds__(1024) void plan_totals_kernel(uint64_t *partials, int64_t nb,
+                                                           void *sub_indptr, int ptr_bytes, int64_t S,
+                                                           int64_t *nnz_out) {
+  __shared__ uint64_t lds[1024 / kWave];
+  uint64_t carry = 0;
+  for (int64_t base = 0; base < nb; base += 1024) {
+    const int64_t i = base + threadIdx.x;
+    const uint64_t v = i < nb ? partials[i] : 0;
+    uint64_t total;
+    const uint64_t ex = block_exclusive_scan<uint64_t, 1024>(v, lds, &total);
+    if (i < nb) partials[i] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) {
+    partials[nb] = carry;
+    store_int(sub_indptr, S, ptr_bytes, static_cast<int64_t>(carry));
+    *nnz_out = static_cast<int64_t>(carry);
+    __threadfence_system();
+  }
+}
+
 // ---- pick ------------------------------------------------------------------
 
 struct PickArgs {
@@ -147,7 +174,43 @@ struct PickArgs {
   int ptr_bytes;
   int replace;
   int log2_group;  // lanes per seed (narrow kernel)
+  // fused hop only (HOP kernels):
+  void *sub_indptr_rw;          // tile-local offsets in, final offsets out
+  const uint64_t *tile_prefix;  // scanned totals of the 1024-seed tiles, or null when offsets are final
+  void *copy_out;               // second copy of every sampled id, widened to copy_bytes ...
+  int64_t copy_base;            // ... at copy_out[copy_base + offset]
+  int copy_bytes;
+  uint4 *clear;                 // clear_n 16-byte words set to all ones (the relabel table)
+  int64_t clear_n;
 };
+
+// Output offset of seed s. In the fused hop the plan left tile-local offsets:
+// the tile's prefix is added here and the final value written back by `writer`.
+template <bool HOP>
+__device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, bool writer) {
+  if (!HOP) return load_int(a.sub_indptr, s, a.ptr_bytes);
+  int64_t optr = load_int(a.sub_indptr_rw, s, a.ptr_bytes);
+  if (a.tile_prefix) {
+    optr += static_cast<int64_t>(a.tile_prefix[s / kPlanBlock]);
+    if (writer) store_int(a.sub_indptr_rw, s, a.ptr_bytes, optr);
+  }
+  return optr;
+}
+
+template <bool HOP>
+__device__ __forceinline__ void pick_store(const PickArgs &a, int64_t pos, int64_t v) {
+  store_int(a.out, pos, a.idx_bytes, v);
+  if (HOP) store_int(a.copy_out, a.copy_base + pos, a.copy_bytes, v);
+}
+
+template <bool HOP>
+__device__ __forceinline__ void pick_clear(const PickArgs &a) {
+  if (!HOP) return;
+  const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.clear_n; i += stride)
+    a.clear[i] = ones;
+}
 
 __device__ __forceinline__ int64_t load_adj(const PickArgs &a, int64_t begin_tagged, int64_t pos) {
   const void *base = (begin_tagged & kCachedTag) ? a.cache_indices : a.indices;
@@ -155,7 +218,9 @@ __device__ __forceinline__ int64_t load_adj(const PickArgs &a, int64_t begin_tag
 }
 
 // k <= 64: group of G = 2^log2_group >= k lanes per seed.
+template <bool HOP>
 __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
+  pick_clear<HOP>(a);
   const int lane = lane_id();
   const int G = 1 << a.log2_group;
   const int gl = lane & (G - 1);
@@ -171,16 +236,16 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
     if (s >= a.S) continue;  // uniform within the group
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
+    const int64_t optr = pick_offset<HOP>(a, s, gl == 0);
     if (deg <= 0) continue;
-    const int64_t optr = load_int(a.sub_indptr, s, a.ptr_bytes);
     if (a.replace) {
       if (gl < k) {
         const int64_t node = load_int(a.seeds, s, a.seed_bytes);
         const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
-        store_int(a.out, optr + gl, a.idx_bytes, load_adj(a, p.begin, static_cast<int64_t>(r)));
+        pick_store<HOP>(a, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
-      if (gl < deg) store_int(a.out, optr + gl, a.idx_bytes, load_adj(a, p.begin, gl));
+      if (gl < deg) pick_store<HOP>(a, optr + gl, load_adj(a, p.begin, gl));
     } else {
       // Floyd: for J = deg-k .. deg-1 draw t in [0, J]; take t unless already
       // taken, then take J. Draws in parallel, resolution in k ballot steps.
@@ -195,7 +260,7 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
         const bool taken = group_ballot_dyn(gl < step && mine == ts, G) != 0;
         if (gl == step) mine = taken ? (deg - k + step) : ts;
       }
-      if (gl < k) store_int(a.out, optr + gl, a.idx_bytes, load_adj(a, p.begin, mine));
+      if (gl < k) pick_store<HOP>(a, optr + gl, load_adj(a, p.begin, mine));
     }
   }
 }
@@ -204,26 +269,26 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
 // are staged in LDS when k fits (IN_LDS), otherwise in the seed's own output
 // segment, which is overwritten by the gathered neighbours at the end
 // (positions are < deg and therefore fit the index width).
-template <bool IN_LDS>
+template <bool IN_LDS, bool HOP>
 __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
   extern __shared__ int64_t chosen_lds[];
+  pick_clear<HOP>(a);
   const int lane = threadIdx.x;
   const int64_t k = a.k;
   for (int64_t s = blockIdx.x; s < a.S; s += gridDim.x) {
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
+    const int64_t optr = pick_offset<HOP>(a, s, lane == 0);
     if (deg <= 0) continue;
-    const int64_t optr = load_int(a.sub_indptr, s, a.ptr_bytes);
     const int64_t node = load_int(a.seeds, s, a.seed_bytes);
     if (a.replace) {
       for (int64_t j = lane; j < k; j += kWave) {
         const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(j),
                                        static_cast<uint64_t>(deg));
-        store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, static_cast<int64_t>(r)));
+        pick_store<HOP>(a, optr + j, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
-      for (int64_t j = lane; j < deg; j += kWave)
-        store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, j));
+      for (int64_t j = lane; j < deg; j += kWave) pick_store<HOP>(a, optr + j, load_adj(a, p.begin, j));
     } else {
       for (int64_t step = 0; step < k; ++step) {
         const int64_t J = deg - k + step;
@@ -248,7 +313,7 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
         int64_t c = 0;
         if (j < k) c = IN_LDS ? chosen_lds[j] : load_int(a.out, optr + j, a.idx_bytes);
         __syncthreads();
-        if (j < k) store_int(a.out, optr + j, a.idx_bytes, load_adj(a, p.begin, c));
+        if (j < k) pick_store<HOP>(a, optr + j, load_adj(a, p.begin, c));
       }
       __syncthreads();
     }
@@ -335,10 +400,20 @@ int64_t shmt_sample_plan_bytes(int64_t S) {
   return S * static_cast<int64_t>(sizeof(SeedPlan)) + (nb + 2) * 8;
 }
 
-int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr,
+// hop != null: fused-hop form. The seeds are also written, widened, to
+// hop->seed_copy, and beyond one tile the offsets stay tile-local: only the
+// scanned tile totals and the grand total are produced (*tile_prefix_out), the
+// pick kernel adds them.
+struct PlanHopExtras {
+  void *seed_copy;
+  int seed_copy_bytes;
+  const uint64_t *tile_prefix_out;
+};
+
+static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr,
                      const shmt_hashmap_t *map, const void *seeds, int seed_bytes, int64_t S,
                      int64_t k, int replace, void *sub_indptr, void *plan, int64_t plan_bytes,
-                     int64_t *nnz_out, void *stream) {
+                     int64_t *nnz_out, void *stream, PlanHopExtras *hop) {
   SHMT_REQUIRE(S >= 0, "shmt_sample_plan: S must be >= 0");
   SHMT_REQUIRE(k >= 0, "shmt_sample_plan: num_picks must be >= 0");
   SHMT_REQUIRE(width_ok(ptr_bytes) && width_ok(seed_bytes),
@@ -372,6 +447,9 @@ int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr
   a.ptr_bytes = ptr_bytes;
   a.seed_bytes = seed_bytes;
   a.replace = replace ? 1 : 0;
+  a.seed_copy = hop ? hop->seed_copy : nullptr;
+  a.seed_copy_bytes = hop ? hop->seed_copy_bytes : 8;
+  if (hop) hop->tile_prefix_out = nullptr;
   const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
 
   if (S <= kPlanSingleMax) {
@@ -392,6 +470,13 @@ int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr
     default: hipLaunchKernelGGL(plan_tile_kernel<2>, grid, dim3(kPlanBlock), 0, s, a); break;
   }
   SHMT_LAUNCH_CHECK();
+  if (hop) {
+    hipLaunchKernelGGL(plan_totals_kernel, dim3(1), dim3(1024), 0, s, a.partials, nb, sub_indptr,
+                       ptr_bytes, S, nnz_out);
+    SHMT_LAUNCH_CHECK();
+    hop->tile_prefix_out = a.partials;
+    return SHMT_OK;
+  }
   int rc = launch_scan_partials(a.partials, nb + 1, s);
   if (rc) return rc;
   hipLaunchKernelGGL(add_tile_offsets_kernel, dim3(grid_for(S + 1, 256)), dim3(256), 0, s,
@@ -401,10 +486,55 @@ int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr
   return SHMT_OK;
 }
 
-int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_bytes,
+int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr,
+                     const shmt_hashmap_t *map, const void *seeds, int seed_bytes, int64_t S,
+                     int64_t k, int replace, void *sub_indptr, void *plan, int64_t plan_bytes,
+                     int64_t *nnz_out, void *stream) {
+  return plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr,
+                   plan, plan_bytes, nnz_out, stream, nullptr);
+}
+
+}  // extern "C"
+
+struct PickHopExtras {
+  void *sub_indptr_rw;
+  const uint64_t *tile_prefix;
+  void *copy_out;
+  int64_t copy_base;
+  int copy_bytes;
+  uint4 *clear;
+  int64_t clear_n;
+};
+
+template <bool HOP>
+static int pick_launch(const PickArgs &a, hipStream_t s) {
+  const int64_t S = a.S, k = a.k;
+  if (k <= kWave) {
+    const int seeds_per_block = 4 * (kWave >> a.log2_group);
+    // the fused form also clears the relabel table: enough threads for that even when S is small
+    int64_t blocks = (S + seeds_per_block - 1) / seeds_per_block;
+    if (HOP) {
+      const int64_t for_clear = (a.clear_n + 256 * 4 - 1) / (256 * 4);
+      if (blocks < for_clear) blocks = for_clear;
+    }
+    hipLaunchKernelGGL(pick_narrow_kernel<HOP>, dim3(grid_for(blocks, 1)), dim3(256), 0, s, a);
+  } else if (k <= kWideMaxPicks) {
+    hipLaunchKernelGGL((pick_wide_kernel<true, HOP>), dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
+                       static_cast<size_t>(k) * sizeof(int64_t), s, a);
+  } else {
+    hipLaunchKernelGGL((pick_wide_kernel<false, HOP>), dim3(grid_for(S, 1, 256 * 32)), dim3(kWave), 0,
+                       s, a);
+  }
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+extern "C" {
+
+static int pick_impl(const void *indices, const void *cache_indices, int idx_bytes,
                      const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
                      const void *sub_indptr, int ptr_bytes, const void *plan, void *sub_indices,
-                     uint64_t rng_seed, uint32_t rng_stream, void *stream) {
+                     uint64_t rng_seed, uint32_t rng_stream, void *stream, const PickHopExtras *hop) {
   SHMT_REQUIRE(S >= 0 && k >= 0, "shmt_sample_pick: S and num_picks must be >= 0");
   SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes),
                "shmt_sample_pick: ID can only be int32 or int64");
@@ -427,21 +557,71 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
   a.ptr_bytes = ptr_bytes;
   a.replace = replace ? 1 : 0;
   a.log2_group = 0;
-  hipStream_t s = as_stream(stream);
   if (k <= kWave) {
     int lg = 2;
     while ((1 << lg) < k) ++lg;
     a.log2_group = lg;
-    const int seeds_per_block = 4 * (kWave >> lg);
-    hipLaunchKernelGGL(pick_narrow_kernel, dim3(grid_for(S, seeds_per_block)), dim3(256), 0, s, a);
-  } else if (k <= kWideMaxPicks) {
-    hipLaunchKernelGGL(pick_wide_kernel<true>, dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
-                       static_cast<size_t>(k) * sizeof(int64_t), s, a);
-  } else {
-    hipLaunchKernelGGL(pick_wide_kernel<false>, dim3(grid_for(S, 1, 256 * 32)), dim3(kWave), 0, s, a);
   }
-  SHMT_LAUNCH_CHECK();
-  return SHMT_OK;
+  a.sub_indptr_rw = nullptr;
+  a.tile_prefix = nullptr;
+  a.copy_out = nullptr;
+  a.copy_base = 0;
+  a.copy_bytes = 8;
+  a.clear = nullptr;
+  a.clear_n = 0;
+  hipStream_t s = as_stream(stream);
+  if (!hop) return pick_launch<false>(a, s);
+  a.sub_indptr_rw = hop->sub_indptr_rw;
+  a.tile_prefix = hop->tile_prefix;
+  a.copy_out = hop->copy_out;
+  a.copy_base = hop->copy_base;
+  a.copy_bytes = hop->copy_bytes;
+  a.clear = hop->clear;
+  a.clear_n = hop->clear_n;
+  return pick_launch<true>(a, s);
+}
+
+int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_bytes,
+                     const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
+                     const void *sub_indptr, int ptr_bytes, const void *plan, void *sub_indices,
+                     uint64_t rng_seed, uint32_t rng_stream, void *stream) {
+  return pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr,
+                   ptr_bytes, plan, sub_indices, rng_seed, rng_stream, stream, nullptr);
+}
+
+int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
+                    const void *cache_indptr, const void *cache_indices, const shmt_hashmap_t *map,
+                    const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
+                    uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr, void *sub_indices,
+                    void *plan, int64_t plan_bytes, int elem_bytes, void *total_out, void *scratch,
+                    int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *nnz_out,
+                    int64_t *count_out, void *stream) {
+  SHMT_REQUIRE(S >= 1 && k >= 1, "shmt_sample_hop: S and num_picks must be >= 1");
+  SHMT_REQUIRE(k <= ((1ll << 31) - 1 - S) / S, "shmt_sample_hop: S * (num_picks + 1) must be < 2^31");
+  SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes) && width_ok(elem_bytes),
+               "shmt_sample_hop: ID can only be int32 or int64");
+  SHMT_REQUIRE(elem_bytes >= seed_bytes && elem_bytes >= idx_bytes,
+               "shmt_sample_hop: elem_bytes must be the wider of the seed and index widths");
+  SHMT_REQUIRE(indices && sub_indices && total_out && unique_out && labels_out && count_out,
+               "shmt_sample_hop: null buffer");
+  const int64_t n_max = S + S * k;
+  RelabelTable table;
+  int rc = relabel_table(n_max, scratch, scratch_bytes, &table);
+  if (rc) return rc;
+  PlanHopExtras plan_hop{total_out, elem_bytes, nullptr};
+  rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
+                 plan_bytes, nnz_out, stream, &plan_hop);
+  if (rc) return rc;
+  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, total_out, S, elem_bytes,
+                               static_cast<uint4 *>(table.slots), table.n16};
+  rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
+                 plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
+  if (rc) return rc;
+  // [seeds, sub_indices] is in total_out and the table is empty: the relabel passes follow, with the
+  // number of sampled ids read from sub_indptr[S]
+  return launch_relabel_passes(total_out, n_max, S, static_cast<const char *>(sub_indptr) + S * ptr_bytes,
+                               ptr_bytes, elem_bytes, scratch, scratch_bytes, unique_out, labels_out,
+                               count_out, as_stream(stream));
 }
 
 int shmt_subcsr_plan(const void *indptr, int ptr_bytes, const void *seeds, int seed_bytes,
