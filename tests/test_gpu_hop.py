@@ -220,3 +220,65 @@ def test_sample_blocks_arguments(capi):
     for x, y in zip(a, b):
         for hx, hy in zip(x, y):
             _same(hx, hy)
+
+
+def test_hop_very_wide_fanout_and_hub(capi):
+    """k beyond the LDS staging limit on a hub row (positions staged in the output segment)."""
+    deg = 20000
+    indptr = torch.tensor([0, deg, deg + 3, deg + 3]).cuda()
+    indices = torch.cat([torch.arange(3, deg + 3), torch.tensor([0, 1, 2])]).cuda()
+    seeds = torch.tensor([1, 0, 2, 0]).cuda()
+    for k in (9000, 65):
+        for replace in (False, True):
+            got = capi.sample_hop(indptr, indices, None, None, None, seeds, k, replace, seed=3)
+            _same(got, _two_step(capi, indptr, indices, None, seeds, k, replace, seed=3))
+            if not replace:
+                hub = got[1][got[0][1]:got[0][2]]
+                assert hub.numel() == k and hub.unique().numel() == k
+
+
+def test_sample_hop_c_abi_matches_separate_entry_points(cabi):
+    """shmt_sample_hop against shmt_sample_plan + shmt_sample_pick + shmt_relabel_segments, raw pointers."""
+    lib = cabi.load()
+    indptr, indices = _graph(scale=13, ptr_dt=torch.int64, idx_dt=torch.int32)
+    indptr, indices = indptr.cuda(), indices.cuda()
+    n = indptr.numel() - 1
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+    stream = cabi.current_stream()
+    for S, k in ((300, 6), (3000, 20), (50, 70)):
+        seeds = torch.randperm(n, generator=torch.Generator().manual_seed(S))[:S].cuda()      # int64
+        n_max = S + S * k
+
+        def buffers():
+            return dict(sp=torch.empty(S + 1, dtype=torch.int64).cuda(), si=torch.empty(S * k, dtype=torch.int32).cuda(),
+                        plan=torch.empty(lib.shmt_sample_plan_bytes(S), dtype=torch.uint8).cuda(),
+                        total=torch.empty(n_max, dtype=torch.int64).cuda(), unique=torch.empty(n_max, dtype=torch.int64).cuda(),
+                        labels=torch.empty(n_max, dtype=torch.int64).cuda(),
+                        scratch=torch.empty(lib.shmt_relabel_scratch_bytes(n_max), dtype=torch.uint8).cuda(),
+                        nnz=torch.zeros(1, dtype=torch.int64).cuda(), count=torch.zeros(1, dtype=torch.int64).cuda())
+        a, b = buffers(), buffers()
+        cabi.check(lib.shmt_sample_hop(indptr.data_ptr(), 8, indices.data_ptr(), 4, None, None, None, seeds.data_ptr(), 8,
+                                       S, k, 0, 42, 1, a["sp"].data_ptr(), a["si"].data_ptr(), a["plan"].data_ptr(),
+                                       a["plan"].numel(), 8, a["total"].data_ptr(), a["scratch"].data_ptr(),
+                                       a["scratch"].numel(), a["unique"].data_ptr(), a["labels"].data_ptr(),
+                                       a["nnz"].data_ptr(), a["count"].data_ptr(), stream))
+        cabi.check(lib.shmt_sample_plan(indptr.data_ptr(), 8, None, None, seeds.data_ptr(), 8, S, k, 0, b["sp"].data_ptr(),
+                                        b["plan"].data_ptr(), b["plan"].numel(), b["nnz"].data_ptr(), stream))
+        cabi.check(lib.shmt_sample_pick(indices.data_ptr(), None, 4, seeds.data_ptr(), 8, S, k, 0, b["sp"].data_ptr(), 8,
+                                        b["plan"].data_ptr(), b["si"].data_ptr(), 42, 1, stream))
+        torch.cuda.synchronize()
+        nnz = int(b["nnz"].item())
+        ptrs = (vp * 2)(seeds.data_ptr(), b["si"].data_ptr())
+        cabi.check(lib.shmt_relabel_segments(ptrs, (i64 * 2)(S, nnz), (ctypes.c_int * 2)(8, 4), 2, None, 0, 8,
+                                             b["total"].data_ptr(), b["scratch"].data_ptr(), b["scratch"].numel(),
+                                             b["unique"].data_ptr(), b["labels"].data_ptr(), b["count"].data_ptr(), stream))
+        torch.cuda.synchronize()
+        assert int(a["nnz"].item()) == nnz and int(a["count"].item()) == int(b["count"].item())
+        u = int(b["count"].item())
+        assert torch.equal(a["sp"], b["sp"]) and torch.equal(a["si"][:nnz], b["si"][:nnz])
+        assert torch.equal(a["total"][:S + nnz], b["total"][:S + nnz])
+        assert torch.equal(a["unique"][:u], b["unique"][:u]) and torch.equal(a["labels"][:S + nnz], b["labels"][:S + nnz])
+    # argument checks
+    assert lib.shmt_sample_hop(indptr.data_ptr(), 8, indices.data_ptr(), 4, None, None, None, seeds.data_ptr(), 8, 0, 5, 0,
+                               1, 0, None, None, None, 0, 8, None, None, 0, None, None, None, None, stream) == -1
+    assert b"must be >= 1" in lib.shmt_last_error()
