@@ -118,6 +118,18 @@ int shmt_set(void *miss_data, void *cache_data, const void *indices,
              int mask_bytes, const void *update, int64_t Q, int64_t row_bytes,
              void *stream);
 
+/* Write-through form of shmt_set. The reference has no such mode (its
+ * CacheTensorSet leaves the host row stale on a hit,
+ * src/cache_feature_set.cu:108-114): here a row that hits is written to
+ * cache_data[slot_i,:] AND to miss_data[indices[i],:], a row that misses to
+ * miss_data[indices[i],:] only, so the id-addressed table stays current and
+ * the cache can be dropped or rebuilt without a write-back. Same arguments
+ * and checks as shmt_set; with neither map nor mask it is shmt_set.          */
+int shmt_set_through(void *miss_data, void *cache_data, const void *indices,
+                     int idx_bytes, const shmt_hashmap_t *map, const void *mask,
+                     int mask_bytes, const void *update, int64_t Q,
+                     int64_t row_bytes, void *stream);
+
 /* ------------------------------------------------------------------ */
 /* Scan. shmt_exclusive_scan: cub_exclusiveSum, src/tensor_relabel.cu:11-26
  * and src/cache_graph_sampling.cu:30-45 — in-place exclusive prefix sum over

@@ -28,6 +28,7 @@ SIGNATURES = {
     "shmt_hashmap_destroy": (None, [_vp]),
     "shmt_fetch": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
     "shmt_set": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
+    "shmt_set_through": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
     "shmt_scan_tmp_bytes": (_i64, [_i64]),
     "shmt_exclusive_scan": (_int, [_vp, _i64, _int, _vp, _i64, _vp]),
     "shmt_inclusive_scan_i32": (_int, [_vp, _i64, _vp, _i64, _vp]),

@@ -54,8 +54,11 @@ constexpr int kRowsWavesPerSimd = 8;  // register budget: 512 / 8 = 64 VGPRs
 constexpr int kRowsInFlight = 2;   // rows a lane group moves concurrently (single-vector rows)
 constexpr int kFindBatch = 4;      // probes per group in flight during phase 1
 
-template <typename VT, int MODE, bool SET, bool ONE_VEC>
+// THROUGH (set only, with a map or mask): rows that hit the cache are written
+// to the id-addressed table as well, so that table never goes stale.
+template <typename VT, int MODE, bool SET, bool ONE_VEC, bool THROUGH = false>
 __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWavesPerSimd / 2) void rows_kernel(RowArgs a) {
+  static_assert(!THROUGH || (SET && MODE != kDirect), "write-through is a cached set");
   const int lane = lane_id();
   const int L = 1 << a.log2_lanes;
   const int gl = lane & (L - 1);
@@ -84,6 +87,9 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
     }
     const int64_t my_table_row =
         reinterpret_cast<int64_t>(slot >= 0 ? a.cache + slot * R : a.miss + idx * R);
+    // write-through: second destination of a row that hit (0: none)
+    const int64_t my_second_row =
+        THROUGH && slot >= 0 ? reinterpret_cast<int64_t>(a.miss + idx * R) : 0;
     const int nrows = static_cast<int>(a.Q - base < tile ? a.Q - base : tile);
 
     // ---- phase 2: move the rows ----
@@ -93,12 +99,17 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
       for (int r0 = 0; r0 < nrows; r0 += kRowsInFlight * rows_per_step) {
         VT v[kRowsInFlight];
         char *trow[kRowsInFlight];
+        char *second[kRowsInFlight];
         // shuffles run with every lane active: a lane can only read the row
         // address held by a lane that takes part in the same instruction
 #pragma unroll
-        for (int u = 0; u < kRowsInFlight; ++u)
+        for (int u = 0; u < kRowsInFlight; ++u) {
           trow[u] = reinterpret_cast<char *>(
               shfl64(my_table_row, (r0 + u * rows_per_step + grp) & (kWave - 1)));
+          second[u] = THROUGH ? reinterpret_cast<char *>(shfl64(
+                                    my_second_row, (r0 + u * rows_per_step + grp) & (kWave - 1)))
+                              : nullptr;
+        }
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int row = r0 + u * rows_per_step + grp;
@@ -114,9 +125,10 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int row = r0 + u * rows_per_step + grp;
           if (row < nrows && in) {
-            if (SET)
+            if (SET) {
               *reinterpret_cast<VT *>(trow[u] + my_off) = v[u];
-            else
+              if (THROUGH && second[u]) *reinterpret_cast<VT *>(second[u] + my_off) = v[u];
+            } else
               __builtin_nontemporal_store(
                   v[u], reinterpret_cast<VT *>(a.dense + (base + row) * R + my_off));
           }
@@ -126,6 +138,8 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
       for (int r0 = 0; r0 < nrows; r0 += rows_per_step) {
         const int row = r0 + grp;
         char *trow = reinterpret_cast<char *>(shfl64(my_table_row, row & (kWave - 1)));
+        char *second =
+            THROUGH ? reinterpret_cast<char *>(shfl64(my_second_row, row & (kWave - 1))) : nullptr;
         if (row >= nrows) continue;
         char *drow = a.dense + (base + row) * R;
         const char *src = SET ? drow : trow;
@@ -143,6 +157,10 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
         }
         for (; off < R; off += step)
           *reinterpret_cast<VT *>(dst + off) = *reinterpret_cast<const VT *>(src + off);
+        if (THROUGH && second) {
+          for (off = my_off; off < R; off += step)
+            *reinterpret_cast<VT *>(second + off) = *reinterpret_cast<const VT *>(src + off);
+        }
       }
     }
   }
@@ -155,6 +173,21 @@ static int pick_vector_bytes(int64_t row_bytes, const void *p0, const void *p1, 
   int v = 16;
   while (v > 1 && (bits & (v - 1))) v >>= 1;
   return v;
+}
+
+template <typename VT, bool ONE_VEC>
+static void launch_through(int mode, unsigned grid, hipStream_t s, const RowArgs &a) {
+  switch (mode) {
+    case kMap16:
+      hipLaunchKernelGGL((rows_kernel<VT, kMap16, true, ONE_VEC, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+    case kMap8:
+      hipLaunchKernelGGL((rows_kernel<VT, kMap8, true, ONE_VEC, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+    default:
+      hipLaunchKernelGGL((rows_kernel<VT, kMask, true, ONE_VEC, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+  }
 }
 
 template <typename VT, bool SET, bool ONE_VEC>
@@ -176,7 +209,15 @@ static void launch_mode(int mode, unsigned grid, hipStream_t s, const RowArgs &a
 }
 
 template <typename VT, bool SET>
-static void launch_vec(bool one_vec, int mode, unsigned grid, hipStream_t s, const RowArgs &a) {
+static void launch_vec(bool one_vec, bool through, int mode, unsigned grid, hipStream_t s,
+                       const RowArgs &a) {
+  if (SET && through && mode != kDirect) {
+    if (one_vec)
+      launch_through<VT, true>(mode, grid, s, a);
+    else
+      launch_through<VT, false>(mode, grid, s, a);
+    return;
+  }
   if (one_vec)
     launch_mode<VT, SET, true>(mode, grid, s, a);
   else
@@ -186,7 +227,7 @@ static void launch_vec(bool one_vec, int mode, unsigned grid, hipStream_t s, con
 template <bool SET>
 static int move_rows(const char *who, void *miss, void *cache, const void *indices, int idx_bytes,
                      const shmt_hashmap_t *map, const void *mask, int mask_bytes, void *dense,
-                     int64_t Q, int64_t row_bytes, void *stream) {
+                     int64_t Q, int64_t row_bytes, void *stream, bool through = false) {
   SHMT_REQUIRE(Q >= 0, "%s: Q must be >= 0", who);
   SHMT_REQUIRE(row_bytes > 0, "%s: row_bytes must be > 0", who);
   SHMT_REQUIRE(width_ok(idx_bytes), "%s: ID can only be int32 or int64 (idx_bytes=%d)", who, idx_bytes);
@@ -231,11 +272,11 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   hipStream_t s = as_stream(stream);
   const bool one_vec = nvec <= (1ll << log2_lanes);
   switch (vb) {
-    case 16: launch_vec<u32x4, SET>(one_vec, mode, grid, s, a); break;
-    case 8: launch_vec<u32x2, SET>(one_vec, mode, grid, s, a); break;
-    case 4: launch_vec<uint32_t, SET>(one_vec, mode, grid, s, a); break;
-    case 2: launch_vec<uint16_t, SET>(one_vec, mode, grid, s, a); break;
-    default: launch_vec<uint8_t, SET>(one_vec, mode, grid, s, a); break;
+    case 16: launch_vec<u32x4, SET>(one_vec, through, mode, grid, s, a); break;
+    case 8: launch_vec<u32x2, SET>(one_vec, through, mode, grid, s, a); break;
+    case 4: launch_vec<uint32_t, SET>(one_vec, through, mode, grid, s, a); break;
+    case 2: launch_vec<uint16_t, SET>(one_vec, through, mode, grid, s, a); break;
+    default: launch_vec<uint8_t, SET>(one_vec, through, mode, grid, s, a); break;
   }
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;
@@ -258,6 +299,13 @@ int shmt_set(void *miss_data, void *cache_data, const void *indices, int idx_byt
              int64_t Q, int64_t row_bytes, void *stream) {
   return shmt::move_rows<true>("shmt_set", miss_data, cache_data, indices, idx_bytes, map, mask,
                                mask_bytes, const_cast<void *>(update), Q, row_bytes, stream);
+}
+
+int shmt_set_through(void *miss_data, void *cache_data, const void *indices, int idx_bytes,
+                     const shmt_hashmap_t *map, const void *mask, int mask_bytes, const void *update,
+                     int64_t Q, int64_t row_bytes, void *stream) {
+  return shmt::move_rows<true>("shmt_set_through", miss_data, cache_data, indices, idx_bytes, map, mask,
+                               mask_bytes, const_cast<void *>(update), Q, row_bytes, stream, true);
 }
 
 }  // extern "C"

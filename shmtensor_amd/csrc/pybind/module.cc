@@ -272,7 +272,8 @@ torch::Tensor fetch_impl(const torch::Tensor &uva_data, const torch::Tensor *gpu
 }
 
 void set_impl(torch::Tensor &uva_data, torch::Tensor *gpu_data, torch::Tensor indices,
-              torch::Tensor update, const StaticHashmap *map, const torch::Tensor *mask) {
+              torch::Tensor update, const StaticHashmap *map, const torch::Tensor *mask,
+              bool write_through = false) {
   check_tables(uva_data, gpu_data);
   indices = cuda_ids(indices, "indices");
   const int64_t numel = indices.numel();
@@ -291,11 +292,11 @@ void set_impl(torch::Tensor &uva_data, torch::Tensor *gpu_data, torch::Tensor in
   if (numel == 0 || rs.row_bytes == 0) return;
   void *cache_ptr = nullptr;
   if (gpu_data) cache_ptr = gpu_data->numel() > 0 ? gpu_data->data_ptr() : update.data_ptr();
-  check(shmt_set(device_address(uva_data, "uva_data"), cache_ptr,
-                 indices.data_ptr(), static_cast<int>(indices.element_size()),
-                 map ? map->handle() : nullptr, mask ? m.data_ptr() : nullptr,
-                 mask ? static_cast<int>(m.element_size()) : 0, update.data_ptr(), numel,
-                 rs.row_bytes, current_stream()));
+  const auto entry = write_through ? shmt_set_through : shmt_set;
+  check(entry(device_address(uva_data, "uva_data"), cache_ptr, indices.data_ptr(),
+              static_cast<int>(indices.element_size()), map ? map->handle() : nullptr,
+              mask ? m.data_ptr() : nullptr, mask ? static_cast<int>(m.element_size()) : 0,
+              update.data_ptr(), numel, rs.row_bytes, current_stream()));
 }
 
 torch::Tensor uva_fetch(torch::Tensor &data, torch::Tensor &indices) {
@@ -313,12 +314,12 @@ void uva_set(torch::Tensor &data, torch::Tensor &indices, torch::Tensor &update)
   set_impl(data, nullptr, indices, update, nullptr, nullptr);
 }
 void cache_set(torch::Tensor uva_data, torch::Tensor gpu_data, torch::Tensor indices,
-               torch::Tensor update, StaticHashmap &hashmap) {
-  set_impl(uva_data, &gpu_data, indices, update, &hashmap, nullptr);
+               torch::Tensor update, StaticHashmap &hashmap, bool write_through) {
+  set_impl(uva_data, &gpu_data, indices, update, &hashmap, nullptr, write_through);
 }
 void cache_set_with_mask(torch::Tensor uva_data, torch::Tensor gpu_data, torch::Tensor indices,
-                         torch::Tensor update, torch::Tensor mask) {
-  set_impl(uva_data, &gpu_data, indices, update, nullptr, &mask);
+                         torch::Tensor update, torch::Tensor mask, bool write_through) {
+  set_impl(uva_data, &gpu_data, indices, update, nullptr, &mask, write_through);
 }
 
 // ---- scan --------------------------------------------------------------------
@@ -745,9 +746,9 @@ PYBIND11_MODULE(ShmTensorLib, m) {
            py::arg("gpu_data"), py::arg("indices"), py::arg("mask"))
       .def("uva_set", &uva_set, py::arg("data"), py::arg("indices"), py::arg("update"))
       .def("cache_set", &cache_set, py::arg("uva_data"), py::arg("gpu_data"), py::arg("indices"),
-           py::arg("update"), py::arg("hashmap"))
+           py::arg("update"), py::arg("hashmap"), py::arg("write_through") = false)
       .def("cache_set_with_mask", &cache_set_with_mask, py::arg("uva_data"), py::arg("gpu_data"),
-           py::arg("indices"), py::arg("update"), py::arg("mask"))
+           py::arg("indices"), py::arg("update"), py::arg("mask"), py::arg("write_through") = false)
       .def("csr_sampling", &csr_sampling, py::arg("indptr"), py::arg("indices"), py::arg("seeds"),
            py::arg("num_picks"), py::arg("replace"), py::arg("seed") = py::none(),
            py::arg("stream_id") = 0)

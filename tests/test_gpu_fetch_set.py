@@ -125,6 +125,41 @@ def test_set_final_state_matches_oracle(capi, oracle):
     assert np.array_equal(gpu_t.cpu().numpy(), gpu)
 
 
+@pytest.mark.parametrize("D,dtype", [(24, np.float32), (64, np.float16), (5, np.int8), (300, np.float32), (3, np.int16)])
+@pytest.mark.parametrize("route", ["map64", "map32", "mask"])
+def test_write_through_set_keeps_the_host_table_current(capi, D, dtype, route):
+    """write_through=True (no counterpart in the reference): hits update the cache row and
+    the host row, misses the host row; closed form on both tables."""
+    rng = np.random.default_rng(D)
+    n, c = 5000, 1800
+    host = (rng.standard_normal((n, D)) * 50).astype(dtype)
+    ids = rng.choice(n, size=c, replace=False)
+    gpu = (host[ids] + 1).astype(dtype)                      # stale-looking cache rows: routing is observable
+    q = np.unique(rng.integers(0, n, size=3000))
+    upd = (rng.standard_normal((q.size, D)) * 50).astype(dtype)
+    data_t = torch.from_numpy(host.copy()).pin_memory()
+    gpu_t = torch.from_numpy(gpu.copy()).cuda()
+    it = torch.int32 if route == "map32" else torch.int64
+    h = capi.CUCOStaticHashmap(torch.from_numpy(ids).to(it).cuda(), torch.arange(c, dtype=it).cuda(), 0.8)
+    q_t, upd_t = torch.from_numpy(q).cuda(), torch.from_numpy(upd).cuda()
+    if route == "mask":
+        capi.cache_set_with_mask(data_t, gpu_t, q_t, upd_t, h.query(q_t), write_through=True)
+    else:
+        capi.cache_set(data_t, gpu_t, q_t, upd_t, h, write_through=True)
+    torch.cuda.synchronize()
+    exp_host, exp_gpu = host.copy(), gpu.copy()
+    exp_host[q] = upd                                        # every updated id, hit or miss
+    slot_of = {int(k): s for s, k in enumerate(ids)}
+    for j, k in enumerate(q):
+        if int(k) in slot_of:
+            exp_gpu[slot_of[int(k)]] = upd[j]
+    assert np.array_equal(data_t.numpy().view(np.uint8), exp_host.view(np.uint8))
+    assert np.array_equal(gpu_t.cpu().numpy().view(np.uint8), exp_gpu.view(np.uint8))
+    # and the reference's own post-condition: a following fetch returns the update
+    assert torch.equal(capi.cache_fetch(data_t, gpu_t, q_t, h), upd_t)
+    assert torch.equal(capi.uva_fetch(data_t, q_t), upd_t)   # also straight from the host table
+
+
 def test_config1_small_fetch(capi, oracle):
     """Small fetch configuration: 200,000 x 128 f32 table, 50,000 cached ids, 65,536 uniform queries."""
     torch.manual_seed(0)
