@@ -16,10 +16,12 @@ int launch_scan_partials(uint64_t *partials, int64_t nb, hipStream_t s);
 // hash-table part of a relabel scratch buffer sized for N ids (n16 16-byte
 // words that must be all ones when the passes start); launch_relabel_passes()
 // runs insert -> first -> unique -> labels on `total`, which earlier kernels of
-// the same stream have filled, for n_fixed + *n_extra_dev ids (at most n_bound).
+// the same stream have filled, for n_fixed + *n_extra_dev ids (at most n_bound);
+// those kernels must also have maintained wide_flag.
 struct RelabelTable {
   void *slots;
   int64_t n16;
+  uint32_t *wide_flag;  // the earlier kernels zero it, then set it if any id lies outside [0, 2^32)
 };
 int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable *out);
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const void *n_extra_dev,

@@ -14,7 +14,8 @@
 // The table is touched only by `insert` and `first`; the last two passes read
 // dense arrays. Slots are 16 bytes {int64 key, uint32 first, pad} at load
 // factor <= 0.5 with a mixed hash (the reference hashes with the low bits of
-// the id, src/tensor_relabel.cu:111-117).
+// the id, src/tensor_relabel.cu:111-117); ids known to fit 32 bits use the
+// same memory as packed 8-byte slots (see rl_packed_insert).
 #include "common.h"
 #include "launchers.h"
 #include "scan_dev.h"
@@ -22,7 +23,7 @@
 namespace shmt {
 
 constexpr int kRlBlock = 256;
-constexpr int kRlItems = 8;
+constexpr int kRlItems = 2;
 constexpr int kRlTile = kRlBlock * kRlItems;
 constexpr int64_t kRlSelfPrefixTiles = 2048;  // up to 4 M ids the unique pass sums the tile counts itself
 
@@ -51,6 +52,10 @@ struct RlSlot {
 };
 static_assert(sizeof(RlSlot) == 16, "slot must be 16 bytes");
 
+// Table slots for the N ids the scratch buffer is sized for. When N is only an
+// upper bound of the id count (fused hop) the whole table is still used:
+// measured, the lower load shortens the probe chains of the insert pass by
+// more than clearing the smaller table would save.
 static int64_t rl_capacity(int64_t N) {
   int64_t cap = 2 * N;
   if (cap < 64) cap = 64;
@@ -58,7 +63,7 @@ static int64_t rl_capacity(int64_t N) {
 }
 
 struct RlLayout {
-  int64_t cap, table_off, rank_off, partial_off, total;
+  int64_t cap, table_off, rank_off, partial_off, flag_off, total;
 };
 
 static RlLayout rl_layout(int64_t N) {
@@ -69,7 +74,8 @@ static RlLayout rl_layout(int64_t N) {
   int64_t rank_bytes = (N * 4 + 127) & ~127ll;
   l.partial_off = l.rank_off + rank_bytes;
   int64_t nb = (N + kRlTile - 1) / kRlTile;
-  l.total = l.partial_off + ((nb * 8 + 127) & ~127ll);
+  l.flag_off = l.partial_off + ((nb * 8 + 127) & ~127ll);
+  l.total = l.flag_off + 128;
   return l;
 }
 
@@ -98,6 +104,57 @@ __device__ __forceinline__ void rl_global_insert(RlSlot *tbl, uint32_t cap, int6
   }
 }
 
+// ---- packed table for ids that fit 32 bits --------------------------------
+// The same memory seen as 8-byte slots {key : 32 | first index : 32} (twice as
+// many of them, so half the load). Key in the high half: one 64-bit atomicMin
+// per probe both claims an empty slot (all ones is the maximum) and lowers the
+// first index of a slot that already holds the key, where the 16-byte format
+// needs a CAS and a separate atomicMin. A smaller entry of another key takes a
+// slot over from a larger one; the thread that caused this carries the
+// displaced entry on along the probe sequence. Slot values only ever decrease,
+// occupied slots never become empty, and an entry moves only across occupied
+// slots, so after the kernel every key sits exactly once in the occupied run
+// that starts at its home slot, with the smallest index it was inserted with.
+constexpr unsigned long long kRlEmpty8 = ~0ull;
+
+// How insert / first address the table: 0 = 16-byte slots, 1 = packed,
+// 2 = packed unless *wide_flag is non-zero (set by an earlier kernel of the
+// stream that saw an id outside [0, 2^32)).
+struct RlPath {
+  int mode;
+  const uint32_t *wide_flag;
+};
+
+__device__ __forceinline__ bool rl_packed(const RlPath &p) {
+  return p.mode == 1 || (p.mode == 2 && *p.wide_flag == 0);
+}
+
+__device__ __forceinline__ uint32_t rl_cap8(uint32_t cap) {
+  return cap <= 0x7FFFFFFFu ? 2 * cap : cap;
+}
+
+__device__ __forceinline__ uint32_t rl_home8(uint32_t key32, uint32_t cap8) {
+  return reduce_range(hash_id(static_cast<int64_t>(key32)), cap8);
+}
+
+__device__ __forceinline__ void rl_packed_insert(unsigned long long *tbl, uint32_t cap8, uint32_t key32,
+                                                 uint32_t i) {
+  unsigned long long w = (static_cast<unsigned long long>(key32) << 32) | i;
+  uint32_t pos = rl_home8(key32, cap8);
+  for (uint32_t probes = 0; probes < cap8; ++probes) {
+    // Look before the atomic: a stale cached view can only show a larger value
+    // than the truth, in which case the atomic below settles it.
+    const unsigned long long seen = tbl[pos];
+    if ((seen >> 32) == (w >> 32) && seen <= w) return;  // key present with an index not larger
+    if (seen > w) {
+      const unsigned long long old = atomicMin(&tbl[pos], w);
+      if (old == kRlEmpty8 || (old >> 32) == (w >> 32)) return;  // claimed, or merged with the same key
+      if (old > w) w = old;  // took the slot from a larger key: carry that entry on
+    }
+    pos = (pos + 1 == cap8) ? 0 : pos + 1;
+  }
+}
+
 constexpr int kRlInsertTile = kRlBlock;          // ids per workgroup pass: one per thread
 constexpr int kRlLdsSlots = 2 * kRlInsertTile;   // per-workgroup staging table, load <= 0.5
 
@@ -107,8 +164,10 @@ constexpr int kRlLdsSlots = 2 * kRlInsertTile;   // per-workgroup staging table,
 // them) and sends one global insert per distinct id, issued by the thread that
 // holds the id's smallest index: at most one global probe chain per thread.
 __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32_t cap,
-                                                             const void *total, int eb, RlCount n) {
+                                                             const void *total, int eb, RlCount n,
+                                                             RlPath path) {
   const int64_t N = rl_count(n);
+  const bool packed = rl_packed(path);
   __shared__ unsigned long long lkey[kRlLdsSlots];
   __shared__ uint32_t lfirst[kRlLdsSlots];
   const int64_t ntiles = (N + kRlInsertTile - 1) / kRlInsertTile;
@@ -138,8 +197,13 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
     __syncthreads();
     // the thread holding the smallest index of an id inserts it for the whole tile:
     // one global probe chain per thread at most
-    if (i < N && lfirst[pos] == static_cast<uint32_t>(i))
-      rl_global_insert(tbl, cap, key, static_cast<uint32_t>(i));
+    if (i < N && lfirst[pos] == static_cast<uint32_t>(i)) {
+      if (packed)
+        rl_packed_insert(reinterpret_cast<unsigned long long *>(tbl), rl_cap8(cap),
+                         static_cast<uint32_t>(key), static_cast<uint32_t>(i));
+      else
+        rl_global_insert(tbl, cap, key, static_cast<uint32_t>(i));
+    }
     __syncthreads();
   }
 }
@@ -147,16 +211,17 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
 // First-occurrence index of every element. The first-slot loads of a
 // thread's eight elements are issued together; only the rare longer probe
 // chains continue one by one.
-__global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
-                                                            const void *total, int eb, RlCount n,
-                                                            void *labels, uint64_t *partials) {
-  const int64_t N = rl_count(n);
-  __shared__ uint64_t lds[kRlBlock / kWave];
+template <bool PACKED>
+__device__ __forceinline__ uint64_t rl_first_tile(const RlSlot *tbl, uint32_t cap, const void *total,
+                                                  int eb, int64_t N, void *labels) {
+  const unsigned long long *tbl8 = reinterpret_cast<const unsigned long long *>(tbl);
+  const uint32_t cap8 = rl_cap8(cap);
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kRlTile;
   int64_t key[kRlItems], idx[kRlItems];
   bool ok[kRlItems];
   uint32_t pos[kRlItems];
-  uint4 slot[kRlItems];
+  uint4 slot[PACKED ? 1 : kRlItems];
+  unsigned long long slot8[PACKED ? kRlItems : 1];
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
     idx[j] = base + j * kRlBlock + threadIdx.x;
@@ -165,31 +230,62 @@ __global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, u
   }
   load_ints<kRlItems>(total, idx, ok, eb, key);
 #pragma unroll
-  for (int j = 0; j < kRlItems; ++j) pos[j] = reduce_range(hash_id(key[j]), cap);
+  for (int j = 0; j < kRlItems; ++j)
+    pos[j] = PACKED ? rl_home8(static_cast<uint32_t>(key[j]), cap8) : reduce_range(hash_id(key[j]), cap);
 #pragma unroll
-  for (int j = 0; j < kRlItems; ++j) slot[j] = *reinterpret_cast<const uint4 *>(&tbl[pos[j]]);
+  for (int j = 0; j < kRlItems; ++j) {
+    if (PACKED)
+      slot8[j] = tbl8[pos[j]];
+    else
+      slot[j] = *reinterpret_cast<const uint4 *>(&tbl[pos[j]]);
+  }
   uint64_t cnt = 0;
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
-    const int64_t i = base + j * kRlBlock + threadIdx.x;
+    const int64_t i = idx[j];
     if (i < N) {
-      uint4 s = slot[j];
       uint32_t p = pos[j];
       uint32_t f = 0xFFFFFFFFu;
-      for (uint32_t probes = 0; probes < cap; ++probes) {
-        const int64_t k = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
-        if (k == key[j]) {
-          f = s.z;
-          break;
+      if (PACKED) {
+        const uint32_t key32 = static_cast<uint32_t>(key[j]);
+        unsigned long long s8 = slot8[j];
+        for (uint32_t probes = 0; probes < cap8; ++probes) {
+          if (static_cast<uint32_t>(s8 >> 32) == key32 && s8 != kRlEmpty8) {
+            f = static_cast<uint32_t>(s8);
+            break;
+          }
+          if (s8 == kRlEmpty8) break;
+          p = (p + 1 == cap8) ? 0 : p + 1;
+          s8 = tbl8[p];
         }
-        if (k == -1) break;
-        p = (p + 1 == cap) ? 0 : p + 1;
-        s = *reinterpret_cast<const uint4 *>(&tbl[p]);
+      } else {
+        uint4 s = slot[j];
+        for (uint32_t probes = 0; probes < cap; ++probes) {
+          const int64_t k = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
+          if (k == key[j]) {
+            f = s.z;
+            break;
+          }
+          if (k == -1) break;
+          p = (p + 1 == cap) ? 0 : p + 1;
+          s = *reinterpret_cast<const uint4 *>(&tbl[p]);
+        }
       }
       store_int(labels, i, eb, static_cast<int64_t>(f));
       cnt += (f == static_cast<uint32_t>(i));
     }
   }
+  return cnt;
+}
+
+__global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
+                                                            const void *total, int eb, RlCount n,
+                                                            void *labels, uint64_t *partials,
+                                                            RlPath path) {
+  const int64_t N = rl_count(n);
+  __shared__ uint64_t lds[kRlBlock / kWave];
+  const uint64_t cnt = rl_packed(path) ? rl_first_tile<true>(tbl, cap, total, eb, N, labels)
+                                       : rl_first_tile<false>(tbl, cap, total, eb, N, labels);
   uint64_t tile_total;
   block_exclusive_scan<uint64_t, kRlBlock>(cnt, lds, &tile_total);
   if (threadIdx.x == 0) partials[blockIdx.x] = tile_total;
@@ -312,7 +408,8 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
 // kernels work on the true count.
 static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
                         int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
-                        void *labels_out, int64_t *count_out, void *stream, bool prepared = false) {
+                        void *labels_out, int64_t *count_out, void *stream, bool prepared = false,
+                        bool ids_flagged = false) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
@@ -338,6 +435,9 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   uint64_t *partials = reinterpret_cast<uint64_t *>(base + l.partial_off);
   const int64_t nb = (N + kRlTile - 1) / kRlTile;
   const uint32_t cap = static_cast<uint32_t>(l.cap);
+  // 4-byte ids always fit the packed table; 8-byte ids use it when an earlier kernel vouches for them
+  RlPath path{elem_bytes == 4 ? 1 : (ids_flagged ? 2 : 0),
+              reinterpret_cast<const uint32_t *>(base + l.flag_off)};
 
   int rc = SHMT_OK;
   if (prepared) {
@@ -353,10 +453,10 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     if (rc) return rc;
   }
   hipLaunchKernelGGL(rl_insert_kernel, dim3(grid_for(N, kRlInsertTile, 256 * 32)), dim3(kRlBlock), 0,
-                     s, tbl, cap, total, elem_bytes, n);
+                     s, tbl, cap, total, elem_bytes, n, path);
   SHMT_LAUNCH_CHECK();
   hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, tbl,
-                     cap, total, elem_bytes, n, labels_out, partials);
+                     cap, total, elem_bytes, n, labels_out, partials, path);
   SHMT_LAUNCH_CHECK();
   const int scanned = nb > kRlSelfPrefixTiles;
   if (scanned) {
@@ -388,6 +488,7 @@ int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable 
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "relabel: scratch must be 16-byte aligned");
   out->slots = static_cast<char *>(scratch) + l.table_off;
   out->n16 = l.cap;
+  out->wide_flag = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + l.flag_off);
   return SHMT_OK;
 }
 
@@ -395,7 +496,8 @@ int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, c
                           int n_extra_bytes, int elem_bytes, void *scratch, int64_t scratch_bytes,
                           void *unique_out, void *labels_out, int64_t *count_out, hipStream_t stream) {
   return relabel_impl(total, nullptr, n_bound, RlCount{n_fixed, n_extra_dev, n_extra_bytes, n_bound},
-                      elem_bytes, scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true);
+                      elem_bytes, scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true,
+                      true);
 }
 
 }  // namespace shmt

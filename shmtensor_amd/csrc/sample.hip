@@ -50,6 +50,7 @@ struct PlanArgs {
   int replace;
   void *seed_copy;      // optional: seeds widened to seed_copy_bytes (head of a relabel input)
   int seed_copy_bytes;
+  uint32_t *wide_flag;  // optional: zeroed here; the pick kernel raises it for ids outside [0, 2^32)
 };
 
 // MODE 0: no cache; 1: wide map; 2: narrow map.
@@ -80,6 +81,7 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
 template <int MODE>
 __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
+  if (a.wide_flag && threadIdx.x == 0) *a.wide_flag = 0;
   uint64_t carry = 0;
   for (int64_t base = 0; base < a.S; base += kPlanBlock) {
     const int64_t i = base + threadIdx.x;
@@ -100,6 +102,7 @@ __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
 template <int MODE>
 __global__ __launch_bounds__(kPlanBlock) void plan_tile_kernel(PlanArgs a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
+  if (a.wide_flag && blockIdx.x == 0 && threadIdx.x == 0) *a.wide_flag = 0;
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kPlanBlock + threadIdx.x;
   const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, i));
   uint64_t total;
@@ -182,7 +185,12 @@ struct PickArgs {
   int copy_bytes;
   uint4 *clear;                 // clear_n 16-byte words set to all ones (the relabel table)
   int64_t clear_n;
+  uint32_t *wide_flag;          // raised when a seed or a sampled id lies outside [0, 2^32)
 };
+
+__device__ __forceinline__ void note_wide_id(const PickArgs &a, int64_t id) {
+  if (static_cast<uint64_t>(id) >> 32) atomicOr(a.wide_flag, 1u);
+}
 
 // Output offset of seed s. In the fused hop the plan left tile-local offsets:
 // the tile's prefix is added here and the final value written back by `writer`.
@@ -190,6 +198,7 @@ template <bool HOP>
 __device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, bool writer) {
   if (!HOP) return load_int(a.sub_indptr, s, a.ptr_bytes);
   int64_t optr = load_int(a.sub_indptr_rw, s, a.ptr_bytes);
+  if (writer) note_wide_id(a, load_int(a.seeds, s, a.seed_bytes));
   if (a.tile_prefix) {
     optr += static_cast<int64_t>(a.tile_prefix[s / kPlanBlock]);
     if (writer) store_int(a.sub_indptr_rw, s, a.ptr_bytes, optr);
@@ -200,7 +209,10 @@ __device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, boo
 template <bool HOP>
 __device__ __forceinline__ void pick_store(const PickArgs &a, int64_t pos, int64_t v) {
   store_int(a.out, pos, a.idx_bytes, v);
-  if (HOP) store_int(a.copy_out, a.copy_base + pos, a.copy_bytes, v);
+  if (HOP) {
+    store_int(a.copy_out, a.copy_base + pos, a.copy_bytes, v);
+    note_wide_id(a, v);
+  }
 }
 
 template <bool HOP>
@@ -407,6 +419,7 @@ int64_t shmt_sample_plan_bytes(int64_t S) {
 struct PlanHopExtras {
   void *seed_copy;
   int seed_copy_bytes;
+  uint32_t *wide_flag;
   const uint64_t *tile_prefix_out;
 };
 
@@ -449,6 +462,7 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   a.replace = replace ? 1 : 0;
   a.seed_copy = hop ? hop->seed_copy : nullptr;
   a.seed_copy_bytes = hop ? hop->seed_copy_bytes : 8;
+  a.wide_flag = hop ? hop->wide_flag : nullptr;
   if (hop) hop->tile_prefix_out = nullptr;
   const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
 
@@ -504,6 +518,7 @@ struct PickHopExtras {
   int copy_bytes;
   uint4 *clear;
   int64_t clear_n;
+  uint32_t *wide_flag;
 };
 
 template <bool HOP>
@@ -569,6 +584,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.copy_bytes = 8;
   a.clear = nullptr;
   a.clear_n = 0;
+  a.wide_flag = nullptr;
   hipStream_t s = as_stream(stream);
   if (!hop) return pick_launch<false>(a, s);
   a.sub_indptr_rw = hop->sub_indptr_rw;
@@ -578,6 +594,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.copy_bytes = hop->copy_bytes;
   a.clear = hop->clear;
   a.clear_n = hop->clear_n;
+  a.wide_flag = hop->wide_flag;
   return pick_launch<true>(a, s);
 }
 
@@ -608,12 +625,12 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
   RelabelTable table;
   int rc = relabel_table(n_max, scratch, scratch_bytes, &table);
   if (rc) return rc;
-  PlanHopExtras plan_hop{total_out, elem_bytes, nullptr};
+  PlanHopExtras plan_hop{total_out, elem_bytes, table.wide_flag, nullptr};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
                  plan_bytes, nnz_out, stream, &plan_hop);
   if (rc) return rc;
   const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, total_out, S, elem_bytes,
-                               static_cast<uint4 *>(table.slots), table.n16};
+                               static_cast<uint4 *>(table.slots), table.n16, table.wide_flag};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                  plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
   if (rc) return rc;

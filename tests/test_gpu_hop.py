@@ -282,3 +282,29 @@ def test_sample_hop_c_abi_matches_separate_entry_points(cabi):
     assert lib.shmt_sample_hop(indptr.data_ptr(), 8, indices.data_ptr(), 4, None, None, None, seeds.data_ptr(), 8, 0, 5, 0,
                                1, 0, None, None, None, 0, 8, None, None, 0, None, None, None, None, stream) == -1
     assert b"must be >= 1" in lib.shmt_last_error()
+
+
+@pytest.mark.parametrize("odd_ids", ["none", "beyond_32_bits", "negative", "uint32_max"])
+def test_hop_relabel_table_format_follows_the_id_range(capi, oracle, odd_ids):
+    """The hop's relabel uses packed 8-byte slots while every id fits 32 bits and falls
+    back to 16-byte slots otherwise; both must give the oracle's labels. Heavy
+    repetition of a few ids and dense id ranges stress slot take-overs in the packed table."""
+    rng = np.random.default_rng(5)
+    n, deg = 4000, 12
+    indptr = np.arange(0, (n + 1) * deg, deg, dtype=np.int64)
+    indices = rng.integers(0, 600, size=n * deg).astype(np.int64)          # few distinct ids, many repeats
+    indices[::7] = rng.integers(0, 2**31, size=indices[::7].size)           # and some spread over 31 bits
+    if odd_ids == "beyond_32_bits":
+        indices[5::11] += 2**32
+    elif odd_ids == "negative":
+        indices[3::13] = -indices[3::13] - 2
+    elif odd_ids == "uint32_max":
+        indices[2::9] = 2**32 - 1
+    seeds = rng.permutation(n)[:3000].astype(np.int64)
+    ip, ix, sd = (torch.from_numpy(x).cuda() for x in (indptr, indices, seeds))
+    for k in (12, 5):
+        sp, si, uniq, lab = capi.sample_hop(ip, ix, None, None, None, sd, k, False, seed=1)
+        exp_unique, (exp_seed_labels, exp_labels) = oracle.relabel([seeds, si.cpu().numpy()])
+        assert np.array_equal(uniq.cpu().numpy(), exp_unique)
+        assert np.array_equal(lab.cpu().numpy(), exp_labels)
+        _same((sp, si, uniq, lab), _two_step(capi, ip, ix, None, sd, k, False, seed=1))
