@@ -207,6 +207,42 @@ int main() {
     EXPECT(std::adjacent_find(s.begin(), s.end()) == s.end() && s.front() >= lo[seg] && s.back() < hi[seg]);
   }
 
+  // ---- the same hop as one launch sequence: sample + relabel([seeds, sampled]) ----
+  {
+    const int64_t S = 7, k = 5, n_max = S + S * k;
+    int64_t *d_sp2 = nullptr, *d_sub2 = nullptr, *d_total = nullptr, *d_uniq2 = nullptr, *d_lab2 = nullptr;
+    int64_t *h_nnz = nullptr, *h_uniq_count = nullptr;
+    void *d_plan2 = nullptr, *d_scratch2 = nullptr;
+    HIP_OK(hipMalloc(&d_sp2, (S + 1) * 8));
+    HIP_OK(hipMalloc(&d_sub2, S * k * 8));
+    HIP_OK(hipMalloc(&d_total, n_max * 8));
+    HIP_OK(hipMalloc(&d_uniq2, n_max * 8));
+    HIP_OK(hipMalloc(&d_lab2, n_max * 8));
+    HIP_OK(hipMalloc(&d_plan2, pbytes));
+    const int64_t sbytes2 = shmt_relabel_scratch_bytes(n_max);
+    HIP_OK(hipMalloc(&d_scratch2, sbytes2));
+    HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&h_nnz), 8, hipHostMallocDefault));
+    HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&h_uniq_count), 8, hipHostMallocDefault));
+    SHMT_OK_(shmt_sample_hop(d_indptr, 8, d_indices, 8, nullptr, nullptr, nullptr, d_seeds, 8, S, k, 0, 7777, 0,
+                             d_sp2, d_sub2, d_plan2, pbytes, 8, d_total, d_scratch2, sbytes2, d_uniq2, d_lab2,
+                             h_nnz, h_uniq_count, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    EXPECT(*h_nnz == 25);
+    EXPECT(to_host(d_sp2, 8) == to_host(d_sub_indptr, 8));
+    EXPECT(to_host(d_sub2, 25) == sub);                      // same seed and stream: same sample
+    std::vector<int64_t> all(seeds);
+    all.insert(all.end(), sub.begin(), sub.end());
+    std::unordered_map<int64_t, int64_t> first2;
+    std::vector<int64_t> uniq2;
+    for (int64_t x : all)
+      if (first2.emplace(x, static_cast<int64_t>(uniq2.size())).second) uniq2.push_back(x);
+    EXPECT(*h_uniq_count == static_cast<int64_t>(uniq2.size()));
+    EXPECT(to_host(d_uniq2, uniq2.size()) == uniq2);
+    EXPECT(to_host(d_total, all.size()) == all);
+    std::vector<int64_t> lab2 = to_host(d_lab2, all.size());
+    for (size_t i = 0; i < all.size(); ++i) EXPECT(lab2[i] == first2[all[i]]);
+  }
+
   shmt_hashmap_destroy(map);
   shmt_hashmap_destroy(fmap);
   printf("cabi_smoke: all checks passed\n");
