@@ -529,7 +529,7 @@ struct PendingHop {
   HopResult result;                       // valid when finished
   int64_t S = 0;
   torch::Tensor sub_indptr, sub_indices, unique, labels;
-  torch::Tensor plan, total, scratch;     // kept until the sizes are in
+  torch::Tensor workspace;                // plan + relabel input + relabel scratch, kept until the sizes are in
   Readback::Slot nnz_slot{}, count_slot{};
 };
 
@@ -553,22 +553,34 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   const int pb = static_cast<int>(g.indptr.element_size());
   const int ib = static_cast<int>(g.indices.element_size());
   const int sb = static_cast<int>(seeds.element_size());
-  const auto dev = torch::kCUDA;
   void *stream = current_stream();
   const int64_t bound = S * num_picks;
   h.S = S;
-  h.sub_indptr = torch::empty({S + 1}, g.indptr.options().device(dev));
-  h.sub_indices = torch::empty({bound}, g.indices.options().device(dev));
-  const int64_t plan_bytes = shmt_sample_plan_bytes(S);
-  h.plan = device_bytes(plan_bytes);
   const int eb = std::max(sb, ib);
-  const auto id_options = seeds.options().dtype(eb == 8 ? torch::kInt64 : torch::kInt32);
+  const auto id_type = eb == 8 ? torch::kInt64 : torch::kInt32;
   const int64_t n_max = S + bound;
-  h.total = torch::empty({n_max}, id_options);
-  h.unique = torch::empty({n_max}, id_options);
-  h.labels = torch::empty({n_max}, id_options);
+  auto aligned = [](int64_t bytes) { return (bytes + 255) & ~int64_t{255}; };
+  // Two allocations per hop (the allocator is shared by all host threads that drive
+  // batches): one for the four results, which are typed views of it, ...
+  torch::Tensor results = device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) + 2 * aligned(n_max * eb));
+  int64_t offset = 0;
+  auto carve = [&](int64_t count, int elem, torch::ScalarType type) {
+    torch::Tensor t = results.narrow(0, offset, count * elem).view(type);
+    offset += aligned(count * elem);
+    return t;
+  };
+  h.sub_indptr = carve(S + 1, pb, g.indptr.scalar_type());
+  h.sub_indices = carve(bound, ib, g.indices.scalar_type());
+  h.unique = carve(n_max, eb, id_type);
+  h.labels = carve(n_max, eb, id_type);
+  // ... and one for everything that does not outlive the hop
+  const int64_t plan_bytes = shmt_sample_plan_bytes(S);
+  const int64_t total_bytes = n_max * eb;
   const int64_t scratch_bytes = shmt_relabel_scratch_bytes(n_max);
-  h.scratch = device_bytes(scratch_bytes);
+  h.workspace = device_bytes(aligned(plan_bytes) + aligned(total_bytes) + scratch_bytes);
+  char *const plan_ptr = static_cast<char *>(h.workspace.data_ptr());
+  char *const total_ptr = plan_ptr + aligned(plan_bytes);
+  char *const scratch_ptr = total_ptr + aligned(total_bytes);
   h.nnz_slot = readback().acquire();
   h.count_slot = readback().acquire();
   check(shmt_sample_hop(device_address(g.indptr, "indptr"), pb, device_address(g.indices, "indices"), ib,
@@ -577,7 +589,7 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
                         g.cached() ? g.hashmap->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks,
                         replace, static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
                         static_cast<uint32_t>(stream_id), h.sub_indptr.data_ptr(), h.sub_indices.data_ptr(),
-                        h.plan.data_ptr(), plan_bytes, eb, h.total.data_ptr(), h.scratch.data_ptr(),
+                        plan_ptr, plan_bytes, eb, total_ptr, scratch_ptr,
                         scratch_bytes, h.unique.data_ptr(), h.labels.data_ptr(), h.nnz_slot.dev,
                         h.count_slot.dev, stream));
   return h;
@@ -594,7 +606,7 @@ HopResult hop_finish(PendingHop &h) {
     h.finished = true;
     // scratch goes back to the allocator of its stream; work queued later on
     // that stream is ordered after the kernels that still read it
-    h.plan = h.total = h.scratch = torch::Tensor();
+    h.workspace = torch::Tensor();
   }
   return h.result;
 }
