@@ -17,15 +17,18 @@ int launch_scan_partials(uint64_t *partials, int64_t nb, hipStream_t s);
 // words that must be all ones when the passes start); launch_relabel_passes()
 // runs insert -> first -> unique -> labels on `total`, which earlier kernels of
 // the same stream have filled, for n_fixed + *n_extra_dev ids (at most n_bound);
-// those kernels must also have maintained wide_flag.
+// those kernels must also have stored `nonce` to *wide_mark if any id lies outside [0, 2^32).
 struct RelabelTable {
   void *slots;
   int64_t n16;
-  uint32_t *wide_flag;  // the earlier kernels zero it, then set it if any id lies outside [0, 2^32)
+  uint64_t *wide_mark;  // where the earlier kernels store `nonce` when an id lies outside [0, 2^32)
+  uint64_t nonce;
 };
 int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable *out);
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const void *n_extra_dev,
                           int n_extra_bytes, int elem_bytes, void *scratch, int64_t scratch_bytes,
-                          void *unique_out, void *labels_out, int64_t *count_out, hipStream_t stream);
+                          void *unique_out, void *labels_out, int64_t *count_out, uint64_t nonce,
+                          hipStream_t stream);
+uint64_t relabel_nonce();
 
 }  // namespace shmt

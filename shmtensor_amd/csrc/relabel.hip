@@ -20,6 +20,8 @@
 #include "launchers.h"
 #include "scan_dev.h"
 
+#include <atomic>
+
 namespace shmt {
 
 constexpr int kRlBlock = 256;
@@ -118,15 +120,19 @@ __device__ __forceinline__ void rl_global_insert(RlSlot *tbl, uint32_t cap, int6
 constexpr unsigned long long kRlEmpty8 = ~0ull;
 
 // How insert / first address the table: 0 = 16-byte slots, 1 = packed,
-// 2 = packed unless *wide_flag is non-zero (set by an earlier kernel of the
-// stream that saw an id outside [0, 2^32)).
+// 2 = packed unless *wide_mark equals this call's nonce. The kernel that
+// writes the ids earlier on the stream stores the nonce there when it sees an
+// id outside [0, 2^32); the mark lives in uninitialised scratch and is never
+// cleared: leftover bits can only pass for the nonce by a 2^-64 accident, and
+// then the 16-byte format is used, which is correct for every id.
 struct RlPath {
   int mode;
-  const uint32_t *wide_flag;
+  const uint64_t *wide_mark;
+  uint64_t nonce;
 };
 
 __device__ __forceinline__ bool rl_packed(const RlPath &p) {
-  return p.mode == 1 || (p.mode == 2 && *p.wide_flag == 0);
+  return p.mode == 1 || (p.mode == 2 && *p.wide_mark != p.nonce);
 }
 
 __device__ __forceinline__ uint32_t rl_cap8(uint32_t cap) {
@@ -371,7 +377,8 @@ struct RlSegments {
 // First pass when the input arrives as segments: empties the table and writes
 // the concatenated, widened ids in one sweep (both are streaming stores).
 __global__ __launch_bounds__(256) void rl_fill_concat_kernel(uint4 *tbl16, int64_t cap, RlSegments segs,
-                                                             void *total, int eb, RlCount n) {
+                                                             void *total, int eb, RlCount n,
+                                                             uint64_t *wide_mark, uint64_t nonce) {
   const int64_t N = rl_count(n);
   int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -382,7 +389,9 @@ __global__ __launch_bounds__(256) void rl_fill_concat_kernel(uint4 *tbl16, int64
     if (i < N) {
       int sgm = 0;
       while (sgm + 1 < segs.n && i >= segs.start[sgm + 1]) ++sgm;
-      store_int(total, i, eb, load_int(segs.ptr[sgm], i - segs.start[sgm], segs.bytes[sgm]));
+      const int64_t id = load_int(segs.ptr[sgm], i - segs.start[sgm], segs.bytes[sgm]);
+      store_int(total, i, eb, id);
+      if (static_cast<uint64_t>(id) >> 32) *wide_mark = nonce;
     }
   }
 }
@@ -390,6 +399,15 @@ __global__ __launch_bounds__(256) void rl_fill_concat_kernel(uint4 *tbl16, int64
 __global__ void rl_zero_count_kernel(int64_t *count_out) {
   *count_out = 0;
   __threadfence_system();
+}
+
+// A value no earlier call has used (and that uninitialised memory is unlikely to hold).
+uint64_t relabel_nonce() {
+  static std::atomic<uint64_t> counter{0x9E3779B97F4A7C15ull};
+  uint64_t z = counter.fetch_add(0x9E3779B97F4A7C15ull, std::memory_order_relaxed);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;  // splitmix64 finaliser
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
 }
 
 }  // namespace shmt
@@ -409,7 +427,7 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
 static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
                         int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
                         void *labels_out, int64_t *count_out, void *stream, bool prepared = false,
-                        bool ids_flagged = false) {
+                        uint64_t prepared_nonce = 0) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
@@ -436,8 +454,10 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   const int64_t nb = (N + kRlTile - 1) / kRlTile;
   const uint32_t cap = static_cast<uint32_t>(l.cap);
   // 4-byte ids always fit the packed table; 8-byte ids use it when an earlier kernel vouches for them
-  RlPath path{elem_bytes == 4 ? 1 : (ids_flagged ? 2 : 0),
-              reinterpret_cast<const uint32_t *>(base + l.flag_off)};
+  // (plain shmt_relabel has no kernel that sees the ids before the insert pass: 16-byte slots)
+  uint64_t *wide_mark = reinterpret_cast<uint64_t *>(base + l.flag_off);
+  const uint64_t nonce = prepared ? prepared_nonce : relabel_nonce();
+  RlPath path{elem_bytes == 4 ? 1 : ((prepared || segs) ? 2 : 0), wide_mark, nonce};
 
   int rc = SHMT_OK;
   if (prepared) {
@@ -446,7 +466,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     const int64_t span = l.cap > N ? l.cap : N;
     hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(span, 256 * 4)), dim3(256), 0, s,
                        reinterpret_cast<uint4 *>(tbl), l.cap, *segs, const_cast<void *>(total),
-                       elem_bytes, n);
+                       elem_bytes, n, wide_mark, nonce);
     SHMT_LAUNCH_CHECK();
   } else {
     rc = launch_fill_ones(tbl, l.cap, s);
@@ -488,16 +508,18 @@ int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable 
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "relabel: scratch must be 16-byte aligned");
   out->slots = static_cast<char *>(scratch) + l.table_off;
   out->n16 = l.cap;
-  out->wide_flag = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + l.flag_off);
+  out->wide_mark = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + l.flag_off);
+  out->nonce = relabel_nonce();
   return SHMT_OK;
 }
 
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const void *n_extra_dev,
                           int n_extra_bytes, int elem_bytes, void *scratch, int64_t scratch_bytes,
-                          void *unique_out, void *labels_out, int64_t *count_out, hipStream_t stream) {
+                          void *unique_out, void *labels_out, int64_t *count_out, uint64_t nonce,
+                          hipStream_t stream) {
   return relabel_impl(total, nullptr, n_bound, RlCount{n_fixed, n_extra_dev, n_extra_bytes, n_bound},
                       elem_bytes, scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true,
-                      true);
+                      nonce);
 }
 
 }  // namespace shmt

@@ -50,7 +50,6 @@ struct PlanArgs {
   int replace;
   void *seed_copy;      // optional: seeds widened to seed_copy_bytes (head of a relabel input)
   int seed_copy_bytes;
-  uint32_t *wide_flag;  // optional: zeroed here; the pick kernel raises it for ids outside [0, 2^32)
 };
 
 // MODE 0: no cache; 1: wide map; 2: narrow map.
@@ -81,7 +80,6 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
 template <int MODE>
 __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
-  if (a.wide_flag && threadIdx.x == 0) *a.wide_flag = 0;
   uint64_t carry = 0;
   for (int64_t base = 0; base < a.S; base += kPlanBlock) {
     const int64_t i = base + threadIdx.x;
@@ -102,7 +100,6 @@ __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
 template <int MODE>
 __global__ __launch_bounds__(kPlanBlock) void plan_tile_kernel(PlanArgs a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
-  if (a.wide_flag && blockIdx.x == 0 && threadIdx.x == 0) *a.wide_flag = 0;
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kPlanBlock + threadIdx.x;
   const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, i));
   uint64_t total;
@@ -185,11 +182,12 @@ struct PickArgs {
   int copy_bytes;
   uint4 *clear;                 // clear_n 16-byte words set to all ones (the relabel table)
   int64_t clear_n;
-  uint32_t *wide_flag;          // raised when a seed or a sampled id lies outside [0, 2^32)
+  uint64_t *wide_mark;          // receives wide_nonce when a seed or a sampled id lies outside [0, 2^32)
+  uint64_t wide_nonce;
 };
 
 __device__ __forceinline__ void note_wide_id(const PickArgs &a, int64_t id) {
-  if (static_cast<uint64_t>(id) >> 32) atomicOr(a.wide_flag, 1u);
+  if (static_cast<uint64_t>(id) >> 32) *a.wide_mark = a.wide_nonce;
 }
 
 // Output offset of seed s. In the fused hop the plan left tile-local offsets:
@@ -419,7 +417,6 @@ int64_t shmt_sample_plan_bytes(int64_t S) {
 struct PlanHopExtras {
   void *seed_copy;
   int seed_copy_bytes;
-  uint32_t *wide_flag;
   const uint64_t *tile_prefix_out;
 };
 
@@ -462,7 +459,6 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   a.replace = replace ? 1 : 0;
   a.seed_copy = hop ? hop->seed_copy : nullptr;
   a.seed_copy_bytes = hop ? hop->seed_copy_bytes : 8;
-  a.wide_flag = hop ? hop->wide_flag : nullptr;
   if (hop) hop->tile_prefix_out = nullptr;
   const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
 
@@ -518,7 +514,8 @@ struct PickHopExtras {
   int copy_bytes;
   uint4 *clear;
   int64_t clear_n;
-  uint32_t *wide_flag;
+  uint64_t *wide_mark;
+  uint64_t wide_nonce;
 };
 
 template <bool HOP>
@@ -584,7 +581,8 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.copy_bytes = 8;
   a.clear = nullptr;
   a.clear_n = 0;
-  a.wide_flag = nullptr;
+  a.wide_mark = nullptr;
+  a.wide_nonce = 0;
   hipStream_t s = as_stream(stream);
   if (!hop) return pick_launch<false>(a, s);
   a.sub_indptr_rw = hop->sub_indptr_rw;
@@ -594,7 +592,8 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.copy_bytes = hop->copy_bytes;
   a.clear = hop->clear;
   a.clear_n = hop->clear_n;
-  a.wide_flag = hop->wide_flag;
+  a.wide_mark = hop->wide_mark;
+  a.wide_nonce = hop->wide_nonce;
   return pick_launch<true>(a, s);
 }
 
@@ -625,12 +624,12 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
   RelabelTable table;
   int rc = relabel_table(n_max, scratch, scratch_bytes, &table);
   if (rc) return rc;
-  PlanHopExtras plan_hop{total_out, elem_bytes, table.wide_flag, nullptr};
+  PlanHopExtras plan_hop{total_out, elem_bytes, nullptr};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
                  plan_bytes, nnz_out, stream, &plan_hop);
   if (rc) return rc;
   const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, total_out, S, elem_bytes,
-                               static_cast<uint4 *>(table.slots), table.n16, table.wide_flag};
+                               static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                  plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
   if (rc) return rc;
@@ -638,7 +637,7 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
   // number of sampled ids read from sub_indptr[S]
   return launch_relabel_passes(total_out, n_max, S, static_cast<const char *>(sub_indptr) + S * ptr_bytes,
                                ptr_bytes, elem_bytes, scratch, scratch_bytes, unique_out, labels_out,
-                               count_out, as_stream(stream));
+                               count_out, table.nonce, as_stream(stream));
 }
 
 int shmt_subcsr_plan(const void *indptr, int ptr_bytes, const void *seeds, int seed_bytes,

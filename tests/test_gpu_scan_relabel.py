@@ -65,6 +65,30 @@ def test_relabel_matches_oracle(capi, oracle, n, dt):
     assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
 
 
+@pytest.mark.parametrize("n", [9, 300, 2049, 100_000, 1_500_000])
+@pytest.mark.parametrize("odd", ["one_wide_id_at_the_end", "many_wide", "negative", "uint32_max", "mixed_widths"])
+def test_relabel_id_ranges_select_the_table_format(capi, oracle, n, odd):
+    """8-byte ids that all fit 32 bits go through the packed table, anything else through
+    16-byte slots; dense ranges and heavy repetition stress slot take-overs. Same labels either way."""
+    rng = np.random.default_rng(n)
+    a = rng.integers(0, max(2, n // 4), size=n).astype(np.int64)
+    a[::5] = rng.integers(0, 2**32, size=a[::5].size)                  # spread over the full 32-bit range
+    b = rng.integers(0, max(2, n // 4), size=n // 2 + 1)
+    b = b.astype(np.int32 if odd == "mixed_widths" else np.int64)
+    if odd == "one_wide_id_at_the_end":
+        b[-1] = 2**32
+    elif odd == "many_wide":
+        a[1::3] += 2**40
+    elif odd == "negative":
+        b[::7] = -b[::7] - 1
+    elif odd == "uint32_max":
+        a[::9] = 2**32 - 1
+    u, (la, lb) = capi.tensor_relabel([torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()])
+    eu, (ea, eb) = oracle.relabel([a, b])
+    assert np.array_equal(u.cpu().numpy(), eu)
+    assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
+
+
 def test_relabel_mixed_dtypes_prefix_property(capi, oracle):
     # the dataloader's call: [int64 seeds, int32 sub_indices] (python/shmtensor/sampling.py:137-138)
     rng = np.random.default_rng(5)
