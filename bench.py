@@ -359,12 +359,14 @@ def bench_sampling(capi, args, result):
     g = torch.Generator(device="cuda").manual_seed(33)
     seed_batches = [torch.randperm(n, device="cuda", generator=g)[:S].contiguous() for _ in range(nbatch)]
 
-    def run_batch(seeds, b, fused=False):
+    indptr_hbm = indptr.cuda()      # 8 bytes per node: small next to the adjacency, which stays split
+
+    def run_batch(seeds, b, fused=False, ptr=None):
         edges = 0
         for hop, k in enumerate(reversed(fanouts)):       # python/shmtensor/sampling.py:128
             if fused:     # the same two operators queued as one call (one host wait per hop)
-                sp, si, uniq, rel = capi.sample_hop(indptr, indices, gp, gi, hmap, seeds, k, False, seed=7777 + b,
-                                                    stream_id=hop)
+                sp, si, uniq, rel = capi.sample_hop(indptr if ptr is None else ptr, indices, gp, gi, hmap, seeds, k,
+                                                    False, seed=7777 + b, stream_id=hop)
             else:
                 sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, hmap, seeds, k, False, seed=7777 + b,
                                                  stream_id=hop)
@@ -373,12 +375,12 @@ def bench_sampling(capi, args, result):
             seeds = uniq
         return edges
 
-    def timed(fused):
+    def timed(fused, ptr=None):
         for b in range(3):
-            run_batch(seed_batches[b], b, fused)
+            run_batch(seed_batches[b], b, fused, ptr)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        edges = sum(run_batch(seed_batches[b], b, fused) for b in range(nbatch))
+        edges = sum(run_batch(seed_batches[b], b, fused, ptr) for b in range(nbatch))
         torch.cuda.synchronize()
         return edges, time.perf_counter() - t0
 
@@ -401,6 +403,10 @@ def bench_sampling(capi, args, result):
     edges, gpu_t = timed(False)
     edges_fused, gpu_t_fused = timed(True)
     assert edges_fused == edges, "fused hop sampled a different number of edges"
+    # the caller's choice, not part of the configuration: the whole indptr in HBM (cold rows then cost one
+    # host-link round trip per hop instead of two)
+    edges_hbm, gpu_t_hbm = timed(True, indptr_hbm)
+    assert edges_hbm == edges, "indptr placement changed the sample"
     overlapped = {}
     for in_flight in (1, 2, 4, 8, 16):
         e, t = timed_in_flight(in_flight)
@@ -414,6 +420,7 @@ def bench_sampling(capi, args, result):
            "sampled_edges_per_s": round(edges / gpu_t, 1),
            "fused_hop_ms_per_batch": round(gpu_t_fused * 1e3 / nbatch, 4),
            "fused_hop_sampled_edges_per_s": round(edges / gpu_t_fused, 1),
+           "fused_hop_indptr_in_hbm_ms_per_batch": round(gpu_t_hbm * 1e3 / nbatch, 4),
            "sample_blocks_batches_in_flight": overlapped}
     if not args.no_cpu:
         from oracle import oracle as orc

@@ -49,7 +49,8 @@ def _unpin(tensor):
 class GPUSamplingDataloader:
 
     def __init__(self, indptr, indices, seeds, batchsize, num_picks, replace=False, use_ddp=False,
-                 shuffle=True, drop_last=False, rng_seed=None, prefetch=1, background=False):
+                 shuffle=True, drop_last=False, rng_seed=None, prefetch=1, background=False,
+                 indptr_on_device=False):
         self.indptr = indptr
         self.indices = indices
         self.seeds = seeds
@@ -78,6 +79,10 @@ class GPUSamplingDataloader:
         self.gpu_indices = None
         self.hashmap = None
 
+        # indptr_on_device: the row offsets (8 bytes per node, small next to the adjacency) live in
+        # HBM whatever the cache holds; a cold row then costs one host-link round trip per hop, not two
+        if indptr_on_device and self.indptr.device.type == "cpu":
+            self.indptr = self.indptr.cuda()
         for name in ("indptr", "indices"):
             t = getattr(self, name)
             if t.device.type == "cpu":

@@ -72,12 +72,21 @@ def test_cache_does_not_change_results(capi, graph):
     assert abs(cached.gpu_indptr.numel() - 1 - np.searchsorted(cost, full // 3)) <= 8
     cached_bytes = cached.gpu_indices.numel() * 8 + (cached.gpu_indptr.numel() - 1) * 18
     assert cached_bytes <= full // 3
+    cached_gpu_indptr = cached.gpu_indptr
     for (a_in, a_out, a_blocks), (b_in, b_out, b_blocks) in zip(plain, cached):
         assert torch.equal(a_in, b_in) and torch.equal(a_out, b_out)
         for x, y in zip(a_blocks, b_blocks):
             assert torch.equal(x.indptr, y.indptr) and torch.equal(x.indices, y.indices)
     cached.clear_cache()
     assert not cached.has_cache and cached.hashmap is None
+    split = _loader(graph, indptr_on_device=True)                   # offsets in HBM, adjacency pinned + cached
+    assert split.indptr.is_cuda and split.indices.is_pinned()
+    split.create_cache(full // 3, sampling_hot)
+    assert split.has_cache and torch.equal(split.gpu_indptr, cached_gpu_indptr)
+    for (a_in, _, a_blocks), (b_in, _, b_blocks) in zip(plain, split):
+        assert torch.equal(a_in, b_in)
+        for x, y in zip(a_blocks, b_blocks):
+            assert torch.equal(x.indptr, y.indptr) and torch.equal(x.indices, y.indices)
     big = _loader(graph)
     big.create_cache(10 * full, sampling_hot)                       # everything fits: CSR moves to the GPU
     assert not big.has_cache and big.indptr.is_cuda and big.indices.is_cuda
@@ -137,7 +146,7 @@ def test_prefetch_and_background_give_the_same_batches(capi, graph, rng_seed):
     base = _collect(_loader(graph, batchsize=100, num_picks=[6, 4, 3], rng_seed=rng_seed))
     assert len(base) == 10
     for kw in (dict(prefetch=3), dict(prefetch=4, background=True), dict(prefetch=1, background=True),
-               dict(prefetch=16)):
+               dict(prefetch=16), dict(indptr_on_device=True), dict(indptr_on_device=True, prefetch=2)):
         dl = _loader(graph, batchsize=100, num_picks=[6, 4, 3], rng_seed=rng_seed, **kw)
         _same_epoch(_collect(dl), base)
         if rng_seed is None:                       # a second epoch over the same loader
