@@ -15,6 +15,13 @@
 //        seed whatever the degree; the reference draws O(deg) numbers per seed
 //        (src/cache_graph_sampling.cu:329-336). k > 64 uses one wave per seed
 //        with the chosen set staged in LDS.
+// hop:   shmt_sample_hop queues plan, pick and the relabel passes of
+//        {seeds, sampled ids} as one sequence. The HOP forms of the kernels
+//        do the relabel's preparation on the side: plan writes the seeds into
+//        the relabel input, pick adds the tile offsets itself (one short
+//        totals kernel instead of two passes over sub_indptr), writes every
+//        sampled id into the relabel input too, empties the relabel table and
+//        marks whether any id falls outside 32 bits.
 #include "common.h"
 #include "hashmap.h"
 #include "hashmap_dev.h"

@@ -168,3 +168,62 @@ def test_background_producer_stops_early_and_reports_errors(capi, graph):
     with pytest.raises(RuntimeError):
         next(iter(bad))
     assert bad._producer is None
+
+
+def test_end_to_end_batch_full_size(capi):
+    """The end-to-end configuration at full size: R-MAT scale 24 (16.8 M nodes, 521 M edges), top 20 % of the
+    adjacency cached, features 16,777,216 x 256 f32 (17.2 GB) pinned with the top-degree 25 % cached, batches of
+    4,096 seeds with fanouts [25, 15, 10] through the dataloader, then the features of the input nodes.
+    Checked by properties: block shapes chain, destination nodes are a prefix of source nodes, every block
+    edge is an edge of the graph, fetched features equal index_select. Skipped when the features cannot be pinned."""
+    import shmtensor
+    from shmtensor_amd.synthetic import rmat_csr
+    indptr_d, indices_d = rmat_csr(24, 16, seed=3)
+    n, dim = indptr_d.numel() - 1, 256
+    try:
+        feats = torch.empty((n, dim), dtype=torch.float32, pin_memory=True)
+    except RuntimeError as exc:
+        pytest.skip("cannot pin 17.2 GB here: %s" % str(exc)[:80])
+    g = torch.Generator(device="cuda").manual_seed(3)
+    for lo in range(0, n, 2_000_000):
+        hi = min(n, lo + 2_000_000)
+        feats[lo:hi].copy_(torch.randn((hi - lo, dim), device="cuda", generator=g))
+    torch.cuda.synchronize()
+    deg = indptr_d[1:] - indptr_d[:-1]
+    by_degree = torch.sort(deg, descending=True, stable=True).indices
+    hot_feat = by_degree[: n // 4].contiguous()
+    feat_cache = capi.uva_fetch(feats, hot_feat)
+    feat_map = capi.CUCOStaticHashmap(hot_feat, torch.arange(hot_feat.numel(), device="cuda"), 0.8)
+    seeds = torch.randperm(n, generator=torch.Generator().manual_seed(55))[: 3 * 4096]
+    dl = shmtensor.GPUSamplingDataloader(indptr_d.cpu(), indices_d.cpu(), seeds, 4096, [25, 15, 10], shuffle=False,
+                                         rng_seed=7, prefetch=3)
+    hot_adj = by_degree[: n // 5].contiguous()
+    dl.gpu_indptr, dl.gpu_indices = capi.create_subcsr(dl.indptr, dl.indices, hot_adj)
+    dl.hashmap = capi.CUCOStaticHashmap(hot_adj, torch.arange(hot_adj.numel(), device="cuda"), 0.8)
+    dl.has_cache = True
+    batches = 0
+    for input_nodes, output_nodes, blocks in dl:
+        assert output_nodes.numel() == 4096 and len(blocks) == 3
+        assert blocks[-1].num_dst == 4096 and blocks[0].num_src == input_nodes.numel()
+        assert blocks[0].num_dst == blocks[1].num_src and blocks[1].num_dst == blocks[2].num_src
+        assert torch.equal(input_nodes[:4096], output_nodes)                 # seeds stay first through every hop
+        # the innermost block (fanout 25 on the widest frontier): every edge (dst -> src) is an edge of the graph
+        blk = blocks[0]
+        counts = blk.indptr[1:] - blk.indptr[:-1]
+        dst = input_nodes[: blk.num_dst]
+        assert torch.equal(counts, torch.clamp(deg[dst], max=25))
+        owner = torch.repeat_interleave(dst, counts)
+        nbr = input_nodes[blk.indices]
+        first = indptr_d[owner]
+        # neighbours are sorted within a row: locate each sampled one by bisection inside its row
+        lo, hi = first.clone(), indptr_d[owner + 1].clone()
+        for _ in range(32):
+            mid = (lo + hi) // 2
+            go_right = (indices_d[mid.clamp(max=indices_d.numel() - 1)].long() < nbr) & (lo < hi)
+            lo = torch.where(go_right, mid + 1, lo)
+            hi = torch.where(go_right, hi, mid)
+        assert bool((indices_d[lo.clamp(max=indices_d.numel() - 1)].long() == nbr).all())
+        x = capi.cache_fetch(feats, feat_cache, input_nodes, feat_map)
+        assert torch.equal(x.cpu(), torch.index_select(feats, 0, input_nodes.cpu()))
+        batches += 1
+    assert batches == 3

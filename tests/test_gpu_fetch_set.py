@@ -223,6 +223,50 @@ def test_sliced_tables_and_grid_stride(capi):
     assert torch.equal(gpu_big[1:], upd) and torch.equal(capi.uva_fetch(data, ids).cpu(), data[ids.cpu()])
 
 
+def test_large_skewed_fetch_full_size(capi):
+    """The large fetch configuration at its full size: 100,000,000 x 128 fp16 rows (25.6 GB) pinned, the
+    40,000,000 lowest ids cached in HBM, 1,048,576 Zipf(1.1) queries. Cached rows are made to differ from
+    their host copies (sign bit flipped), so the result shows which table every row came from; then the set
+    pass over 262,144 cached rows. Skipped when the machine cannot pin the table."""
+    from shmtensor_amd.synthetic import zipf_ranks
+    n, c, d = 100_000_000, 40_000_000, 128
+    try:
+        table = torch.empty((n, d), dtype=torch.float16, pin_memory=True)
+    except RuntimeError as exc:
+        pytest.skip("cannot pin 25.6 GB here: %s" % str(exc)[:80])
+    g = torch.Generator(device="cuda").manual_seed(2)
+    cache = torch.empty((c, d), dtype=torch.float16, device="cuda")
+    chunk = 4_000_000
+    for lo in range(0, n, chunk):
+        part = torch.randn((chunk, d), device="cuda", generator=g).to(torch.float16)
+        table[lo:lo + chunk].copy_(part)
+        if lo < c:
+            cache[lo:lo + chunk] = -part                  # distinguishable from the host copy, bit-exactly invertible
+    torch.cuda.synchronize()
+    del part
+    keys = torch.arange(c, device="cuda")
+    h = capi.CUCOStaticHashmap(keys, keys, 0.8)
+    assert h.capacity() == 50_000_000
+    q = zipf_ranks(1 << 20, n, 1.1, seed=100)
+    hit = q < c
+    assert 0.97 < float(hit.float().mean()) < 0.99 and int((~hit).sum()) > 10_000
+    out = capi.cache_fetch(table, cache, q, h)
+    expect = torch.index_select(table, 0, q.cpu()).cuda()
+    expect = torch.where(hit[:, None], -expect, expect)
+    assert torch.equal(out.view(torch.int16), expect.view(torch.int16))
+    assert torch.equal(capi.cache_fetch_with_mask(table, cache, q, h.query(q)).view(torch.int16), expect.view(torch.int16))
+    del out, expect
+    rows = torch.randperm(c, device="cuda", generator=g)[:262_144].contiguous()
+    upd = torch.randn((262_144, d), device="cuda", generator=g).to(torch.float16)
+    host_before = torch.index_select(table, 0, rows.cpu())
+    capi.cache_set(table, cache, rows, upd, h)
+    assert torch.equal(capi.cache_fetch(table, cache, rows, h).view(torch.int16), upd.view(torch.int16))
+    assert torch.equal(torch.index_select(table, 0, rows.cpu()).view(torch.int16), host_before.view(torch.int16))
+    capi.cache_set(table, cache, rows, upd, h, write_through=True)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.index_select(table, 0, rows.cpu()).view(torch.int16), upd.cpu().view(torch.int16))
+
+
 def test_large_skewed_fetch_scaled(capi):
     """The large fetch configuration at 1/25 scale: 4,000,000 x 128 fp16 rows pinned, the
     1,600,000 lowest ids cached, 1,048,576 Zipf(1.1) queries; then a set pass over 262,144

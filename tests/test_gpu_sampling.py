@@ -205,3 +205,41 @@ def test_rmat_three_hop_pipeline(capi, oracle):
         total_edges += si.numel()
         seeds, ref_seeds = u, eu
     assert total_edges > 50_000
+
+
+def test_config3_full_size_properties(capi):
+    """Configuration 3 at full size (R-MAT scale 21, 116 M edges, top 30 % of rows cached, 1,024 seeds,
+    fanouts [15, 10, 5] in the dataloader's order): properties that need no CPU pass over the graph.
+    Counts are min(k, degree); every sampled id is a neighbour of its seed, without repeats; the cache is
+    transparent; the fused hop equals the separate operators; relabel inverts and keeps the seeds first."""
+    from shmtensor_amd.synthetic import rmat_csr
+    indptr_d, indices_d = rmat_csr(21, 30, seed=1)
+    n = indptr_d.numel() - 1
+    indptr, indices = indptr_d.cpu().pin_memory(), indices_d.cpu().pin_memory()
+    deg = indptr_d[1:] - indptr_d[:-1]
+    hot = torch.sort(deg, descending=True, stable=True).indices[: n * 3 // 10].contiguous()
+    gp, gi = capi.create_subcsr(indptr, indices, hot)
+    h = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel(), device="cuda"), 0.8)
+    # every edge as one sorted key (rows ascending, neighbours sorted within a row)
+    rows = torch.repeat_interleave(torch.arange(n, device="cuda"), deg)
+    edge_keys = rows * n + indices_d.long()
+    del rows
+    seeds = torch.randperm(n, device="cuda", generator=torch.Generator(device="cuda").manual_seed(33))[:1024]
+    for hop, k in enumerate([5, 10, 15]):
+        sp, si = capi.csr_cache_sampling(indptr, indices, gp, gi, h, seeds, k, False, seed=7777, stream_id=hop)
+        assert torch.equal(sp[1:] - sp[:-1], torch.clamp(deg[seeds], max=k))
+        owner = torch.repeat_interleave(seeds, sp[1:] - sp[:-1])
+        keys = owner * n + si.long()
+        pos = torch.searchsorted(edge_keys, keys)
+        assert bool((edge_keys[pos.clamp(max=edge_keys.numel() - 1)] == keys).all())      # real neighbours
+        slot = torch.repeat_interleave(torch.arange(seeds.numel(), device="cuda"), sp[1:] - sp[:-1])
+        assert torch.unique(slot * n + si.long()).numel() == si.numel()                    # no repeats in a row
+        sp2, si2 = capi.csr_sampling(indptr, indices, seeds, k, False, seed=7777, stream_id=hop)
+        assert torch.equal(sp, sp2) and torch.equal(si, si2)                               # cache is transparent
+        u, (ls, ln) = capi.tensor_relabel([seeds, si])
+        fsp, fsi, fu, fl = capi.sample_hop(indptr, indices, gp, gi, h, seeds, k, False, seed=7777, stream_id=hop)
+        assert torch.equal(fsp, sp) and torch.equal(fsi, si) and torch.equal(fu, u) and torch.equal(fl, ln)
+        assert torch.equal(u[: seeds.numel()], seeds) and torch.equal(u[ln], si.long())
+        assert u.numel() == torch.unique(torch.cat([seeds, si.long()])).numel()
+        seeds = u
+    assert seeds.numel() > 100_000
