@@ -89,6 +89,26 @@ def test_relabel_id_ranges_select_the_table_format(capi, oracle, n, odd):
     assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
 
 
+def test_relabel_is_shift_invariant_across_table_formats(capi):
+    """relabel(x + 2^40) must give the labels of relabel(x) and the shifted unique list: the first call
+    runs on 16-byte slots, the second on packed slots, over many sizes and repetition patterns."""
+    g = torch.Generator(device="cuda").manual_seed(21)
+    shift = 1 << 40
+    for case in range(40):
+        n = int(torch.randint(1, 2_000_000 if case % 4 == 0 else 60_000, (1,), generator=g, device="cuda"))
+        span = [3, 50, n // 8 + 1, n, 4 * n, 2**32][case % 6]
+        x = torch.randint(0, span, (n,), generator=g, device="cuda")
+        if case % 5 == 0:                      # hub-like skew: a few ids take most positions
+            hubs = torch.randint(0, 7, (n,), generator=g, device="cuda")
+            x = torch.where(torch.rand(n, generator=g, device="cuda") < 0.7, hubs, x)
+        split = int(torch.randint(0, n + 1, (1,), generator=g, device="cuda"))
+        u0, (a0, b0) = capi.tensor_relabel([x[:split], x[split:]])
+        u1, (a1, b1) = capi.tensor_relabel([x[:split] + shift, x[split:] + shift])
+        assert torch.equal(u0 + shift, u1), case
+        assert torch.equal(a0, a1) and torch.equal(b0, b1), case
+        assert torch.equal(u0[torch.cat([a0, b0])], x), case
+
+
 def test_relabel_mixed_dtypes_prefix_property(capi, oracle):
     # the dataloader's call: [int64 seeds, int32 sub_indices] (python/shmtensor/sampling.py:137-138)
     rng = np.random.default_rng(5)
