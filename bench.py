@@ -254,6 +254,15 @@ def bench_fetch(capi, args, result):
             "sample": "%d passes of one 1,048,576-query Zipf batch over the same host table (oracle gather, "
                       "OpenMP); torch.index_select with %d threads on the same batch: %.2f GB/s"
                       % (reps, torch.get_num_threads(), Q * R / torch_t / 1e9)}
+        # CPU set: the reference's cpu_data[idx] = update idiom (example/test_cache_set.py:183-184)
+        sidx_cpu, upd_cpu = sidx.cpu(), upd.cpu()
+        host[sidx_cpu] = upd_cpu
+        t1 = time.perf_counter()
+        for _ in range(5):
+            host[sidx_cpu] = upd_cpu
+        set_t = (time.perf_counter() - t1) / 5
+        extra["cache_set_262144"]["cpu_index_put_ms"] = round(set_t * 1e3, 3)
+        extra["cache_set_262144"]["cpu_threads"] = torch.get_num_threads()
     del host, cache, hmap
 
 
