@@ -718,6 +718,7 @@ std::vector<std::vector<HopResult>> sample_blocks(
             out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b));
         } catch (...) {
           failures[j] = std::current_exception();
+          next_batch = B;  // the call will fail: the other workers stop after their current batch
         }
       });
     }
