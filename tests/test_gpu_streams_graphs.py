@@ -65,3 +65,46 @@ def test_fetch_query_and_set_replay_in_a_hip_graph(capi, cache):
         assert torch.equal(static_out, expect), it
         assert torch.equal(static_slots, slot), it
         assert float(static_out.abs().sum()) > 0
+
+
+def test_fused_hop_replays_in_a_hip_graph(capi, cabi):
+    """shmt_sample_hop never waits for the host (sizes go to device memory here), so the whole hop can be
+    captured once and replayed on new seeds: every replay is compared with the eager operator, with eager
+    work and synchronisations in between. One replay feeds ids beyond 32 bits (the relabel then switches
+    table format inside the captured kernels) and the next goes back."""
+    from shmtensor_amd.synthetic import rmat_csr
+    lib = cabi.load()
+    indptr, indices = rmat_csr(13, 12, seed=3)
+    indices = indices.long()
+    n = indptr.numel() - 1
+    S, k = 3000, 8
+    n_max = S + S * k
+    seeds = torch.zeros(S, dtype=torch.int64, device="cuda")
+    graph_indices = indices.clone()
+    buf = dict(sp=torch.empty(S + 1, dtype=torch.int64, device="cuda"), si=torch.empty(S * k, dtype=torch.int64, device="cuda"),
+               plan=torch.empty(lib.shmt_sample_plan_bytes(S), dtype=torch.uint8, device="cuda"),
+               total=torch.empty(n_max, dtype=torch.int64, device="cuda"), unique=torch.empty(n_max, dtype=torch.int64, device="cuda"),
+               labels=torch.empty(n_max, dtype=torch.int64, device="cuda"),
+               scratch=torch.empty(lib.shmt_relabel_scratch_bytes(n_max), dtype=torch.uint8, device="cuda"),
+               nnz=torch.zeros(1, dtype=torch.int64, device="cuda"), count=torch.zeros(1, dtype=torch.int64, device="cuda"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cabi.check(lib.shmt_sample_hop(indptr.data_ptr(), 8, graph_indices.data_ptr(), 8, None, None, None, seeds.data_ptr(), 8,
+                                       S, k, 0, 5, 2, buf["sp"].data_ptr(), buf["si"].data_ptr(), buf["plan"].data_ptr(),
+                                       buf["plan"].numel(), 8, buf["total"].data_ptr(), buf["scratch"].data_ptr(),
+                                       buf["scratch"].numel(), buf["unique"].data_ptr(), buf["labels"].data_ptr(),
+                                       buf["nnz"].data_ptr(), buf["count"].data_ptr(), cabi.current_stream()))
+    g = torch.Generator().manual_seed(12)
+    for it in range(5):
+        seeds.copy_(torch.randperm(n, generator=g)[:S])
+        graph_indices.copy_(indices)
+        if it == 2:
+            graph_indices[::3] += 1 << 33          # ids that need the 16-byte table format
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = capi.sample_hop(indptr, graph_indices, None, None, None, seeds, k, False, seed=5, stream_id=2)
+        nnz, u = int(buf["nnz"].item()), int(buf["count"].item())
+        assert nnz == want[1].numel() and u == want[2].numel(), it
+        assert torch.equal(buf["sp"], want[0]) and torch.equal(buf["si"][:nnz], want[1]), it
+        assert torch.equal(buf["unique"][:u], want[2]) and torch.equal(buf["labels"][S:S + nnz], want[3]), it
