@@ -1,0 +1,28 @@
+"""Common part of the host tensor providers: an object that owns some mapping
+of host memory (a shared-memory segment, a memory-mapped file), exposes it as
+`tensor_` and forwards the usual read-only tensor attributes to it. The
+mapping is released by a finalizer that holds only plain values, never the
+object or its tensor."""
+import math
+import weakref
+
+import torch
+
+
+class HostTensorView:
+    tensor_ = None
+
+    def _adopt(self, tensor, release, *release_args):
+        """Install `tensor` as the view and arrange for `release(*release_args)`
+        to run once when this object goes away (or at interpreter exit)."""
+        self.tensor_ = tensor
+        self._finalizer = weakref.finalize(self, release, *release_args)
+
+    shape = property(lambda self: self.tensor_.shape)
+    dtype = property(lambda self: self.tensor_.dtype)
+    device = property(lambda self: self.tensor_.device)
+    size = property(lambda self: self.tensor_.size)
+
+
+def tensor_nbytes(shape, dtype):
+    return math.prod(int(d) for d in shape) * torch.empty(0, dtype=dtype).element_size()
