@@ -190,13 +190,13 @@ def bench_fetch(capi, args, result):
     # streaming ceiling of the same kernel: sequential ids on the HBM table (a plain copy)
     qs = torch.arange(Q, device="cuda")
     t = gpu_time_ms(lambda: capi.uva_fetch(cache, qs), 30)
-    extra["sequential_copy_same_kernel"] = {"ms": round(t["median"], 4),
+    extra["sequential_copy_same_kernel"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4),
                                             "algorithmic_GBs": round(algo_bytes / t["median"] / 1e6, 1)}
     # all-hit: uniform queries over the cached ids (no locality), HBM bound
     qh = torch.randint(0, C, (Q,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
     t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qh, hmap), 30)
     a = algo_bytes / (t["median"] * 1e-3) / 1e9
-    extra["fetch_all_hit"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(a, 1),
+    extra["fetch_all_hit"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "algorithmic_GBs": round(a, 1),
                               "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 1)}
     tm = gpu_time_ms(lambda: capi.cache_fetch_with_mask(host, cache, qh, qh), 30)
     a = algo_bytes / (tm["median"] * 1e-3) / 1e9
@@ -206,11 +206,11 @@ def bench_fetch(capi, args, result):
     qm = torch.randint(C, N, (Q,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
     t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qm, hmap), 10)
     m = Q * R / (t["median"] * 1e-3) / 1e9
-    extra["fetch_all_miss"] = {"ms": round(t["median"], 4), "host_link_GBs": round(m, 2),
+    extra["fetch_all_miss"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "host_link_GBs": round(m, 2),
                                "frac_of_pinned_copy": round(m / h2d, 4)}
     t = gpu_time_ms(lambda: capi.uva_fetch(host, qm), 10)
     m = Q * R / (t["median"] * 1e-3) / 1e9
-    extra["uva_fetch"] = {"ms": round(t["median"], 4), "host_link_GBs": round(m, 2),
+    extra["uva_fetch"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "host_link_GBs": round(m, 2),
                           "frac_of_pinned_copy": round(m / h2d, 4)}
 
     # cache_set pass of config 4: 262,144 unique cached rows
@@ -220,7 +220,7 @@ def bench_fetch(capi, args, result):
     t = gpu_time_ms(lambda: capi.cache_set(host, cache, sidx, upd, hmap), 30)
     assert torch.equal(capi.cache_fetch(host, cache, sidx, hmap), upd)
     a = ns * (2 * R + 8) / (t["median"] * 1e-3) / 1e9
-    extra["cache_set_262144"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(a, 1),
+    extra["cache_set_262144"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "algorithmic_GBs": round(a, 1),
                                  "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
 
     # scatter to the host table over the link (all misses): 262,144 uncached rows
@@ -228,7 +228,7 @@ def bench_fetch(capi, args, result):
     t = gpu_time_ms(lambda: capi.cache_set(host, cache, sm, upd, hmap), 10)
     torch.cuda.synchronize()
     assert torch.equal(host[sm[:64].cpu()].view(torch.int16), upd[:64].cpu().view(torch.int16))
-    extra["cache_set_all_miss_262144"] = {"ms": round(t["median"], 4),
+    extra["cache_set_all_miss_262144"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4),
                                           "host_link_write_GBs": round(ns * R / t["median"] / 1e6, 2)}
 
     # CPU baseline: the reference's cpu_fetch idiom is data[query.cpu()] (example/test_cache_fetch.py:138);
@@ -291,7 +291,7 @@ def bench_fetch_small(capi, args, result):
     res = {"hit_rate": round(hit, 4)}
     for name, qq in (("as_specified", q), ("all_hit", q_hit), ("all_miss", q_miss)):
         t = gpu_time_ms(lambda: capi.cache_fetch(table, cache, qq, hmap), 30)
-        res[name] = {"ms": round(t["median"], 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 2),
+        res[name] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 2),
                      "algorithmic_GBs": round(Q * (2 * R + 8) / t["median"] / 1e6, 1)}
     if not args.no_cpu:
         qc = q.cpu()
