@@ -8,7 +8,7 @@
 //            distinct id of the tile (64-bit CAS on the key, atomicMin the index)
 //   first    first[i] = smallest index holding the same key (kept in the
 //            labels buffer); per-tile count of i with first[i] == i
-//   partials exclusive scan of the per-tile counts (own launch only beyond 4 M ids)
+//   partials exclusive scan of the per-tile counts (own launch only beyond 1 M ids)
 //   unique   rank of every first occurrence; unique[rank] = key; rank_of[i]
 //   labels   labels[i] = rank_of[first[i]]
 // The table is touched only by `insert` and `first`; the last two passes read
@@ -27,7 +27,7 @@ namespace shmt {
 constexpr int kRlBlock = 256;
 constexpr int kRlItems = 2;
 constexpr int kRlTile = kRlBlock * kRlItems;
-constexpr int64_t kRlSelfPrefixTiles = 2048;  // up to 4 M ids the unique pass sums the tile counts itself
+constexpr int64_t kRlSelfPrefixTiles = 2048;  // up to 1 M ids the unique pass sums the tile counts itself
 
 // Number of input ids: a host-known part plus, optionally, a part that only
 // the device knows (the length of the last segment, e.g. the nnz a sampling
