@@ -503,10 +503,12 @@ struct CsrArgs {
   torch::Tensor indptr, indices;
   std::optional<torch::Tensor> gpu_indptr, gpu_indices;
   StaticHashmap *hashmap;
+  // what the kernels dereference for indptr / indices (translated once per call, not once per hop)
+  void *indptr_dev = nullptr, *indices_dev = nullptr;
   bool cached() const { return hashmap != nullptr; }
 };
 
-void check_csr(const CsrArgs &g) {
+void check_csr(CsrArgs &g) {
   TORCH_CHECK(!g.cached() || (g.gpu_indptr.has_value() && g.gpu_indices.has_value()),
               "sample_hop: a hashmap needs gpu_indptr and gpu_indices");
   id_bytes(g.indptr, "indptr");
@@ -520,6 +522,8 @@ void check_csr(const CsrArgs &g) {
                     g.gpu_indices->scalar_type() == g.indices.scalar_type(),
                 "cached CSR must have the dtypes of the full CSR");
   }
+  g.indptr_dev = device_address(g.indptr, "indptr");
+  g.indices_dev = device_address(g.indices, "indices");
 }
 
 // A hop whose kernels are queued on the stream that was current when it was
@@ -583,7 +587,7 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   char *const scratch_ptr = total_ptr + aligned(total_bytes);
   h.nnz_slot = readback().acquire();
   h.count_slot = readback().acquire();
-  check(shmt_sample_hop(device_address(g.indptr, "indptr"), pb, device_address(g.indices, "indices"), ib,
+  check(shmt_sample_hop(g.indptr_dev, pb, g.indices_dev, ib,
                         g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
                         g.cached() ? g.gpu_indices->data_ptr() : nullptr,
                         g.cached() ? g.hashmap->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks,
@@ -615,7 +619,7 @@ HopResult sample_hop(torch::Tensor indptr, torch::Tensor indices,
                      std::optional<torch::Tensor> gpu_indptr, std::optional<torch::Tensor> gpu_indices,
                      StaticHashmap *hashmap, torch::Tensor seeds, int64_t num_picks, bool replace,
                      std::optional<int64_t> seed, int64_t stream_id) {
-  const CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
   check_csr(g);
   PendingHop h = hop_issue(g, seeds, num_picks, replace, seed, stream_id);
   return hop_finish(h);
@@ -674,7 +678,7 @@ std::vector<std::vector<HopResult>> sample_blocks(
     std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, std::vector<torch::Tensor> seeds,
     std::vector<int64_t> num_picks, bool replace, std::optional<std::vector<int64_t>> seeds_rng,
     int64_t max_in_flight) {
-  const CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
   check_csr(g);
   const int64_t B = static_cast<int64_t>(seeds.size());
   TORCH_CHECK(!seeds_rng.has_value() || static_cast<int64_t>(seeds_rng->size()) == B,
