@@ -214,86 +214,54 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
   }
 }
 
-// First-occurrence index of every element. The first-slot loads of a
-// thread's eight elements are issued together; only the rare longer probe
-// chains continue one by one.
+// First-occurrence index of every element: one id per thread, a workgroup of
+// kRlTile threads per tile (the tile whose count of first occurrences the
+// unique pass ranks). One id per thread keeps every value in registers and
+// every probe chain in its own lane; with several ids per thread the chains of
+// a lane ran one after the other and a small input ran on a handful of
+// workgroups.
 template <bool PACKED>
-__device__ __forceinline__ uint64_t rl_first_tile(const RlSlot *tbl, uint32_t cap, const void *total,
-                                                  int eb, int64_t N, void *labels) {
-  const unsigned long long *tbl8 = reinterpret_cast<const unsigned long long *>(tbl);
-  const uint32_t cap8 = rl_cap8(cap);
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * kRlTile;
-  int64_t key[kRlItems], idx[kRlItems];
-  bool ok[kRlItems];
-  uint32_t pos[kRlItems];
-  uint4 slot[PACKED ? 1 : kRlItems];
-  unsigned long long slot8[PACKED ? kRlItems : 1];
-#pragma unroll
-  for (int j = 0; j < kRlItems; ++j) {
-    idx[j] = base + j * kRlBlock + threadIdx.x;
-    ok[j] = idx[j] < N;
-    key[j] = -1;
-  }
-  load_ints<kRlItems>(total, idx, ok, eb, key);
-#pragma unroll
-  for (int j = 0; j < kRlItems; ++j)
-    pos[j] = PACKED ? rl_home8(static_cast<uint32_t>(key[j]), cap8) : reduce_range(hash_id(key[j]), cap);
-#pragma unroll
-  for (int j = 0; j < kRlItems; ++j) {
-    if (PACKED)
-      slot8[j] = tbl8[pos[j]];
-    else
-      slot[j] = *reinterpret_cast<const uint4 *>(&tbl[pos[j]]);
-  }
-  uint64_t cnt = 0;
-#pragma unroll
-  for (int j = 0; j < kRlItems; ++j) {
-    const int64_t i = idx[j];
-    if (i < N) {
-      uint32_t p = pos[j];
-      uint32_t f = 0xFFFFFFFFu;
-      if (PACKED) {
-        const uint32_t key32 = static_cast<uint32_t>(key[j]);
-        unsigned long long s8 = slot8[j];
-        for (uint32_t probes = 0; probes < cap8; ++probes) {
-          if (static_cast<uint32_t>(s8 >> 32) == key32 && s8 != kRlEmpty8) {
-            f = static_cast<uint32_t>(s8);
-            break;
-          }
-          if (s8 == kRlEmpty8) break;
-          p = (p + 1 == cap8) ? 0 : p + 1;
-          s8 = tbl8[p];
-        }
-      } else {
-        uint4 s = slot[j];
-        for (uint32_t probes = 0; probes < cap; ++probes) {
-          const int64_t k = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
-          if (k == key[j]) {
-            f = s.z;
-            break;
-          }
-          if (k == -1) break;
-          p = (p + 1 == cap) ? 0 : p + 1;
-          s = *reinterpret_cast<const uint4 *>(&tbl[p]);
-        }
-      }
-      store_int(labels, i, eb, static_cast<int64_t>(f));
-      cnt += (f == static_cast<uint32_t>(i));
+__device__ __forceinline__ uint32_t rl_first_of(const RlSlot *tbl, uint32_t cap, int64_t key) {
+  if (PACKED) {
+    const unsigned long long *tbl8 = reinterpret_cast<const unsigned long long *>(tbl);
+    const uint32_t cap8 = rl_cap8(cap);
+    const uint32_t key32 = static_cast<uint32_t>(key);
+    uint32_t p = rl_home8(key32, cap8);
+    for (uint32_t probes = 0; probes < cap8; ++probes) {
+      const unsigned long long s8 = tbl8[p];
+      if (s8 == kRlEmpty8) break;
+      if (static_cast<uint32_t>(s8 >> 32) == key32) return static_cast<uint32_t>(s8);
+      p = (p + 1 == cap8) ? 0 : p + 1;
+    }
+  } else {
+    uint32_t p = reduce_range(hash_id(key), cap);
+    for (uint32_t probes = 0; probes < cap; ++probes) {
+      const uint4 s = *reinterpret_cast<const uint4 *>(&tbl[p]);
+      const int64_t k = static_cast<int64_t>((static_cast<uint64_t>(s.y) << 32) | s.x);
+      if (k == key) return s.z;
+      if (k == -1) break;
+      p = (p + 1 == cap) ? 0 : p + 1;
     }
   }
-  return cnt;
+  return 0xFFFFFFFFu;
 }
 
-__global__ __launch_bounds__(kRlBlock) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
-                                                            const void *total, int eb, RlCount n,
-                                                            void *labels, uint64_t *partials,
-                                                            RlPath path) {
+__global__ __launch_bounds__(kRlTile) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
+                                                           const void *total, int eb, RlCount n,
+                                                           void *labels, uint64_t *partials,
+                                                           RlPath path) {
   const int64_t N = rl_count(n);
-  __shared__ uint64_t lds[kRlBlock / kWave];
-  const uint64_t cnt = rl_packed(path) ? rl_first_tile<true>(tbl, cap, total, eb, N, labels)
-                                       : rl_first_tile<false>(tbl, cap, total, eb, N, labels);
+  __shared__ uint64_t lds[kRlTile / kWave];
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kRlTile + threadIdx.x;
+  uint64_t cnt = 0;
+  if (i < N) {
+    const int64_t key = load_int(total, i, eb);
+    const uint32_t f = rl_packed(path) ? rl_first_of<true>(tbl, cap, key) : rl_first_of<false>(tbl, cap, key);
+    store_int(labels, i, eb, static_cast<int64_t>(f));
+    cnt = (f == static_cast<uint32_t>(i));
+  }
   uint64_t tile_total;
-  block_exclusive_scan<uint64_t, kRlBlock>(cnt, lds, &tile_total);
+  block_exclusive_scan<uint64_t, kRlTile>(cnt, lds, &tile_total);
   if (threadIdx.x == 0) partials[blockIdx.x] = tile_total;
 }
 
@@ -475,7 +443,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   hipLaunchKernelGGL(rl_insert_kernel, dim3(grid_for(N, kRlInsertTile, 256 * 32)), dim3(kRlBlock), 0,
                      s, tbl, cap, total, elem_bytes, n, path);
   SHMT_LAUNCH_CHECK();
-  hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, tbl,
+  hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlTile), 0, s, tbl,
                      cap, total, elem_bytes, n, labels_out, partials, path);
   SHMT_LAUNCH_CHECK();
   const int scanned = nb > kRlSelfPrefixTiles;
