@@ -49,6 +49,18 @@ struct RowArgs {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+// Table rows are addressed through integers that travelled across lanes, so
+// the compiler cannot tell that they point to global memory; saying so turns
+// generic (flat) accesses into global ones.
+template <typename VT>
+__device__ __forceinline__ VT gload(const char *p) {
+  return *reinterpret_cast<const VT __attribute__((address_space(1))) *>(reinterpret_cast<uintptr_t>(p));
+}
+template <typename VT>
+__device__ __forceinline__ void gstore(char *p, VT v) {
+  *reinterpret_cast<VT __attribute__((address_space(1))) *>(reinterpret_cast<uintptr_t>(p)) = v;
+}
+
 constexpr int kRowsBlock = 256;    // threads per workgroup
 constexpr int kRowsWavesPerSimd = 8;  // register budget: 512 / 8 = 64 VGPRs
 constexpr int kRowsInFlight = 2;   // rows a lane group moves concurrently (single-vector rows)
@@ -118,7 +130,7 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
               v[u] = __builtin_nontemporal_load(
                   reinterpret_cast<const VT *>(a.dense + (base + row) * R + my_off));
             else
-              v[u] = *reinterpret_cast<const VT *>(trow[u] + my_off);
+              v[u] = gload<VT>(trow[u] + my_off);
           }
         }
 #pragma unroll
@@ -126,8 +138,8 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
           const int row = r0 + u * rows_per_step + grp;
           if (row < nrows && in) {
             if (SET) {
-              *reinterpret_cast<VT *>(trow[u] + my_off) = v[u];
-              if (THROUGH && second[u]) *reinterpret_cast<VT *>(second[u] + my_off) = v[u];
+              gstore<VT>(trow[u] + my_off, v[u]);
+              if (THROUGH && second[u]) gstore<VT>(second[u] + my_off, v[u]);
             } else
               __builtin_nontemporal_store(
                   v[u], reinterpret_cast<VT *>(a.dense + (base + row) * R + my_off));
@@ -146,20 +158,20 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
         char *dst = SET ? trow : drow;
         int64_t off = my_off;
         for (; off + 3 * step < R; off += 4 * step) {
-          const VT v0 = *reinterpret_cast<const VT *>(src + off);
-          const VT v1 = *reinterpret_cast<const VT *>(src + off + step);
-          const VT v2 = *reinterpret_cast<const VT *>(src + off + 2 * step);
-          const VT v3 = *reinterpret_cast<const VT *>(src + off + 3 * step);
-          *reinterpret_cast<VT *>(dst + off) = v0;
-          *reinterpret_cast<VT *>(dst + off + step) = v1;
-          *reinterpret_cast<VT *>(dst + off + 2 * step) = v2;
-          *reinterpret_cast<VT *>(dst + off + 3 * step) = v3;
+          const VT v0 = gload<VT>(src + off);
+          const VT v1 = gload<VT>(src + off + step);
+          const VT v2 = gload<VT>(src + off + 2 * step);
+          const VT v3 = gload<VT>(src + off + 3 * step);
+          gstore<VT>(dst + off, v0);
+          gstore<VT>(dst + off + step, v1);
+          gstore<VT>(dst + off + 2 * step, v2);
+          gstore<VT>(dst + off + 3 * step, v3);
         }
         for (; off < R; off += step)
-          *reinterpret_cast<VT *>(dst + off) = *reinterpret_cast<const VT *>(src + off);
+          gstore<VT>(dst + off, gload<VT>(src + off));
         if (THROUGH && second) {
           for (off = my_off; off < R; off += step)
-            *reinterpret_cast<VT *>(second + off) = *reinterpret_cast<const VT *>(src + off);
+            gstore<VT>(second + off, gload<VT>(src + off));
         }
       }
     }
