@@ -531,6 +531,24 @@ def bench_e2e(capi, args, result):
     torch.cuda.synchronize()
     wall_fused = time.perf_counter() - w0
     assert torch.equal(inp_f, inp), "fused hops gave different input nodes"
+    # the same again with the feature fetch queued behind the last relabel (row count read on the device)
+    rng = [7777 + b for b in range(nbatch)]
+    picks = list(reversed(fanouts))
+    cap = int(1.25 * inp.numel())
+    fetched_ms = {}
+    for k_in_flight in (1, 2, 4):
+        capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats, feat_cache,
+                                 feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
+        torch.cuda.synchronize()
+        w0 = time.perf_counter()
+        got = capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats,
+                                       feat_cache, feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
+        torch.cuda.synchronize()
+        fetched_ms[str(k_in_flight)] = round((time.perf_counter() - w0) * 1e3 / nbatch, 3)
+        hops_l, x_l = got[nbatch - 1]
+        assert torch.equal(hops_l[-1][2], inp), "sample_blocks_fetch gave different input nodes"
+        assert torch.equal(x_l, capi.cache_fetch(feats, feat_cache, inp, feat_map)), "sample_blocks_fetch rows differ"
+        del got, hops_l, x_l
     # sampling + relabel only, several batches advancing concurrently
     in_flight_ms = {}
     for k_in_flight in (1, 4, 8):
@@ -575,6 +593,7 @@ def bench_e2e(capi, args, result):
         "batch_ms_wall": round(wall * 1e3 / nbatch, 3), "batches_per_s": round(nbatch / wall, 2),
         "fused_hop_batch_ms_wall": round(wall_fused * 1e3 / nbatch, 3),
         "background_prefetch_batch_ms_wall": round(wall_pipe * 1e3 / nbatch, 3),
+        "sample_blocks_fetch_batch_ms_wall_by_batches_in_flight": fetched_ms,
         "sample_blocks_ms_per_batch_by_batches_in_flight": in_flight_ms,
         "sampled_edges_per_s": round(tot_edges / (t_s * 1e-3), 1),
         "fetch_payload_GBs": round(tot_nodes * D * 4 / (t_f * 1e-3) / 1e9, 2)}

@@ -108,6 +108,25 @@ int shmt_fetch(const void *miss_data, const void *cache_data,
                const void *mask, int mask_bytes, void *out, int64_t Q,
                int64_t row_bytes, void *stream);
 
+/* shmt_fetch for a number of rows that only the GPU knows yet: moves the
+ * first min(max_rows, *count) rows, where `count` is an int64 in device
+ * memory written by earlier work of the stream (count_out of shmt_relabel*
+ * / shmt_sample_hop, with unique_out as `indices`). `indices` (and `mask`)
+ * hold at least that many entries, `out` has room for max_rows rows; rows
+ * past the count are left untouched. If count_seen is not NULL (pinned host
+ * memory) the kernel copies *count there as it starts, so the host learns
+ * the count while the rows are still moving. With this the last relabel of
+ * a mini-batch and the fetch of its input features run back to back without
+ * a host wait between them; the reference reads the count on the host
+ * (src/tensor_relabel.cu:173) before the caller can fetch
+ * (src/cache_feature_fetch.cu:131-185).                                    */
+int shmt_fetch_counted(const void *miss_data, const void *cache_data,
+                       const void *indices, int idx_bytes,
+                       const shmt_hashmap_t *map, const void *mask,
+                       int mask_bytes, void *out, int64_t max_rows,
+                       const int64_t *count, int64_t *count_seen,
+                       int64_t row_bytes, void *stream);
+
 /* Feature set: UVATensorSet src/cache_feature_set.cu:39-75, CacheTensorSet
  * :118-165, CacheTensorSetWithMask :209-248. Mirror of shmt_fetch:
  *   (slot_i >= 0 ? cache_data[slot_i,:] : miss_data[indices[i],:]) = update[i,:]

@@ -38,6 +38,8 @@ struct RowArgs {
   const void *mask;
   MapView map;
   int64_t Q;
+  const int64_t *count;  // when set: only the first min(Q, *count) rows are moved (device memory)
+  int64_t *count_seen;   // when set: receives *count as soon as the kernel starts (pinned host memory)
   int64_t row_bytes;
   int idx_bytes;
   int mask_bytes;
@@ -83,11 +85,20 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
   const int64_t R = a.row_bytes;
   const int64_t step = static_cast<int64_t>(L) * sizeof(VT);
   const int64_t my_off = static_cast<int64_t>(gl) * sizeof(VT);
+  int64_t Q = a.Q;
+  if (a.count) {
+    const int64_t counted = *a.count;
+    if (counted < Q) Q = counted;
+    if (a.count_seen && blockIdx.x == 0 && threadIdx.x == 0) {
+      *a.count_seen = counted;
+      __threadfence_system();
+    }
+  }
 
-  for (int64_t base = wave * tile; base < a.Q; base += nwaves * tile) {
+  for (int64_t base = wave * tile; base < Q; base += nwaves * tile) {
     // ---- phase 1: where does each row of the tile live? ----
     const int64_t i = base + lane;
-    const bool live = lane < tile && i < a.Q;
+    const bool live = lane < tile && i < Q;
     const int64_t idx = live ? load_int(a.indices, i, a.idx_bytes) : 0;
     int64_t slot = -1;
     if (MODE == kMask) {
@@ -102,7 +113,7 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
     // write-through: second destination of a row that hit (0: none)
     const int64_t my_second_row =
         THROUGH && slot >= 0 ? reinterpret_cast<int64_t>(a.miss + idx * R) : 0;
-    const int nrows = static_cast<int>(a.Q - base < tile ? a.Q - base : tile);
+    const int nrows = static_cast<int>(Q - base < tile ? Q - base : tile);
 
     // ---- phase 2: move the rows ----
     if (ONE_VEC) {
@@ -239,7 +250,8 @@ static void launch_vec(bool one_vec, bool through, int mode, unsigned grid, hipS
 template <bool SET>
 static int move_rows(const char *who, void *miss, void *cache, const void *indices, int idx_bytes,
                      const shmt_hashmap_t *map, const void *mask, int mask_bytes, void *dense,
-                     int64_t Q, int64_t row_bytes, void *stream, bool through = false) {
+                     int64_t Q, int64_t row_bytes, void *stream, bool through = false,
+                     const int64_t *count = nullptr, int64_t *count_seen = nullptr) {
   SHMT_REQUIRE(Q >= 0, "%s: Q must be >= 0", who);
   SHMT_REQUIRE(row_bytes > 0, "%s: row_bytes must be > 0", who);
   SHMT_REQUIRE(width_ok(idx_bytes), "%s: ID can only be int32 or int64 (idx_bytes=%d)", who, idx_bytes);
@@ -266,6 +278,8 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   a.mask = mask;
   if (map) a.map = map->view; else a.map = MapView{nullptr, 1, 0};
   a.Q = Q;
+  a.count = count;
+  a.count_seen = count_seen;
   a.row_bytes = row_bytes;
   a.idx_bytes = idx_bytes;
   a.mask_bytes = mask_bytes;
@@ -304,6 +318,16 @@ int shmt_fetch(const void *miss_data, const void *cache_data, const void *indice
   return shmt::move_rows<false>("shmt_fetch", const_cast<void *>(miss_data),
                                 const_cast<void *>(cache_data), indices, idx_bytes, map, mask,
                                 mask_bytes, out, Q, row_bytes, stream);
+}
+
+int shmt_fetch_counted(const void *miss_data, const void *cache_data, const void *indices,
+                       int idx_bytes, const shmt_hashmap_t *map, const void *mask, int mask_bytes,
+                       void *out, int64_t max_rows, const int64_t *count, int64_t *count_seen,
+                       int64_t row_bytes, void *stream) {
+  SHMT_REQUIRE(count != nullptr, "shmt_fetch_counted: count is null");
+  return shmt::move_rows<false>("shmt_fetch_counted", const_cast<void *>(miss_data),
+                                const_cast<void *>(cache_data), indices, idx_bytes, map, mask,
+                                mask_bytes, out, max_rows, row_bytes, stream, false, count, count_seen);
 }
 
 int shmt_set(void *miss_data, void *cache_data, const void *indices, int idx_bytes,

@@ -535,10 +535,15 @@ struct PendingHop {
   torch::Tensor sub_indptr, sub_indices, unique, labels;
   torch::Tensor workspace;                // plan + relabel input + relabel scratch, kept until the sizes are in
   Readback::Slot nnz_slot{}, count_slot{};
+  int64_t *count_dev = nullptr;           // set when the count goes to device memory (see hop_issue)
 };
 
+// With `count_on_device` the number of unique ids is written to device memory
+// (h.count_dev) instead of the host slot, for a kernel queued behind the hop
+// to read; that kernel must then forward it to h.count_slot.dev, or
+// hop_finish never sees it (issue_counted_fetch does).
 PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, bool replace,
-                     std::optional<int64_t> seed, int64_t stream_id) {
+                     std::optional<int64_t> seed, int64_t stream_id, bool count_on_device = false) {
   PendingHop h;
   seeds = cuda_ids(seeds, "seeds");
   TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0");
@@ -566,7 +571,8 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   auto aligned = [](int64_t bytes) { return (bytes + 255) & ~int64_t{255}; };
   // Two allocations per hop (the allocator is shared by all host threads that drive
   // batches): one for the four results, which are typed views of it, ...
-  torch::Tensor results = device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) + 2 * aligned(n_max * eb));
+  torch::Tensor results = device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) +
+                                       2 * aligned(n_max * eb) + (count_on_device ? 256 : 0));
   int64_t offset = 0;
   auto carve = [&](int64_t count, int elem, torch::ScalarType type) {
     torch::Tensor t = results.narrow(0, offset, count * elem).view(type);
@@ -577,6 +583,8 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   h.sub_indices = carve(bound, ib, g.indices.scalar_type());
   h.unique = carve(n_max, eb, id_type);
   h.labels = carve(n_max, eb, id_type);
+  if (count_on_device)
+    h.count_dev = reinterpret_cast<int64_t *>(static_cast<char *>(results.data_ptr()) + offset);
   // ... and one for everything that does not outlive the hop
   const int64_t plan_bytes = shmt_sample_plan_bytes(S);
   const int64_t total_bytes = n_max * eb;
@@ -595,7 +603,7 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
                         static_cast<uint32_t>(stream_id), h.sub_indptr.data_ptr(), h.sub_indices.data_ptr(),
                         plan_ptr, plan_bytes, eb, total_ptr, scratch_ptr,
                         scratch_bytes, h.unique.data_ptr(), h.labels.data_ptr(), h.nnz_slot.dev,
-                        h.count_slot.dev, stream));
+                        count_on_device ? h.count_dev : h.count_slot.dev, stream));
   return h;
 }
 
@@ -613,6 +621,65 @@ HopResult hop_finish(PendingHop &h) {
     h.workspace = torch::Tensor();
   }
   return h.result;
+}
+
+// Feature table of the fused "last relabel -> fetch" (sample_blocks_fetch).
+struct FeatureArgs {
+  torch::Tensor uva_data;
+  std::optional<torch::Tensor> gpu_data;
+  StaticHashmap *hashmap;   // null: every row comes from uva_data
+  int64_t max_rows;         // rows of the speculative output; < 0: the hop's bound; 0: do not speculate
+  void *uva_dev = nullptr;
+  bool cached() const { return hashmap != nullptr; }
+};
+
+void check_features(FeatureArgs &f) {
+  TORCH_CHECK(!f.cached() || f.gpu_data.has_value(), "a feature hashmap needs gpu_data");
+  check_tables(f.uva_data, f.cached() ? &*f.gpu_data : nullptr);
+  f.uva_dev = device_address(f.uva_data, "uva_data");
+}
+
+torch::Tensor fetch_rows(const FeatureArgs &f, const torch::Tensor &ids) {
+  return fetch_impl(f.uva_data, f.cached() ? &*f.gpu_data : nullptr, ids, f.hashmap, nullptr);
+}
+
+// Queues the fetch of the rows of the hop's unique ids behind the hop, before
+// the host knows how many there are: the kernel takes the count from device
+// memory and forwards it to the host slot hop_finish waits on. Returns the
+// output sized for `rows` ids (the caller narrows it once the count is in).
+torch::Tensor issue_counted_fetch(const PendingHop &h, const FeatureArgs &f, int64_t rows) {
+  const RowShape rs = row_shape(f.uva_data, rows);
+  torch::Tensor out = torch::empty(rs.out_sizes, f.uva_data.options().device(torch::kCUDA));
+  void *cache_ptr = nullptr;
+  if (f.cached()) cache_ptr = f.gpu_data->numel() > 0 ? f.gpu_data->data_ptr() : out.data_ptr();
+  check(shmt_fetch_counted(f.uva_dev, cache_ptr, h.unique.data_ptr(),
+                           static_cast<int>(h.unique.element_size()),
+                           f.cached() ? f.hashmap->handle() : nullptr, nullptr, 0, out.data_ptr(), rows,
+                           h.count_dev, h.count_slot.dev, rs.row_bytes, current_stream()));
+  return out;
+}
+
+// One hop followed by the fetch of the feature rows of its unique ids. When
+// the speculative output is large enough (the usual case) no host wait
+// separates the relabel from the fetch; otherwise the rows are fetched once
+// the count is known.
+std::pair<HopResult, torch::Tensor> hop_then_fetch(const CsrArgs &g, const FeatureArgs &f,
+                                                   torch::Tensor seeds, int64_t num_picks, bool replace,
+                                                   std::optional<int64_t> seed, int64_t stream_id) {
+  const int64_t row_bytes = row_shape(f.uva_data, 0).row_bytes;
+  const bool speculate = f.max_rows != 0 && row_bytes > 0;
+  PendingHop h = hop_issue(g, seeds, num_picks, replace, seed, stream_id, speculate);
+  if (h.count_dev == nullptr) {  // not speculating, or a degenerate hop that ran unfused
+    HopResult r = hop_finish(h);
+    return {r, fetch_rows(f, std::get<2>(r))};
+  }
+  const int64_t bound = h.unique.numel();
+  const int64_t rows = f.max_rows < 0 ? bound : std::min(bound, f.max_rows);
+  torch::Tensor out = issue_counted_fetch(h, f, rows);
+  HopResult r = hop_finish(h);
+  const int64_t U = std::get<2>(r).numel();
+  if (U <= rows) return {r, out.narrow(0, 0, U)};
+  return {r, fetch_rows(f, std::get<2>(r))};
 }
 
 HopResult sample_hop(torch::Tensor indptr, torch::Tensor indices,
@@ -642,24 +709,38 @@ class CurrentStreamScope {
 
 constexpr int64_t kMaxBatchesInFlight = 32;
 
+struct BatchResult {
+  std::vector<HopResult> hops;
+  torch::Tensor features;  // defined only when features were asked for
+};
+
 // All hops of one batch on the current stream: hop h samples `num_picks[h]`
 // neighbours of the previous hop's unique ids (RNG stream h when a seed is
 // given), as the dataloader's loop does (python/shmtensor/sampling.py:128-143; `num_picks` is
-// already in call order, i.e. the reversed fanout list).
-std::vector<HopResult> run_hops(const CsrArgs &g, torch::Tensor seeds,
-                                const std::vector<int64_t> &num_picks, bool replace,
-                                std::optional<int64_t> seed) {
-  std::vector<HopResult> hops;
-  hops.reserve(num_picks.size());
+// already in call order, i.e. the reversed fanout list). With `features` the
+// rows of the last hop's unique ids (the input nodes of the mini-batch) are
+// fetched as well, queued directly behind that hop.
+
+BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<int64_t> &num_picks,
+                     bool replace, std::optional<int64_t> seed, const FeatureArgs *features) {
+  BatchResult batch;
+  batch.hops.reserve(num_picks.size());
   for (size_t hop = 0; hop < num_picks.size(); ++hop) {
     // without an RNG seed every call draws from the fixed default seed, stream 0,
     // as every call of the reference does (src/cache_graph_sampling.cu:204,407)
     const int64_t rng_stream = seed.has_value() ? static_cast<int64_t>(hop) : 0;
-    PendingHop pending = hop_issue(g, seeds, num_picks[hop], replace, seed, rng_stream);
-    hops.push_back(hop_finish(pending));
-    seeds = std::get<2>(hops.back());
+    if (features && hop + 1 == num_picks.size()) {
+      auto last = hop_then_fetch(g, *features, seeds, num_picks[hop], replace, seed, rng_stream);
+      batch.hops.push_back(last.first);
+      batch.features = last.second;
+    } else {
+      PendingHop pending = hop_issue(g, seeds, num_picks[hop], replace, seed, rng_stream);
+      batch.hops.push_back(hop_finish(pending));
+    }
+    seeds = std::get<2>(batch.hops.back());
   }
-  return hops;
+  if (features && num_picks.empty()) batch.features = fetch_rows(*features, cuda_ids(seeds, "seeds"));
+  return batch;
 }
 
 // Multi-hop sampling of several independent seed batches. Every batch is a
@@ -673,13 +754,10 @@ std::vector<HopResult> run_hops(const CsrArgs &g, torch::Tensor seeds,
 // default seed and stream 0); they are ordered after the calling
 // stream's earlier work and before its later work, and their memory is
 // registered with the calling stream.
-std::vector<std::vector<HopResult>> sample_blocks(
-    torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
-    std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, std::vector<torch::Tensor> seeds,
-    std::vector<int64_t> num_picks, bool replace, std::optional<std::vector<int64_t>> seeds_rng,
-    int64_t max_in_flight) {
-  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
-  check_csr(g);
+std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch::Tensor> &seeds,
+                                       const std::vector<int64_t> &num_picks, bool replace,
+                                       const std::optional<std::vector<int64_t>> &seeds_rng,
+                                       int64_t max_in_flight, const FeatureArgs *features) {
   const int64_t B = static_cast<int64_t>(seeds.size());
   TORCH_CHECK(!seeds_rng.has_value() || static_cast<int64_t>(seeds_rng->size()) == B,
               "seeds_rng must have one entry per batch");
@@ -689,11 +767,11 @@ std::vector<std::vector<HopResult>> sample_blocks(
   auto rng_of = [&](int64_t b) {
     return seeds_rng ? std::optional<int64_t>((*seeds_rng)[b]) : std::nullopt;
   };
-  std::vector<std::vector<HopResult>> out(B);
+  std::vector<BatchResult> out(B);
   const int64_t K = std::min<int64_t>({max_in_flight, kMaxBatchesInFlight, B});
   if (K <= 1) {
     py::gil_scoped_release no_gil;  // lets a Python thread that prefetches batches run beside the caller
-    for (int64_t b = 0; b < B; ++b) out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b));
+    for (int64_t b = 0; b < B; ++b) out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b), features);
     return out;
   }
   const auto caller = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
@@ -719,7 +797,7 @@ std::vector<std::vector<HopResult>> sample_blocks(
           c10::hip::set_device(device);
           CurrentStreamScope scope(lanes[j]);  // torch's current stream is per thread
           for (int64_t b = next_batch++; b < B; b = next_batch++)
-            out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b));
+            out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b), features);
         } catch (...) {
           failures[j] = std::current_exception();
           next_batch = B;  // the call will fail: the other workers stop after their current batch
@@ -737,10 +815,53 @@ std::vector<std::vector<HopResult>> sample_blocks(
   }
   for (auto &f : failures)
     if (f) std::rethrow_exception(f);
-  for (auto &hops : out)
-    for (auto &r : hops)
+  auto hand_over = [&](const torch::Tensor &t) {
+    if (t.defined() && t.is_cuda() && t.numel() > 0) t.record_stream(caller.unwrap());
+  };
+  for (auto &batch : out) {
+    for (auto &r : batch.hops)
       for (const torch::Tensor &t : {std::get<0>(r), std::get<1>(r), std::get<2>(r), std::get<3>(r)})
-        if (t.defined() && t.is_cuda() && t.numel() > 0) t.record_stream(caller.unwrap());
+        hand_over(t);
+    hand_over(batch.features);
+  }
+  return out;
+}
+
+std::vector<std::vector<HopResult>> sample_blocks(
+    torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
+    std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, std::vector<torch::Tensor> seeds,
+    std::vector<int64_t> num_picks, bool replace, std::optional<std::vector<int64_t>> seeds_rng,
+    int64_t max_in_flight) {
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+  check_csr(g);
+  std::vector<std::vector<HopResult>> out;
+  for (BatchResult &b : drive_batches(g, seeds, num_picks, replace, seeds_rng, max_in_flight, nullptr))
+    out.push_back(std::move(b.hops));
+  return out;
+}
+
+// sample_blocks plus, per batch, the feature rows of its input nodes (the
+// unique ids of the last hop): `features[b][i, :]` = row of `unique[i]`, as
+// cache_fetch(uva_data, gpu_data, unique, data_hashmap) returns it (uva_fetch
+// without a data_hashmap). The fetch is queued behind the last relabel before
+// the host knows the number of unique ids, into an output of `max_rows` rows
+// (None: the bound S * (k + 1) of the last hop; 0: never speculate); a batch
+// with more unique ids than that is fetched after its count is known.
+std::vector<std::pair<std::vector<HopResult>, torch::Tensor>> sample_blocks_fetch(
+    torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
+    std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, std::vector<torch::Tensor> seeds,
+    std::vector<int64_t> num_picks, bool replace, torch::Tensor uva_data,
+    std::optional<torch::Tensor> gpu_data, StaticHashmap *data_hashmap,
+    std::optional<std::vector<int64_t>> seeds_rng, int64_t max_in_flight,
+    std::optional<int64_t> max_rows) {
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+  check_csr(g);
+  TORCH_CHECK(!max_rows.has_value() || *max_rows >= 0, "max_rows must be >= 0");
+  FeatureArgs f{uva_data, gpu_data, data_hashmap, max_rows.value_or(-1)};
+  check_features(f);
+  std::vector<std::pair<std::vector<HopResult>, torch::Tensor>> out;
+  for (BatchResult &b : drive_batches(g, seeds, num_picks, replace, seeds_rng, max_in_flight, &f))
+    out.emplace_back(std::move(b.hops), std::move(b.features));
   return out;
 }
 
@@ -781,7 +902,12 @@ PYBIND11_MODULE(ShmTensorLib, m) {
            py::arg("replace"), py::arg("seed") = py::none(), py::arg("stream_id") = 0)
       .def("sample_blocks", &sample_blocks, py::arg("indptr"), py::arg("indices"), py::arg("gpu_indptr"),
            py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"),
-           py::arg("replace"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4);
+           py::arg("replace"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4)
+      .def("sample_blocks_fetch", &sample_blocks_fetch, py::arg("indptr"), py::arg("indices"),
+           py::arg("gpu_indptr"), py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"),
+           py::arg("num_picks"), py::arg("replace"), py::arg("uva_data"), py::arg("gpu_data"),
+           py::arg("data_hashmap"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4,
+           py::arg("max_rows") = py::none());
 
   py::class_<StaticHashmap>(m, "CUCOStaticHashmap")
       .def(py::init<torch::Tensor, torch::Tensor, double>())

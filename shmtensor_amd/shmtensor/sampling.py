@@ -50,7 +50,7 @@ class GPUSamplingDataloader:
 
     def __init__(self, indptr, indices, seeds, batchsize, num_picks, replace=False, use_ddp=False,
                  shuffle=True, drop_last=False, rng_seed=None, prefetch=1, background=False,
-                 indptr_on_device=False):
+                 indptr_on_device=False, features=None):
         self.indptr = indptr
         self.indices = indices
         self.seeds = seeds
@@ -73,6 +73,13 @@ class GPUSamplingDataloader:
         self.background = bool(background)
         self._ready = collections.deque()
         self._producer = None
+        # features=(uva_data, gpu_data, hashmap) (or (uva_data, None, None)): every batch also
+        # carries the feature rows of its input nodes, as cache_fetch / uva_fetch return them, and
+        # __next__ yields (input_nodes, output_nodes, blocks, input_features). The fetch is queued
+        # behind the last relabel without a host wait between them, into an output sized from the
+        # largest batch seen so far (a batch that outgrows it is fetched after its count is known).
+        self.features = features
+        self._feature_rows = 0
 
         self.has_cache = False
         self.gpu_indptr = None
@@ -158,19 +165,30 @@ class GPUSamplingDataloader:
         if self.rng_seed is not None:
             rng = [int(self.rng_seed) + batches_drawn + j for j in range(count)]
         cached = self.has_cache
+        graph = (self.indptr, self.indices, self.gpu_indptr if cached else None,
+                 self.gpu_indices if cached else None, self.hashmap if cached else None)
         # the last fanout is applied to the seed layer (sampling.py:128)
-        chains = capi.sample_blocks(self.indptr, self.indices, self.gpu_indptr if cached else None,
-                                    self.gpu_indices if cached else None, self.hashmap if cached else None,
-                                    groups, list(reversed(self.num_picks)), self.replace, seeds_rng=rng,
-                                    max_in_flight=self.prefetch)
+        picks = list(reversed(self.num_picks))
+        if self.features is None:
+            chains = capi.sample_blocks(*graph, groups, picks, self.replace, seeds_rng=rng,
+                                        max_in_flight=self.prefetch)
+            rows = [None] * len(groups)
+        else:
+            uva_data, gpu_data, data_map = self.features
+            guess = self._feature_rows + self._feature_rows // 4 + 1024 if self._feature_rows else 0
+            fetched = capi.sample_blocks_fetch(*graph, groups, picks, self.replace, uva_data, gpu_data, data_map,
+                                               seeds_rng=rng, max_in_flight=self.prefetch, max_rows=guess)
+            chains = [hops for hops, _ in fetched]
+            rows = [x for _, x in fetched]
+            self._feature_rows = max([self._feature_rows] + [x.shape[0] for x in rows])
         out = []
-        for seeds, chain in zip(groups, chains):
+        for seeds, chain, x in zip(groups, chains, rows):
             blocks, dst = [], seeds
             for sub_indptr, _, unique_tensor, relabel_indices in chain:
                 blocks.insert(0, create_block_from_csc(sub_indptr, relabel_indices, torch.Tensor(),
                                                        unique_tensor.numel(), dst.numel()))
                 dst = unique_tensor
-            out.append((dst, seeds, blocks))
+            out.append((dst, seeds, blocks) if self.features is None else (dst, seeds, blocks, x))
         return out
 
     def _produce(self, first_batch, batches_drawn, out_queue, stop):
@@ -225,8 +243,10 @@ class GPUSamplingDataloader:
         group, done = item
         current = torch.cuda.current_stream()
         current.wait_event(done)
-        for dst, _, blocks in group:       # produced on other streams, consumed on this one
-            for t in (dst,) + tuple(x for blk in blocks if isinstance(blk, CSCBlock) for x in blk[:2]):
+        for item in group:                 # produced on other streams, consumed on this one
+            dst, blocks = item[0], item[2]
+            for t in (dst,) + tuple(item[3:]) + tuple(x for blk in blocks if isinstance(blk, CSCBlock)
+                                                      for x in blk[:2]):
                 if t.numel() > 0:
                     t.record_stream(current)
         self._ready.extend(group)
@@ -237,10 +257,10 @@ class GPUSamplingDataloader:
             raise StopIteration
         if not self._ready:
             self._refill()
-        input_nodes, output_nodes, blocks = self._ready.popleft()
+        batch = self._ready.popleft()      # (input_nodes, output_nodes, blocks[, input_features])
         self.curr += 1
         self._batches_drawn += 1
-        return input_nodes, output_nodes, blocks
+        return batch
 
     # ---- cache ---------------------------------------------------------------------
 

@@ -137,6 +137,20 @@ int main() {
     const char *expect = it == slot_of.end() ? h_table + q[i] * row_bytes : cache_rows.data() + it->second * row_bytes;
     EXPECT(std::equal(expect, expect + row_bytes, out.begin() + i * row_bytes));
   }
+  // the same fetch told on the device how many rows there are: the first `counted`
+  // rows arrive, the rest of the output is left alone
+  const int64_t counted = Q / 3;
+  int64_t *d_count = to_device(std::vector<int64_t>{counted});
+  HIP_OK(hipMemsetAsync(d_out, 0x5A, Q * row_bytes, stream));
+  SHMT_OK_(shmt_fetch_counted(table_alias, d_cache, d_q, 4, fmap, nullptr, 0, d_out, Q, d_count, nullptr,
+                              row_bytes, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  std::vector<char> part = to_host(d_out, Q * row_bytes);
+  EXPECT(std::equal(part.begin(), part.begin() + counted * row_bytes, out.begin()));
+  for (int64_t i = counted * row_bytes; i < Q * row_bytes; ++i) EXPECT(part[i] == 0x5A);
+  EXPECT(shmt_fetch_counted(table_alias, d_cache, d_q, 4, fmap, nullptr, 0, d_out, Q, nullptr, nullptr,
+                            row_bytes, stream) == SHMT_EINVAL);
+  HIP_OK(hipFree(d_count));
   // pageable host memory is refused instead of faulting
   std::vector<char> pageable(4096);
   void *alias = nullptr;

@@ -154,6 +154,31 @@ def test_prefetch_and_background_give_the_same_batches(capi, graph, rng_seed):
         assert dl._producer is None
 
 
+@pytest.mark.parametrize("cached_rows", [True, False])
+def test_features_option_adds_the_rows_of_the_input_nodes(capi, graph, cached_rows):
+    """features=(table, cache rows, map): same batches, plus the feature rows of
+    the input nodes exactly as a separate cache_fetch / uva_fetch returns them."""
+    n = graph[0]
+    gen = torch.Generator().manual_seed(8)
+    table = torch.randn(n, 20, generator=gen).pin_memory()
+    hot = torch.randperm(n, generator=gen)[: n // 3]
+    rows = (table[hot] - 2.0).cuda()               # a hit is told from a miss by its content
+    rows_map = capi.CUCOStaticHashmap(hot.cuda(), torch.arange(hot.numel()).cuda(), 0.8)
+    feats = (table, rows, rows_map) if cached_rows else (table, None, None)
+    base = _collect(_loader(graph, batchsize=100, num_picks=[6, 4, 3], rng_seed=5))
+    for kw in (dict(), dict(prefetch=3), dict(prefetch=2, background=True)):
+        dl = _loader(graph, batchsize=100, num_picks=[6, 4, 3], rng_seed=5, features=feats, **kw)
+        got = [(i.clone(), o.clone(), [(b.indptr.clone(), b.indices.clone(), b.num_src, b.num_dst) for b in blocks], x)
+               for i, o, blocks, x in dl]
+        _same_epoch([g[:3] for g in got], base)
+        for input_nodes, _, _, x in got:
+            want = capi.cache_fetch(table, rows, input_nodes, rows_map) if cached_rows else \
+                capi.uva_fetch(table, input_nodes)
+            assert torch.equal(x, want)
+        assert dl._feature_rows == max(g[0].numel() for g in got)
+        dl.close()
+
+
 def test_background_producer_stops_early_and_reports_errors(capi, graph):
     dl = _loader(graph, batchsize=50, prefetch=2, background=True)
     it = iter(dl)

@@ -293,3 +293,61 @@ def test_large_skewed_fetch_scaled(capi):
     assert torch.equal(capi.cache_fetch(table, cache, rows, h).view(torch.int16), upd.view(torch.int16))
     torch.cuda.synchronize()
     assert torch.equal(table.view(torch.int16), before.view(torch.int16))      # hits never touch the host copy
+
+
+@pytest.mark.parametrize("route", ["direct", "map", "mask"])
+@pytest.mark.parametrize("count", [0, 1, 63, 64, 700, 5000, 9000])
+def test_c_abi_fetch_with_the_row_count_in_device_memory(cabi, route, count):
+    """shmt_fetch_counted moves min(max_rows, *count) rows, leaves the rest of
+    the output alone and forwards the count to the host."""
+    import ctypes
+    lib = cabi.load()
+    g = torch.Generator().manual_seed(count)
+    table = torch.randn(4000, 48, generator=g)
+    table_dev = table.cuda()
+    ids = torch.randperm(4000, generator=g)[:1500]
+    cache = (table[ids] + 1.0).cuda()                  # a hit is told from a miss by its content
+    max_rows = 5000
+    idx = torch.randint(0, 4000, (max(count, max_rows),), generator=g)
+    slot_of = torch.full((4000,), -1, dtype=torch.int64)
+    slot_of[ids] = torch.arange(1500)
+    expect = torch.where((slot_of[idx] >= 0)[:, None], table[idx] + 1.0, table[idx]) if route != "direct" \
+        else table[idx]
+    idx_dev = idx.cuda()
+    hnd, mask, keep = None, None, []
+    if route == "map":
+        keys, vals = ids.cuda(), torch.arange(1500).cuda()
+        nbytes = lib.shmt_hashmap_table_bytes(1500, 0.8, 8, 8)
+        keep.append(torch.empty(nbytes, dtype=torch.uint8).cuda())
+        hnd = ctypes.c_void_p()
+        cabi.check(lib.shmt_hashmap_create(ctypes.byref(hnd), keys.data_ptr(), vals.data_ptr(), 1500, 8, 8, 0.8,
+                                           keep[0].data_ptr(), nbytes, cabi.current_stream()))
+    elif route == "mask":
+        mask = slot_of[idx].cuda()
+    out = torch.full((max_rows, 48), -7.0).cuda()
+    count_dev = torch.tensor([count]).cuda()
+    seen = torch.full((1,), -1, dtype=torch.int64).pin_memory()
+    seen_dev = ctypes.c_void_p()
+    cabi.check(lib.shmt_host_devptr(seen.data_ptr(), ctypes.byref(seen_dev)))
+    cabi.check(lib.shmt_fetch_counted(table_dev.data_ptr(), cache.data_ptr() if route != "direct" else None,
+                                      idx_dev.data_ptr(), 8, hnd, mask.data_ptr() if mask is not None else None,
+                                      8 if mask is not None else 0, out.data_ptr(), max_rows,
+                                      count_dev.data_ptr(), seen_dev, 48 * 4,
+                                      cabi.current_stream()))
+    torch.cuda.synchronize()
+    moved = min(count, max_rows)
+    assert torch.equal(out[:moved].cpu(), expect[:moved])
+    assert bool((out[moved:] == -7.0).all())
+    assert seen.item() == count
+    # without a host slot; and a null count is an argument error, not a launch
+    out2 = torch.full((max_rows, 48), -7.0).cuda()
+    cabi.check(lib.shmt_fetch_counted(table_dev.data_ptr(), cache.data_ptr() if route != "direct" else None,
+                                      idx_dev.data_ptr(), 8, hnd, mask.data_ptr() if mask is not None else None,
+                                      8 if mask is not None else 0, out2.data_ptr(), max_rows,
+                                      count_dev.data_ptr(), None, 48 * 4, cabi.current_stream()))
+    assert torch.equal(out2, out)
+    assert lib.shmt_fetch_counted(table_dev.data_ptr(), None, idx_dev.data_ptr(), 8, None, None, 0,
+                                  out2.data_ptr(), max_rows, None, None, 48 * 4, None) != 0
+    if hnd is not None:
+        torch.cuda.synchronize()
+        lib.shmt_hashmap_destroy(hnd)

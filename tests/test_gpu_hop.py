@@ -308,3 +308,67 @@ def test_hop_relabel_table_format_follows_the_id_range(capi, oracle, odd_ids):
         assert np.array_equal(uniq.cpu().numpy(), exp_unique)
         assert np.array_equal(lab.cpu().numpy(), exp_labels)
         _same((sp, si, uniq, lab), _two_step(capi, ip, ix, None, sd, k, False, seed=1))
+
+
+@pytest.mark.parametrize("max_rows", [None, 0, 600, 100000])
+@pytest.mark.parametrize("in_flight", [1, 4])
+@pytest.mark.parametrize("cached_rows", [True, False])
+def test_sample_blocks_fetch_equals_sample_blocks_then_fetch(capi, max_rows, in_flight, cached_rows):
+    """The feature fetch queued behind the last relabel (row count read on the
+    device) returns what a separate fetch of the batch's input nodes returns,
+    whether the speculative output is the bound, too small (600 rows: the
+    count is then waited for), generous, or not used at all (0)."""
+    indptr, indices = _graph(scale=13)
+    indptr_h, indices_h = indptr.cpu().pin_memory(), indices.cpu().pin_memory()
+    n = indptr.numel() - 1
+    gen = torch.Generator().manual_seed(4)
+    hot = torch.randperm(n, generator=gen)[: n // 3].cuda()
+    gp, gi = capi.create_subcsr(indptr_h, indices_h, hot)
+    h = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel()).cuda(), 0.8)
+    table = torch.randn(n, 24, generator=gen).pin_memory()
+    rows_hot = torch.randperm(n, generator=gen)[: n // 4]
+    gpu_rows = (table[rows_hot] + 1.0).cuda()          # a hit is told from a miss by its content
+    rows_map = capi.CUCOStaticHashmap(rows_hot.cuda(), torch.arange(rows_hot.numel()).cuda(), 0.8)
+    sizes = [300, 1, 0, 257, 1500, 33]
+    batches = [torch.randperm(n, generator=gen)[:s].cuda() for s in sizes]
+    rng = [50 + b for b in range(len(batches))]
+    for picks in ([4, 6], [3], []):
+        want_hops = capi.sample_blocks(indptr_h, indices_h, gp, gi, h, batches, picks, False, seeds_rng=rng)
+        for repeat in range(2):
+            got = capi.sample_blocks_fetch(indptr_h, indices_h, gp, gi, h, batches, picks, False, table,
+                                           gpu_rows if cached_rows else None,
+                                           rows_map if cached_rows else None, seeds_rng=rng,
+                                           max_in_flight=in_flight, max_rows=max_rows)
+            assert len(got) == len(batches)
+            for b, (hops, rows) in enumerate(got):
+                assert len(hops) == len(picks)
+                for x, y in zip(hops, want_hops[b]):
+                    _same(x, y)
+                nodes = hops[-1][2] if picks else batches[b]
+                if cached_rows:
+                    want = capi.cache_fetch(table, gpu_rows, nodes, rows_map)
+                else:
+                    want = capi.uva_fetch(table, nodes)
+                assert rows.shape == want.shape and torch.equal(rows, want)
+
+
+def test_sample_blocks_fetch_arguments(capi):
+    indptr = torch.tensor([0, 3, 3, 4]).cuda()
+    indices = torch.tensor([2, 1, 0, 2]).cuda()
+    table = torch.arange(12.0).reshape(3, 4).cuda()        # a device-resident table is accepted
+    seeds = [torch.tensor([0, 2]).cuda(), torch.tensor([1]).cuda()]
+    got = capi.sample_blocks_fetch(indptr, indices, None, None, None, seeds, [5], False, table, None, None)
+    for hops, rows in got:
+        assert torch.equal(rows, table[hops[-1][2]])
+    one_d = torch.arange(3.0).cuda()                       # 1-D data gives 1-D rows, as cache_fetch does
+    got = capi.sample_blocks_fetch(indptr, indices, None, None, None, seeds, [5], False, one_d, None, None)
+    for hops, rows in got:
+        assert rows.dim() == 1 and torch.equal(rows, one_d[hops[-1][2]])
+    with pytest.raises(RuntimeError):                      # a hashmap without its cache rows
+        capi.sample_blocks_fetch(indptr, indices, None, None, None, seeds, [5], False, table, None,
+                                 capi.CUCOStaticHashmap(torch.arange(2).cuda(), torch.arange(2).cuda(), 0.5))
+    with pytest.raises(RuntimeError):
+        capi.sample_blocks_fetch(indptr, indices, None, None, None, seeds, [5], False, table, None, None,
+                                 max_rows=-1)
+    with pytest.raises(RuntimeError):                      # pageable host memory
+        capi.sample_blocks_fetch(indptr, indices, None, None, None, seeds, [5], False, table.cpu(), None, None)
