@@ -395,15 +395,16 @@ def bench_sampling(capi, args, result):
 
     picks = list(reversed(fanouts))
 
-    def timed_in_flight(in_flight):
-        """All batches through sample_blocks: up to `in_flight` of them advance concurrently."""
+    def timed_in_flight(in_flight, row_offsets=indptr):
+        """All batches through sample_blocks (hops chained on the device): up to `in_flight` of them
+        advance concurrently."""
         rng = [7777 + b for b in range(nbatch)]
         for _ in range(2):
-            capi.sample_blocks(indptr, indices, gp, gi, hmap, seed_batches, picks, False, seeds_rng=rng,
+            capi.sample_blocks(row_offsets, indices, gp, gi, hmap, seed_batches, picks, False, seeds_rng=rng,
                                max_in_flight=in_flight)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        res = capi.sample_blocks(indptr, indices, gp, gi, hmap, seed_batches, picks, False, seeds_rng=rng,
+        res = capi.sample_blocks(row_offsets, indices, gp, gi, hmap, seed_batches, picks, False, seeds_rng=rng,
                                  max_in_flight=in_flight)
         torch.cuda.synchronize()
         t = time.perf_counter() - t0
@@ -422,6 +423,8 @@ def bench_sampling(capi, args, result):
         assert e == edges, "batched hops sampled a different number of edges"
         overlapped["%d_batches_in_flight" % in_flight] = {"ms_per_batch": round(t * 1e3 / nbatch, 4),
                                                           "sampled_edges_per_s": round(e / t, 1)}
+    e, t_chain_hbm = timed_in_flight(1, indptr_hbm)
+    assert e == edges, "indptr placement changed the sample"
     res = {"graph": "R-MAT scale %d ef 30 symmetrised: %d nodes, %d edges; top 30 %% by degree cached"
                     % (args.sampling_scale, n, indices.numel()),
            "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
@@ -430,6 +433,8 @@ def bench_sampling(capi, args, result):
            "fused_hop_ms_per_batch": round(gpu_t_fused * 1e3 / nbatch, 4),
            "fused_hop_sampled_edges_per_s": round(edges / gpu_t_fused, 1),
            "fused_hop_indptr_in_hbm_ms_per_batch": round(gpu_t_hbm * 1e3 / nbatch, 4),
+           "chained_hops_ms_per_batch": overlapped["1_batches_in_flight"]["ms_per_batch"],
+           "chained_hops_indptr_in_hbm_ms_per_batch": round(t_chain_hbm * 1e3 / nbatch, 4),
            "sample_blocks_batches_in_flight": overlapped}
     if not args.no_cpu:
         from oracle import oracle as orc

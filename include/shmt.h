@@ -263,6 +263,36 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices,
                     void *labels_out, int64_t *nnz_out, int64_t *count_out,
                     void *stream);
 
+/* shmt_sample_hop for a number of seeds that only the GPU knows yet, so that
+ * the hops of a mini-batch (python/shmtensor/sampling.py:128-143: the unique
+ * ids of one hop are the seeds of the next) queue back to back without the
+ * host reading a size in between; the reference waits on the host inside
+ * every sampling and relabel call (src/cache_graph_sampling.cu:195,403,
+ * src/tensor_relabel.cu:173). `seeds` holds min(max_seeds, *seeds_len)
+ * seeds, seeds_len being an int64 in device memory written by earlier work
+ * of the stream (count_dev_out of the previous hop, whose unique_out is
+ * then `seeds`); seeds_len == NULL means max_seeds seeds. Every buffer is
+ * sized as shmt_sample_hop sizes it for S = max_seeds; the results are laid
+ * out for the true number of seeds S': sub_indptr has S' + 1 entries,
+ * total_out / labels_out hold the S' seeds followed by the sampled ids.
+ * count_dev_out (device memory, may be NULL) receives the number of
+ * distinct ids like count_out does.                                        */
+int shmt_sample_hop_chained(const void *indptr, int ptr_bytes,
+                            const void *indices, int idx_bytes,
+                            const void *cache_indptr,
+                            const void *cache_indices,
+                            const shmt_hashmap_t *map, const void *seeds,
+                            int seed_bytes, int64_t max_seeds,
+                            const int64_t *seeds_len, int64_t k, int replace,
+                            uint64_t rng_seed, uint32_t rng_stream,
+                            void *sub_indptr, void *sub_indices, void *plan,
+                            int64_t plan_bytes, int elem_bytes,
+                            void *total_out, void *scratch,
+                            int64_t scratch_bytes, void *unique_out,
+                            void *labels_out, int64_t *nnz_out,
+                            int64_t *count_out, int64_t *count_dev_out,
+                            void *stream);
+
 /* Cached sub-CSR: CreateCacheCSR, src/cache_graph_sampling.cu:455-492
  * (CSRIndicesCopyKernel :428-453). Step 1 writes
  * cache_indptr[0..C] = exclusive scan of deg(seeds[i]) (width ptr_bytes) and

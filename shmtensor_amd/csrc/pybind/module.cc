@@ -531,25 +531,27 @@ void check_csr(CsrArgs &g) {
 struct PendingHop {
   bool finished = false;
   HopResult result;                       // valid when finished
-  int64_t S = 0;
+  int64_t S = 0;                          // number of seeds the buffers are sized for
+  bool counted_seeds = false;             // the kernels took the true number of seeds from device memory
   torch::Tensor sub_indptr, sub_indices, unique, labels;
   torch::Tensor workspace;                // plan + relabel input + relabel scratch, kept until the sizes are in
   Readback::Slot nnz_slot{}, count_slot{};
-  int64_t *count_dev = nullptr;           // set when the count goes to device memory (see hop_issue)
+  int64_t *count_dev = nullptr;           // fused hops: the number of unique ids in device memory as well
 };
 
-// With `count_on_device` the number of unique ids is written to device memory
-// (h.count_dev) instead of the host slot, for a kernel queued behind the hop
-// to read; that kernel must then forward it to h.count_slot.dev, or
-// hop_finish never sees it (issue_counted_fetch does).
-PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, bool replace,
-                     std::optional<int64_t> seed, int64_t stream_id, bool count_on_device = false) {
+// Queues one hop. `seeds_len` (device memory) makes it a chained hop: `seeds`
+// then holds an unknown number of ids, at most seeds.numel(), and the kernels
+// read the true number there (the count_dev of the hop before, whose unique
+// buffer is `seeds`); every buffer is sized for the bound.
+PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds_len, int64_t num_picks,
+                     bool replace, std::optional<int64_t> seed, int64_t stream_id) {
   PendingHop h;
   seeds = cuda_ids(seeds, "seeds");
   TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0");
   const int64_t S = seeds.numel();
   const bool fused = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
   if (!fused) {  // degenerate or very large bound: the two operators one after the other
+    TORCH_CHECK(seeds_len == nullptr, "internal: a chained hop must be a fused one");
     auto sampled = sample_impl(g.indptr, g.indices, g.cached() ? &*g.gpu_indptr : nullptr,
                                g.cached() ? &*g.gpu_indices : nullptr, g.hashmap, seeds, num_picks,
                                replace, seed, stream_id);
@@ -565,14 +567,15 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   void *stream = current_stream();
   const int64_t bound = S * num_picks;
   h.S = S;
+  h.counted_seeds = seeds_len != nullptr;
   const int eb = std::max(sb, ib);
   const auto id_type = eb == 8 ? torch::kInt64 : torch::kInt32;
   const int64_t n_max = S + bound;
   auto aligned = [](int64_t bytes) { return (bytes + 255) & ~int64_t{255}; };
   // Two allocations per hop (the allocator is shared by all host threads that drive
-  // batches): one for the four results, which are typed views of it, ...
-  torch::Tensor results = device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) +
-                                       2 * aligned(n_max * eb) + (count_on_device ? 256 : 0));
+  // batches): one for the four results, which are typed views of it, and the count ...
+  torch::Tensor results =
+      device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) + 2 * aligned(n_max * eb) + 256);
   int64_t offset = 0;
   auto carve = [&](int64_t count, int elem, torch::ScalarType type) {
     torch::Tensor t = results.narrow(0, offset, count * elem).view(type);
@@ -583,8 +586,7 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   h.sub_indices = carve(bound, ib, g.indices.scalar_type());
   h.unique = carve(n_max, eb, id_type);
   h.labels = carve(n_max, eb, id_type);
-  if (count_on_device)
-    h.count_dev = reinterpret_cast<int64_t *>(static_cast<char *>(results.data_ptr()) + offset);
+  h.count_dev = reinterpret_cast<int64_t *>(static_cast<char *>(results.data_ptr()) + offset);
   // ... and one for everything that does not outlive the hop
   const int64_t plan_bytes = shmt_sample_plan_bytes(S);
   const int64_t total_bytes = n_max * eb;
@@ -595,26 +597,28 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, int64_t num_picks, b
   char *const scratch_ptr = total_ptr + aligned(total_bytes);
   h.nnz_slot = readback().acquire();
   h.count_slot = readback().acquire();
-  check(shmt_sample_hop(g.indptr_dev, pb, g.indices_dev, ib,
-                        g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
-                        g.cached() ? g.gpu_indices->data_ptr() : nullptr,
-                        g.cached() ? g.hashmap->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks,
-                        replace, static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
-                        static_cast<uint32_t>(stream_id), h.sub_indptr.data_ptr(), h.sub_indices.data_ptr(),
-                        plan_ptr, plan_bytes, eb, total_ptr, scratch_ptr,
-                        scratch_bytes, h.unique.data_ptr(), h.labels.data_ptr(), h.nnz_slot.dev,
-                        count_on_device ? h.count_dev : h.count_slot.dev, stream));
+  check(shmt_sample_hop_chained(
+      g.indptr_dev, pb, g.indices_dev, ib, g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
+      g.cached() ? g.gpu_indices->data_ptr() : nullptr, g.cached() ? g.hashmap->handle() : nullptr,
+      seeds.data_ptr(), sb, S, seeds_len, num_picks, replace,
+      static_cast<uint64_t>(seed.value_or(kDefaultSeed)), static_cast<uint32_t>(stream_id),
+      h.sub_indptr.data_ptr(), h.sub_indices.data_ptr(), plan_ptr, plan_bytes, eb, total_ptr, scratch_ptr,
+      scratch_bytes, h.unique.data_ptr(), h.labels.data_ptr(), h.nnz_slot.dev, h.count_slot.dev, h.count_dev,
+      stream));
   return h;
 }
 
 // Must run with the stream of hop_issue current (the wait falls back to
-// synchronising the current stream).
-HopResult hop_finish(PendingHop &h) {
+// synchronising the current stream). `true_seeds`: the number of seeds of a
+// chained hop, i.e. the number of unique ids of the hop before it.
+HopResult hop_finish(PendingHop &h, int64_t true_seeds = -1) {
   if (!h.finished) {
+    const int64_t S = h.counted_seeds ? true_seeds : h.S;
+    TORCH_CHECK(S >= 0 && S <= h.S, "internal: chained hop finished without its seed count");
     const int64_t nnz = Readback::wait(h.nnz_slot);
     const int64_t U = Readback::wait(h.count_slot);
-    h.result = std::make_tuple(h.sub_indptr, h.sub_indices.narrow(0, 0, nnz), h.unique.narrow(0, 0, U),
-                               h.labels.narrow(0, h.S, nnz));
+    h.result = std::make_tuple(h.sub_indptr.narrow(0, 0, S + 1), h.sub_indices.narrow(0, 0, nnz),
+                               h.unique.narrow(0, 0, U), h.labels.narrow(0, S, nnz));
     h.finished = true;
     // scratch goes back to the allocator of its stream; work queued later on
     // that stream is ordered after the kernels that still read it
@@ -645,8 +649,8 @@ torch::Tensor fetch_rows(const FeatureArgs &f, const torch::Tensor &ids) {
 
 // Queues the fetch of the rows of the hop's unique ids behind the hop, before
 // the host knows how many there are: the kernel takes the count from device
-// memory and forwards it to the host slot hop_finish waits on. Returns the
-// output sized for `rows` ids (the caller narrows it once the count is in).
+// memory. Returns the output sized for `rows` ids (the caller narrows it once
+// the count is in).
 torch::Tensor issue_counted_fetch(const PendingHop &h, const FeatureArgs &f, int64_t rows) {
   const RowShape rs = row_shape(f.uva_data, rows);
   torch::Tensor out = torch::empty(rs.out_sizes, f.uva_data.options().device(torch::kCUDA));
@@ -655,31 +659,8 @@ torch::Tensor issue_counted_fetch(const PendingHop &h, const FeatureArgs &f, int
   check(shmt_fetch_counted(f.uva_dev, cache_ptr, h.unique.data_ptr(),
                            static_cast<int>(h.unique.element_size()),
                            f.cached() ? f.hashmap->handle() : nullptr, nullptr, 0, out.data_ptr(), rows,
-                           h.count_dev, h.count_slot.dev, rs.row_bytes, current_stream()));
+                           h.count_dev, nullptr, rs.row_bytes, current_stream()));
   return out;
-}
-
-// One hop followed by the fetch of the feature rows of its unique ids. When
-// the speculative output is large enough (the usual case) no host wait
-// separates the relabel from the fetch; otherwise the rows are fetched once
-// the count is known.
-std::pair<HopResult, torch::Tensor> hop_then_fetch(const CsrArgs &g, const FeatureArgs &f,
-                                                   torch::Tensor seeds, int64_t num_picks, bool replace,
-                                                   std::optional<int64_t> seed, int64_t stream_id) {
-  const int64_t row_bytes = row_shape(f.uva_data, 0).row_bytes;
-  const bool speculate = f.max_rows != 0 && row_bytes > 0;
-  PendingHop h = hop_issue(g, seeds, num_picks, replace, seed, stream_id, speculate);
-  if (h.count_dev == nullptr) {  // not speculating, or a degenerate hop that ran unfused
-    HopResult r = hop_finish(h);
-    return {r, fetch_rows(f, std::get<2>(r))};
-  }
-  const int64_t bound = h.unique.numel();
-  const int64_t rows = f.max_rows < 0 ? bound : std::min(bound, f.max_rows);
-  torch::Tensor out = issue_counted_fetch(h, f, rows);
-  HopResult r = hop_finish(h);
-  const int64_t U = std::get<2>(r).numel();
-  if (U <= rows) return {r, out.narrow(0, 0, U)};
-  return {r, fetch_rows(f, std::get<2>(r))};
 }
 
 HopResult sample_hop(torch::Tensor indptr, torch::Tensor indices,
@@ -688,7 +669,7 @@ HopResult sample_hop(torch::Tensor indptr, torch::Tensor indices,
                      std::optional<int64_t> seed, int64_t stream_id) {
   CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
   check_csr(g);
-  PendingHop h = hop_issue(g, seeds, num_picks, replace, seed, stream_id);
+  PendingHop h = hop_issue(g, seeds, nullptr, num_picks, replace, seed, stream_id);
   return hop_finish(h);
 }
 
@@ -714,32 +695,73 @@ struct BatchResult {
   torch::Tensor features;  // defined only when features were asked for
 };
 
+// Ids a chained hop's buffers may be sized for: hop h + 1 is queued behind hop
+// h without waiting for h's sizes as long as its bound (every seed of the
+// bound-sized unique list of h with all its picks) stays below this.
+constexpr int64_t kChainLimit = 1ll << 21;
+
 // All hops of one batch on the current stream: hop h samples `num_picks[h]`
 // neighbours of the previous hop's unique ids (RNG stream h when a seed is
 // given), as the dataloader's loop does (python/shmtensor/sampling.py:128-143; `num_picks` is
-// already in call order, i.e. the reversed fanout list). With `features` the
+// already in call order, i.e. the reversed fanout list). Consecutive hops are
+// chained on the device while their bounds allow: the next hop takes its seeds
+// and their number from the buffers of the one before and is queued at once,
+// and the host reads all sizes of the chain afterwards. With `features` the
 // rows of the last hop's unique ids (the input nodes of the mini-batch) are
 // fetched as well, queued directly behind that hop.
-
 BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<int64_t> &num_picks,
                      bool replace, std::optional<int64_t> seed, const FeatureArgs *features) {
   BatchResult batch;
   batch.hops.reserve(num_picks.size());
+  std::vector<PendingHop> chain;  // queued hops whose sizes have not been read yet
+  auto finish_chain = [&]() {
+    for (PendingHop &h : chain) {
+      const int64_t true_seeds = batch.hops.empty() ? -1 : std::get<2>(batch.hops.back()).numel();
+      batch.hops.push_back(hop_finish(h, true_seeds));
+    }
+    chain.clear();
+  };
   for (size_t hop = 0; hop < num_picks.size(); ++hop) {
     // without an RNG seed every call draws from the fixed default seed, stream 0,
     // as every call of the reference does (src/cache_graph_sampling.cu:204,407)
     const int64_t rng_stream = seed.has_value() ? static_cast<int64_t>(hop) : 0;
-    if (features && hop + 1 == num_picks.size()) {
-      auto last = hop_then_fetch(g, *features, seeds, num_picks[hop], replace, seed, rng_stream);
-      batch.hops.push_back(last.first);
-      batch.features = last.second;
-    } else {
-      PendingHop pending = hop_issue(g, seeds, num_picks[hop], replace, seed, rng_stream);
-      batch.hops.push_back(hop_finish(pending));
+    const int64_t k = num_picks[hop];
+    const int64_t *seeds_len = nullptr;
+    if (!chain.empty()) {
+      const PendingHop &prev = chain.back();
+      if (k > 0 && prev.unique.numel() <= kChainLimit / (k + 1)) {
+        seeds = prev.unique;
+        seeds_len = prev.count_dev;
+      } else {
+        finish_chain();
+      }
     }
-    seeds = std::get<2>(batch.hops.back());
+    if (chain.empty() && !batch.hops.empty()) seeds = std::get<2>(batch.hops.back());
+    PendingHop h = hop_issue(g, seeds, seeds_len, k, replace, seed, rng_stream);
+    if (h.finished)
+      batch.hops.push_back(h.result);  // ran as two separate operators (never a chained hop)
+    else
+      chain.push_back(std::move(h));
   }
-  if (features && num_picks.empty()) batch.features = fetch_rows(*features, cuda_ids(seeds, "seeds"));
+  if (!features) {
+    finish_chain();
+    return batch;
+  }
+  const FeatureArgs &f = *features;
+  const bool speculate = f.max_rows != 0 && row_shape(f.uva_data, 0).row_bytes > 0;
+  if (chain.empty() || !speculate) {
+    finish_chain();
+    batch.features = fetch_rows(f, batch.hops.empty() ? cuda_ids(seeds, "seeds") : std::get<2>(batch.hops.back()));
+    return batch;
+  }
+  // the rows of the last hop's unique ids, fetched before the host knows how many there are
+  const PendingHop &last = chain.back();
+  const int64_t bound = last.unique.numel();
+  const int64_t rows = f.max_rows < 0 ? bound : std::min(bound, f.max_rows);
+  torch::Tensor out = issue_counted_fetch(last, f, rows);
+  finish_chain();
+  const torch::Tensor &nodes = std::get<2>(batch.hops.back());
+  batch.features = nodes.numel() <= rows ? out.narrow(0, 0, nodes.numel()) : fetch_rows(f, nodes);
   return batch;
 }
 

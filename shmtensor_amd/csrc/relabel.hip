@@ -8,7 +8,7 @@
 //            distinct id of the tile (64-bit CAS on the key, atomicMin the index)
 //   first    first[i] = smallest index holding the same key (kept in the
 //            labels buffer); per-tile count of i with first[i] == i
-//   partials exclusive scan of the per-tile counts (own launch only beyond 1 M ids)
+//   partials exclusive scan of the per-tile counts (own launch only beyond 2 M ids)
 //   unique   rank of every first occurrence; unique[rank] = key; rank_of[i]
 //   labels   labels[i] = rank_of[first[i]]
 // The table is touched only by `insert` and `first`; the last two passes read
@@ -16,6 +16,8 @@
 // factor <= 0.5 with a mixed hash (the reference hashes with the low bits of
 // the id, src/tensor_relabel.cu:111-117); ids known to fit 32 bits use the
 // same memory as packed 8-byte slots (see rl_packed_insert).
+// Up to 8,192 ids all of this is one launch of one workgroup with its table
+// in LDS (rl_small_kernel).
 #include "common.h"
 #include "launchers.h"
 #include "scan_dev.h"
@@ -27,23 +29,29 @@ namespace shmt {
 constexpr int kRlBlock = 256;
 constexpr int kRlItems = 2;
 constexpr int kRlTile = kRlBlock * kRlItems;
-constexpr int64_t kRlSelfPrefixTiles = 2048;  // up to 1 M ids the unique pass sums the tile counts itself
+constexpr int64_t kRlSelfPrefixTiles = 4096;  // up to 2 M ids the unique pass sums the tile counts itself
 
 // Number of input ids: a host-known part plus, optionally, a part that only
 // the device knows (the length of the last segment, e.g. the nnz a sampling
 // kernel produced earlier on the same stream).
 struct RlCount {
   int64_t fixed;
+  const int64_t *fixed_dev;  // when set: the first part is this device-side figure, at most `fixed`
   const void *extra;  // device address of the extra length, or null
   int extra_bytes;    // its width, 4 or 8
   int64_t limit;      // what launches and buffers were sized for; the count is clamped to it
 };
 
 __device__ __forceinline__ int64_t rl_count(const RlCount &n) {
-  if (!n.extra) return n.fixed;
-  int64_t extra = load_int(n.extra, 0, n.extra_bytes);
+  if (!n.extra && !n.fixed_dev) return n.fixed;
+  int64_t first = n.fixed;
+  if (n.fixed_dev) {
+    const int64_t f = *n.fixed_dev;
+    first = f < 0 ? 0 : (f < n.fixed ? f : n.fixed);
+  }
+  int64_t extra = n.extra ? load_int(n.extra, 0, n.extra_bytes) : 0;
   if (extra < 0) extra = 0;
-  const int64_t N = n.fixed + extra;
+  const int64_t N = first + extra;
   return N < n.limit ? N : n.limit;
 }
 
@@ -269,7 +277,8 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
                                                              const void *labels,
                                                              const uint64_t *partials,
                                                              void *unique_out, uint32_t *rank_of,
-                                                             int64_t *count_out, int scanned) {
+                                                             int64_t *count_out, int64_t *count_copy,
+                                                             int scanned) {
   const int64_t N = rl_count(n);
   __shared__ uint32_t lds[kRlBlock / kWave];
   __shared__ uint64_t lds64[kRlBlock / kWave];
@@ -319,6 +328,7 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
   // the workgroup holding the last id reports the number of distinct ids
   const int64_t last_tile = N > 0 ? (N - 1) / kRlTile : 0;
   if (static_cast<int64_t>(blockIdx.x) == last_tile && threadIdx.x == 0) {
+    if (count_copy) *count_copy = static_cast<int64_t>(tile_prefix + tile_total);
     *count_out = static_cast<int64_t>(tile_prefix + tile_total);
     __threadfence_system();
   }
@@ -364,7 +374,127 @@ __global__ __launch_bounds__(256) void rl_fill_concat_kernel(uint4 *tbl16, int64
   }
 }
 
-__global__ void rl_zero_count_kernel(int64_t *count_out) {
+// ---- small inputs: one workgroup, table in LDS -----------------------------
+// Up to kRlSmallMax ids the five passes are one launch: the ids and an index
+// table (slot = smallest index seen for the key that claimed it; keys are
+// compared through the LDS copy of the ids, so any id width works) live in
+// the workgroup's LDS, the grid-wide dependencies between the passes become
+// workgroup barriers, and no global atomic is issued. The table memory is
+// reused for the rank array once every first occurrence is known.
+constexpr int kRlSmallMax = 8192;
+constexpr int kRlSmallBlock = 1024;
+constexpr int kRlSmallItems = kRlSmallMax / kRlSmallBlock;
+constexpr int kRlSmallSlots = 2 * kRlSmallMax;
+static_assert(kRlSmallItems == 8, "the rank scan packs eight 16-bit counters into two words");
+
+template <bool SEGS>
+__global__ __launch_bounds__(kRlSmallBlock) void rl_small_kernel(const void *total_in, RlSegments segs,
+                                                                 void *total_out, int eb, RlCount n,
+                                                                 void *unique_out, void *labels_out,
+                                                                 int64_t *count_out, int64_t *count_copy) {
+  __shared__ int64_t keys[kRlSmallMax];
+  __shared__ uint32_t tbl[kRlSmallSlots];
+  __shared__ uint64_t scan_lds[kRlSmallBlock / kWave];
+  const int N = static_cast<int>(rl_count(n));
+  const int t = threadIdx.x;
+  for (int p = t; p < kRlSmallSlots; p += kRlSmallBlock) tbl[p] = 0xFFFFFFFFu;
+  // element i = j * kRlSmallBlock + t: coalesced loads and stores for every j
+  int64_t id[kRlSmallItems];
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const int i = j * kRlSmallBlock + t;
+    id[j] = 0;
+    if (i < N) {
+      if (SEGS) {
+        int sgm = 0;
+        while (sgm + 1 < segs.n && i >= segs.start[sgm + 1]) ++sgm;
+        id[j] = load_int(segs.ptr[sgm], i - segs.start[sgm], segs.bytes[sgm]);
+        store_int(total_out, i, eb, id[j]);
+      } else {
+        id[j] = load_int(total_in, i, eb);
+      }
+      keys[i] = id[j];
+    }
+  }
+  __syncthreads();
+  // insert: claim the first free slot of the probe sequence with the element's index, or lower the
+  // index of the slot that already stands for the same key
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const uint32_t i = j * kRlSmallBlock + t;
+    if (static_cast<int>(i) < N) {
+      uint32_t p = hash_id(id[j]) & (kRlSmallSlots - 1);
+      for (int probes = 0; probes < kRlSmallSlots; ++probes) {
+        uint32_t cur = tbl[p];
+        if (cur == 0xFFFFFFFFu) {
+          cur = atomicCAS(&tbl[p], 0xFFFFFFFFu, i);
+          if (cur == 0xFFFFFFFFu) break;
+        }
+        if (keys[cur] == id[j]) {
+          if (cur > i) atomicMin(&tbl[p], i);
+          break;
+        }
+        p = (p + 1) & (kRlSmallSlots - 1);
+      }
+    }
+  }
+  __syncthreads();
+  // first occurrence of every element; count the elements that are their own first occurrence,
+  // eight 16-bit counters (one per j) packed into two words
+  uint32_t first[kRlSmallItems];
+  uint64_t lo = 0, hi = 0;
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const uint32_t i = j * kRlSmallBlock + t;
+    first[j] = 0xFFFFFFFFu;
+    if (static_cast<int>(i) < N) {
+      uint32_t p = hash_id(id[j]) & (kRlSmallSlots - 1);
+      for (int probes = 0; probes < kRlSmallSlots; ++probes) {
+        const uint32_t cur = tbl[p];
+        if (cur == 0xFFFFFFFFu) break;  // cannot happen: every key was inserted
+        if (keys[cur] == id[j]) {
+          first[j] = cur;
+          break;
+        }
+        p = (p + 1) & (kRlSmallSlots - 1);
+      }
+      const uint64_t win = first[j] == i;
+      if (j < 4) lo += win << (16 * j); else hi += win << (16 * (j - 4));
+    }
+  }
+  // index order is j-major: rank = (winners of all smaller j) + (winners of this j in threads below)
+  uint64_t tot_lo, tot_hi;
+  const uint64_t ex_lo = block_exclusive_scan<uint64_t, kRlSmallBlock>(lo, scan_lds, &tot_lo);
+  const uint64_t ex_hi = block_exclusive_scan<uint64_t, kRlSmallBlock>(hi, scan_lds, &tot_hi);
+  // (the scans' barriers also mean every thread is done with the table: it becomes rank_of)
+  uint32_t below = 0;
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const uint32_t i = j * kRlSmallBlock + t;
+    const uint64_t ex = j < 4 ? ex_lo >> (16 * j) : ex_hi >> (16 * (j - 4));
+    const uint64_t tot = j < 4 ? tot_lo >> (16 * j) : tot_hi >> (16 * (j - 4));
+    if (static_cast<int>(i) < N && first[j] == i) {
+      const uint32_t rank = below + static_cast<uint32_t>(ex & 0xFFFF);
+      store_int(unique_out, rank, eb, id[j]);
+      tbl[i] = rank;
+    }
+    below += static_cast<uint32_t>(tot & 0xFFFF);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const int i = j * kRlSmallBlock + t;
+    if (i < N) store_int(labels_out, i, eb, static_cast<int64_t>(tbl[first[j]]));
+  }
+  if (t == 0) {
+    if (count_copy) *count_copy = static_cast<int64_t>(below);
+    *count_out = static_cast<int64_t>(below);
+    __threadfence_system();
+  }
+}
+
+__global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
+  if (count_copy) *count_copy = 0;
   *count_out = 0;
   __threadfence_system();
 }
@@ -395,14 +525,14 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
 static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
                         int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
                         void *labels_out, int64_t *count_out, void *stream, bool prepared = false,
-                        uint64_t prepared_nonce = 0) {
+                        uint64_t prepared_nonce = 0, int64_t *count_copy = nullptr) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
   SHMT_REQUIRE(count_out != nullptr, "shmt_relabel: count_out is null");
   hipStream_t s = as_stream(stream);
   if (N == 0) {
-    hipLaunchKernelGGL(rl_zero_count_kernel, dim3(1), dim3(1), 0, s, count_out);
+    hipLaunchKernelGGL(rl_zero_count_kernel, dim3(1), dim3(1), 0, s, count_out, count_copy);
     SHMT_LAUNCH_CHECK();
     return SHMT_OK;
   }
@@ -426,6 +556,18 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   uint64_t *wide_mark = reinterpret_cast<uint64_t *>(base + l.flag_off);
   const uint64_t nonce = prepared ? prepared_nonce : relabel_nonce();
   RlPath path{elem_bytes == 4 ? 1 : ((prepared || segs) ? 2 : 0), wide_mark, nonce};
+
+  if (N <= kRlSmallMax) {
+    if (segs)
+      hipLaunchKernelGGL(rl_small_kernel<true>, dim3(1), dim3(kRlSmallBlock), 0, s, nullptr, *segs,
+                         const_cast<void *>(total), elem_bytes, n, unique_out, labels_out, count_out,
+                         count_copy);
+    else
+      hipLaunchKernelGGL(rl_small_kernel<false>, dim3(1), dim3(kRlSmallBlock), 0, s, total, RlSegments{},
+                         nullptr, elem_bytes, n, unique_out, labels_out, count_out, count_copy);
+    SHMT_LAUNCH_CHECK();
+    return SHMT_OK;
+  }
 
   int rc = SHMT_OK;
   if (prepared) {
@@ -453,7 +595,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   }
   hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s,
                      total, elem_bytes, n, labels_out, partials, unique_out, rank_of, count_out,
-                     scanned);
+                     count_copy, scanned);
   SHMT_LAUNCH_CHECK();
   hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, labels_out,
                      elem_bytes, n, rank_of);
@@ -475,19 +617,20 @@ int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable 
   }
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "relabel: scratch must be 16-byte aligned");
   out->slots = static_cast<char *>(scratch) + l.table_off;
-  out->n16 = l.cap;
+  out->n16 = N <= kRlSmallMax ? 0 : l.cap;  // small inputs are relabelled in LDS: nothing to empty
   out->wide_mark = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + l.flag_off);
   out->nonce = relabel_nonce();
   return SHMT_OK;
 }
 
-int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const void *n_extra_dev,
-                          int n_extra_bytes, int elem_bytes, void *scratch, int64_t scratch_bytes,
-                          void *unique_out, void *labels_out, int64_t *count_out, uint64_t nonce,
-                          hipStream_t stream) {
-  return relabel_impl(total, nullptr, n_bound, RlCount{n_fixed, n_extra_dev, n_extra_bytes, n_bound},
-                      elem_bytes, scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true,
-                      nonce);
+int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const int64_t *n_fixed_dev,
+                          const void *n_extra_dev, int n_extra_bytes, int elem_bytes, void *scratch,
+                          int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
+                          int64_t *count_copy, uint64_t nonce, hipStream_t stream) {
+  return relabel_impl(total, nullptr, n_bound,
+                      RlCount{n_fixed, n_fixed_dev, n_extra_dev, n_extra_bytes, n_bound}, elem_bytes,
+                      scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true, nonce,
+                      count_copy);
 }
 
 }  // namespace shmt
@@ -497,7 +640,7 @@ extern "C" {
 int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
                  void *stream) {
-  return relabel_impl(total, nullptr, N, RlCount{N, nullptr, 8, N}, elem_bytes, scratch, scratch_bytes,
+  return relabel_impl(total, nullptr, N, RlCount{N, nullptr, nullptr, 8, N}, elem_bytes, scratch, scratch_bytes,
                       unique_out, labels_out, count_out, stream);
 }
 
@@ -529,7 +672,7 @@ int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, 
     segs.bytes[i] = 8;
   }
   SHMT_REQUIRE(N == 0 || total_out != nullptr, "shmt_relabel_segments: total_out is null");
-  RlCount n{N, nullptr, 8, N};
+  RlCount n{N, nullptr, nullptr, 8, N};
   if (last_len_dev) {
     // the last segment's true length lives on the device; N stays the bound
     n.fixed = N - seg_lens[nseg - 1];

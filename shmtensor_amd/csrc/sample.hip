@@ -21,7 +21,11 @@
 //        the relabel input, pick adds the tile offsets itself (one short
 //        totals kernel instead of two passes over sub_indptr), writes every
 //        sampled id into the relabel input too, empties the relabel table and
-//        marks whether any id falls outside 32 bits.
+//        marks whether any id falls outside 32 bits. The number of seeds may
+//        itself live in device memory (the count a previous hop produced):
+//        launches and buffers are then sized for a bound and every kernel
+//        clamps to the true number, so consecutive hops queue without a host
+//        wait between them.
 #include "common.h"
 #include "hashmap.h"
 #include "hashmap_dev.h"
@@ -57,13 +61,23 @@ struct PlanArgs {
   int replace;
   void *seed_copy;      // optional: seeds widened to seed_copy_bytes (head of a relabel input)
   int seed_copy_bytes;
+  const int64_t *S_len;  // optional: true number of seeds in device memory, S is then its bound
+  uint64_t *total_word;  // optional (single-workgroup form): second copy of the total, in device memory
 };
+
+// Number of seeds a kernel works on: the host's figure, or the device-side
+// count clamped to it.
+__device__ __forceinline__ int64_t seed_count(int64_t bound, const int64_t *len) {
+  if (!len) return bound;
+  const int64_t n = *len;
+  return n < 0 ? 0 : (n < bound ? n : bound);
+}
 
 // MODE 0: no cache; 1: wide map; 2: narrow map.
 template <int MODE>
-__device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
+__device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t S, int64_t i) {
   // called by whole waves; lanes past S use a harmless key and produce cnt 0
-  const bool live = i < a.S;
+  const bool live = i < S;
   int64_t node = live ? load_int(a.seeds, i, a.seed_bytes) : -1;
   if (live && a.seed_copy) store_int(a.seed_copy, i, a.seed_copy_bytes, node);
   int64_t slot = -1;
@@ -87,17 +101,19 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t i) {
 template <int MODE>
 __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
+  const int64_t S = seed_count(a.S, a.S_len);
   uint64_t carry = 0;
-  for (int64_t base = 0; base < a.S; base += kPlanBlock) {
+  for (int64_t base = 0; base < S; base += kPlanBlock) {
     const int64_t i = base + threadIdx.x;
-    const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, i));
+    const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, S, i));
     uint64_t total;
     const uint64_t ex = block_exclusive_scan<uint64_t, kPlanBlock>(cnt, lds, &total);
-    if (i < a.S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(carry + ex));
+    if (i < S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(carry + ex));
     carry += total;
   }
   if (threadIdx.x == 0) {
-    store_int(a.sub_indptr, a.S, a.ptr_bytes, static_cast<int64_t>(carry));
+    store_int(a.sub_indptr, S, a.ptr_bytes, static_cast<int64_t>(carry));
+    if (a.total_word) *a.total_word = carry;
     *a.nnz_out = static_cast<int64_t>(carry);
     __threadfence_system();
   }
@@ -107,11 +123,12 @@ __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
 template <int MODE>
 __global__ __launch_bounds__(kPlanBlock) void plan_tile_kernel(PlanArgs a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
+  const int64_t S = seed_count(a.S, a.S_len);
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kPlanBlock + threadIdx.x;
-  const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, i));
+  const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, S, i));
   uint64_t total;
   const uint64_t ex = block_exclusive_scan<uint64_t, kPlanBlock>(cnt, lds, &total);
-  if (i < a.S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(ex));
+  if (i < S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(ex));
   if (threadIdx.x == 0) {
     a.partials[blockIdx.x] = total;
     if (blockIdx.x == 0) a.partials[gridDim.x] = 0;  // becomes the grand total after the scan
@@ -143,9 +160,11 @@ __global__ __launch_bounds__(256) void add_tile_offsets_kernel(void *data, int e
 // (partials[nb] becomes the grand total) and publishes the total; the tile
 // offsets themselves are added by the pick kernel.
 __global__ __launch_bounds__(1024) void plan_totals_kernel(uint64_t *partials, int64_t nb,
-                                                           void *sub_indptr, int ptr_bytes, int64_t S,
+                                                           void *sub_indptr, int ptr_bytes,
+                                                           int64_t S_bound, const int64_t *S_len,
                                                            int64_t *nnz_out) {
   __shared__ uint64_t lds[1024 / kWave];
+  const int64_t S = seed_count(S_bound, S_len);
   uint64_t carry = 0;
   for (int64_t base = 0; base < nb; base += 1024) {
     const int64_t i = base + threadIdx.x;
@@ -184,9 +203,9 @@ struct PickArgs {
   // fused hop only (HOP kernels):
   void *sub_indptr_rw;          // tile-local offsets in, final offsets out
   const uint64_t *tile_prefix;  // scanned totals of the 1024-seed tiles, or null when offsets are final
-  void *copy_out;               // second copy of every sampled id, widened to copy_bytes ...
-  int64_t copy_base;            // ... at copy_out[copy_base + offset]
-  int copy_bytes;
+  const int64_t *S_len;         // optional: true number of seeds in device memory, S is then its bound
+  void *copy_out;               // second copy of every sampled id, widened to copy_bytes, at
+  int copy_bytes;               // copy_out[number of seeds + offset]: the relabel input after the seeds
   uint4 *clear;                 // clear_n 16-byte words set to all ones (the relabel table)
   int64_t clear_n;
   uint64_t *wide_mark;          // receives wide_nonce when a seed or a sampled id lies outside [0, 2^32)
@@ -212,10 +231,10 @@ __device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, boo
 }
 
 template <bool HOP>
-__device__ __forceinline__ void pick_store(const PickArgs &a, int64_t pos, int64_t v) {
+__device__ __forceinline__ void pick_store(const PickArgs &a, int64_t S, int64_t pos, int64_t v) {
   store_int(a.out, pos, a.idx_bytes, v);
   if (HOP) {
-    store_int(a.copy_out, a.copy_base + pos, a.copy_bytes, v);
+    store_int(a.copy_out, S + pos, a.copy_bytes, v);
     note_wide_id(a, v);
   }
 }
@@ -247,10 +266,11 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
   const int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + threadIdx.x / kWave;
   const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
   const int k = static_cast<int>(a.k);
+  const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
 
-  for (int64_t s0 = wave * groups_per_wave; s0 < a.S; s0 += nwaves * groups_per_wave) {
+  for (int64_t s0 = wave * groups_per_wave; s0 < S; s0 += nwaves * groups_per_wave) {
     const int64_t s = s0 + (lane >> a.log2_group);
-    if (s >= a.S) continue;  // uniform within the group
+    if (s >= S) continue;  // uniform within the group
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
     const int64_t optr = pick_offset<HOP>(a, s, gl == 0);
@@ -259,10 +279,10 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
       if (gl < k) {
         const int64_t node = load_int(a.seeds, s, a.seed_bytes);
         const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
-        pick_store<HOP>(a, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
+        pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
-      if (gl < deg) pick_store<HOP>(a, optr + gl, load_adj(a, p.begin, gl));
+      if (gl < deg) pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, gl));
     } else {
       // Floyd: for J = deg-k .. deg-1 draw t in [0, J]; take t unless already
       // taken, then take J. Draws in parallel, resolution in k ballot steps.
@@ -277,7 +297,7 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
         const bool taken = group_ballot_dyn(gl < step && mine == ts, G) != 0;
         if (gl == step) mine = taken ? (deg - k + step) : ts;
       }
-      if (gl < k) pick_store<HOP>(a, optr + gl, load_adj(a, p.begin, mine));
+      if (gl < k) pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, mine));
     }
   }
 }
@@ -292,7 +312,8 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
   pick_clear<HOP>(a);
   const int lane = threadIdx.x;
   const int64_t k = a.k;
-  for (int64_t s = blockIdx.x; s < a.S; s += gridDim.x) {
+  const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
+  for (int64_t s = blockIdx.x; s < S; s += gridDim.x) {
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
     const int64_t optr = pick_offset<HOP>(a, s, lane == 0);
@@ -302,10 +323,10 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
       for (int64_t j = lane; j < k; j += kWave) {
         const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(j),
                                        static_cast<uint64_t>(deg));
-        pick_store<HOP>(a, optr + j, load_adj(a, p.begin, static_cast<int64_t>(r)));
+        pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
-      for (int64_t j = lane; j < deg; j += kWave) pick_store<HOP>(a, optr + j, load_adj(a, p.begin, j));
+      for (int64_t j = lane; j < deg; j += kWave) pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, j));
     } else {
       for (int64_t step = 0; step < k; ++step) {
         const int64_t J = deg - k + step;
@@ -330,7 +351,7 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
         int64_t c = 0;
         if (j < k) c = IN_LDS ? chosen_lds[j] : load_int(a.out, optr + j, a.idx_bytes);
         __syncthreads();
-        if (j < k) pick_store<HOP>(a, optr + j, load_adj(a, p.begin, c));
+        if (j < k) pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, c));
       }
       __syncthreads();
     }
@@ -424,7 +445,9 @@ int64_t shmt_sample_plan_bytes(int64_t S) {
 struct PlanHopExtras {
   void *seed_copy;
   int seed_copy_bytes;
+  const int64_t *S_len;             // true number of seeds in device memory, or null
   const uint64_t *tile_prefix_out;
+  const uint64_t *total_out;        // where the kernels leave the total (nnz) in device memory
 };
 
 static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr,
@@ -466,7 +489,13 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   a.replace = replace ? 1 : 0;
   a.seed_copy = hop ? hop->seed_copy : nullptr;
   a.seed_copy_bytes = hop ? hop->seed_copy_bytes : 8;
-  if (hop) hop->tile_prefix_out = nullptr;
+  a.S_len = hop ? hop->S_len : nullptr;
+  const int64_t tiles = (S + kPlanBlock - 1) / kPlanBlock;
+  a.total_word = hop && S > 0 ? a.partials + tiles : nullptr;  // where plan_totals_kernel leaves it too
+  if (hop) {
+    hop->tile_prefix_out = nullptr;
+    hop->total_out = a.total_word;
+  }
   const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
 
   if (S <= kPlanSingleMax) {
@@ -489,7 +518,7 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   SHMT_LAUNCH_CHECK();
   if (hop) {
     hipLaunchKernelGGL(plan_totals_kernel, dim3(1), dim3(1024), 0, s, a.partials, nb, sub_indptr,
-                       ptr_bytes, S, nnz_out);
+                       ptr_bytes, S, a.S_len, nnz_out);
     SHMT_LAUNCH_CHECK();
     hop->tile_prefix_out = a.partials;
     return SHMT_OK;
@@ -516,8 +545,8 @@ int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr
 struct PickHopExtras {
   void *sub_indptr_rw;
   const uint64_t *tile_prefix;
+  const int64_t *S_len;
   void *copy_out;
-  int64_t copy_base;
   int copy_bytes;
   uint4 *clear;
   int64_t clear_n;
@@ -583,8 +612,8 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   }
   a.sub_indptr_rw = nullptr;
   a.tile_prefix = nullptr;
+  a.S_len = nullptr;
   a.copy_out = nullptr;
-  a.copy_base = 0;
   a.copy_bytes = 8;
   a.clear = nullptr;
   a.clear_n = 0;
@@ -594,8 +623,8 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   if (!hop) return pick_launch<false>(a, s);
   a.sub_indptr_rw = hop->sub_indptr_rw;
   a.tile_prefix = hop->tile_prefix;
+  a.S_len = hop->S_len;
   a.copy_out = hop->copy_out;
-  a.copy_base = hop->copy_base;
   a.copy_bytes = hop->copy_bytes;
   a.clear = hop->clear;
   a.clear_n = hop->clear_n;
@@ -612,13 +641,13 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
                    ptr_bytes, plan, sub_indices, rng_seed, rng_stream, stream, nullptr);
 }
 
-int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
+static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
                     const void *cache_indptr, const void *cache_indices, const shmt_hashmap_t *map,
-                    const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
-                    uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr, void *sub_indices,
-                    void *plan, int64_t plan_bytes, int elem_bytes, void *total_out, void *scratch,
-                    int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *nnz_out,
-                    int64_t *count_out, void *stream) {
+                    const void *seeds, int seed_bytes, int64_t S, const int64_t *S_len, int64_t k,
+                    int replace, uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr,
+                    void *sub_indices, void *plan, int64_t plan_bytes, int elem_bytes, void *total_out,
+                    void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
+                    int64_t *nnz_out, int64_t *count_out, int64_t *count_copy, void *stream) {
   SHMT_REQUIRE(S >= 1 && k >= 1, "shmt_sample_hop: S and num_picks must be >= 1");
   SHMT_REQUIRE(k <= ((1ll << 31) - 1 - S) / S, "shmt_sample_hop: S * (num_picks + 1) must be < 2^31");
   SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes) && width_ok(elem_bytes),
@@ -631,20 +660,47 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
   RelabelTable table;
   int rc = relabel_table(n_max, scratch, scratch_bytes, &table);
   if (rc) return rc;
-  PlanHopExtras plan_hop{total_out, elem_bytes, nullptr};
+  PlanHopExtras plan_hop{total_out, elem_bytes, S_len, nullptr, nullptr};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
                  plan_bytes, nnz_out, stream, &plan_hop);
   if (rc) return rc;
-  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, total_out, S, elem_bytes,
+  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, S_len, total_out, elem_bytes,
                                static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                  plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
   if (rc) return rc;
   // [seeds, sub_indices] is in total_out and the table is empty: the relabel passes follow, with the
-  // number of sampled ids read from sub_indptr[S]
-  return launch_relabel_passes(total_out, n_max, S, static_cast<const char *>(sub_indptr) + S * ptr_bytes,
-                               ptr_bytes, elem_bytes, scratch, scratch_bytes, unique_out, labels_out,
-                               count_out, table.nonce, as_stream(stream));
+  // number of sampled ids (and of seeds, when it is a device-side figure) read from device memory
+  return launch_relabel_passes(total_out, n_max, S, S_len, plan_hop.total_out, 8, elem_bytes, scratch,
+                               scratch_bytes, unique_out, labels_out, count_out, count_copy, table.nonce,
+                               as_stream(stream));
+}
+
+int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
+                    const void *cache_indptr, const void *cache_indices, const shmt_hashmap_t *map,
+                    const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
+                    uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr, void *sub_indices,
+                    void *plan, int64_t plan_bytes, int elem_bytes, void *total_out, void *scratch,
+                    int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *nnz_out,
+                    int64_t *count_out, void *stream) {
+  return hop_impl(indptr, ptr_bytes, indices, idx_bytes, cache_indptr, cache_indices, map, seeds, seed_bytes,
+                  S, nullptr, k, replace, rng_seed, rng_stream, sub_indptr, sub_indices, plan, plan_bytes,
+                  elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out, count_out,
+                  nullptr, stream);
+}
+
+int shmt_sample_hop_chained(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
+                            const void *cache_indptr, const void *cache_indices,
+                            const shmt_hashmap_t *map, const void *seeds, int seed_bytes,
+                            int64_t max_seeds, const int64_t *seeds_len, int64_t k, int replace,
+                            uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr, void *sub_indices,
+                            void *plan, int64_t plan_bytes, int elem_bytes, void *total_out,
+                            void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
+                            int64_t *nnz_out, int64_t *count_out, int64_t *count_dev_out, void *stream) {
+  return hop_impl(indptr, ptr_bytes, indices, idx_bytes, cache_indptr, cache_indices, map, seeds, seed_bytes,
+                  max_seeds, seeds_len, k, replace, rng_seed, rng_stream, sub_indptr, sub_indices, plan,
+                  plan_bytes, elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out,
+                  count_out, count_dev_out, stream);
 }
 
 int shmt_subcsr_plan(const void *indptr, int ptr_bytes, const void *seeds, int seed_bytes,

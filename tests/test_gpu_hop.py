@@ -372,3 +372,80 @@ def test_sample_blocks_fetch_arguments(capi):
                                  max_rows=-1)
     with pytest.raises(RuntimeError):                      # pageable host memory
         capi.sample_blocks_fetch(indptr, indices, None, None, None, seeds, [5], False, table.cpu(), None, None)
+
+
+@pytest.mark.parametrize("cached", [False, True])
+@pytest.mark.parametrize("S,picks,replace", [(200, (3, 4, 5), 0), (1500, (6, 3), 0), (40, (70, 2), 0),
+                                             (300, (4, 4), 1)])
+def test_c_abi_chained_hops_need_no_host_wait(cabi, cached, S, picks, replace):
+    """shmt_sample_hop_chained: every hop takes its number of seeds from the device-side count of
+    the hop before it and all hops are queued before anything is read back; results equal those
+    of shmt_sample_hop called hop by hop with the host reading each count."""
+    lib = cabi.load()
+    indptr, indices = _graph(scale=13, ptr_dt=torch.int64, idx_dt=torch.int32)
+    indptr, indices = indptr.cuda(), indices.cuda()
+    n = indptr.numel() - 1
+    stream = cabi.current_stream()
+    gp = gi = hnd = None
+    keep = []
+    if cached:
+        hot = torch.randperm(n, generator=torch.Generator().manual_seed(2))[: n // 2].cuda()
+        deg = indptr[hot + 1] - indptr[hot]
+        gp = torch.cat([torch.zeros(1, dtype=torch.int64).cuda(), torch.cumsum(deg, 0)])
+        gi = torch.cat([indices[indptr[v]:indptr[v + 1]] for v in hot.tolist()])
+        nbytes = lib.shmt_hashmap_table_bytes(hot.numel(), 0.8, 8, 8)
+        keep.append(torch.empty(nbytes, dtype=torch.uint8).cuda())
+        hnd = ctypes.c_void_p()
+        cabi.check(lib.shmt_hashmap_create(ctypes.byref(hnd), hot.data_ptr(), torch.arange(hot.numel()).cuda().data_ptr(),
+                                           hot.numel(), 8, 8, 0.8, keep[0].data_ptr(), nbytes, stream))
+    seeds0 = torch.randperm(n, generator=torch.Generator().manual_seed(S))[:S].cuda()
+
+    def buffers(s_max, k):
+        n_max = s_max + s_max * k
+        return dict(sp=torch.full((s_max + 1,), -1, dtype=torch.int64).cuda(),
+                    si=torch.empty(s_max * k, dtype=torch.int32).cuda(),
+                    plan=torch.empty(lib.shmt_sample_plan_bytes(s_max), dtype=torch.uint8).cuda(),
+                    total=torch.empty(n_max, dtype=torch.int64).cuda(), unique=torch.empty(n_max, dtype=torch.int64).cuda(),
+                    labels=torch.empty(n_max, dtype=torch.int64).cuda(),
+                    scratch=torch.empty(lib.shmt_relabel_scratch_bytes(n_max), dtype=torch.uint8).cuda(),
+                    nnz=torch.full((1,), -1, dtype=torch.int64).cuda(), count=torch.full((1,), -1, dtype=torch.int64).cuda(),
+                    count_dev=torch.full((1,), -1, dtype=torch.int64).cuda())
+
+    def graph_args():
+        return (indptr.data_ptr(), 8, indices.data_ptr(), 4, gp.data_ptr() if cached else None,
+                gi.data_ptr() if cached else None, hnd)
+
+    # chained: nothing is read back until every hop is queued
+    chained, seeds, s_max, s_len = [], seeds0, S, None
+    for hop, k in enumerate(picks):
+        b = buffers(s_max, k)
+        cabi.check(lib.shmt_sample_hop_chained(*graph_args(), seeds.data_ptr(), 8, s_max, s_len, k, replace, 42, hop,
+                                               b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(),
+                                               b["plan"].numel(), 8, b["total"].data_ptr(), b["scratch"].data_ptr(),
+                                               b["scratch"].numel(), b["unique"].data_ptr(), b["labels"].data_ptr(),
+                                               b["nnz"].data_ptr(), b["count"].data_ptr(), b["count_dev"].data_ptr(),
+                                               stream))
+        chained.append(b)
+        seeds, s_len, s_max = b["unique"], b["count_dev"].data_ptr(), s_max + s_max * k
+    torch.cuda.synchronize()
+    # hop by hop, the host reading each count
+    seeds = seeds0
+    for hop, k in enumerate(picks):
+        s_now = seeds.numel()
+        b = buffers(s_now, k)
+        cabi.check(lib.shmt_sample_hop(*graph_args(), seeds.data_ptr(), 8, s_now, k, replace, 42, hop,
+                                       b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(), b["plan"].numel(), 8,
+                                       b["total"].data_ptr(), b["scratch"].data_ptr(), b["scratch"].numel(),
+                                       b["unique"].data_ptr(), b["labels"].data_ptr(), b["nnz"].data_ptr(),
+                                       b["count"].data_ptr(), stream))
+        torch.cuda.synchronize()
+        c = chained[hop]
+        nnz, u = int(b["nnz"].item()), int(b["count"].item())
+        assert (int(c["nnz"].item()), int(c["count"].item()), int(c["count_dev"].item())) == (nnz, u, u), hop
+        assert torch.equal(c["sp"][:s_now + 1], b["sp"]) and torch.equal(c["si"][:nnz], b["si"][:nnz]), hop
+        assert torch.equal(c["total"][:s_now + nnz], b["total"][:s_now + nnz]), hop
+        assert torch.equal(c["unique"][:u], b["unique"][:u]), hop
+        assert torch.equal(c["labels"][:s_now + nnz], b["labels"][:s_now + nnz]), hop
+        seeds = b["unique"][:u].clone()
+    if hnd is not None:
+        lib.shmt_hashmap_destroy(hnd)

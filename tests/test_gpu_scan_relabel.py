@@ -51,7 +51,10 @@ def test_relabel_reference_kat(capi):
     assert isinstance(labels, list) and u.dtype == torch.int64
 
 
-@pytest.mark.parametrize("n", [1, 2, 7, 8, 9, 255, 256, 257, 2047, 2048, 2049, 100_000, 3_000_000])
+# 5,460 / 5,461 / 5,462: 8,191 / 8,192 / 8,194 ids in all, either side of the largest input that one
+# workgroup relabels in LDS
+@pytest.mark.parametrize("n", [1, 2, 7, 8, 9, 255, 256, 257, 2047, 2048, 2049, 5460, 5461, 5462, 100_000,
+                               3_000_000])
 @pytest.mark.parametrize("dt", [np.int32, np.int64])
 def test_relabel_matches_oracle(capi, oracle, n, dt):
     rng = np.random.default_rng(n)
@@ -65,7 +68,7 @@ def test_relabel_matches_oracle(capi, oracle, n, dt):
     assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
 
 
-@pytest.mark.parametrize("n", [9, 300, 2049, 100_000, 1_500_000])
+@pytest.mark.parametrize("n", [9, 300, 2049, 5461, 5462, 100_000, 1_500_000])
 @pytest.mark.parametrize("odd", ["one_wide_id_at_the_end", "many_wide", "negative", "uint32_max", "mixed_widths"])
 def test_relabel_id_ranges_select_the_table_format(capi, oracle, n, odd):
     """8-byte ids that all fit 32 bits go through the packed table, anything else through
@@ -146,3 +149,27 @@ def test_relabel_full_size_properties(capi):
     first = torch.full((u.numel(),), x.numel(), device="cuda", dtype=torch.int64)
     first.scatter_reduce_(0, l, torch.arange(x.numel(), device="cuda"), reduce="amin")
     assert bool((first[1:] > first[:-1]).all())
+
+
+@pytest.mark.parametrize("n", [1, 100, 8191, 8192, 8193, 50_000])
+@pytest.mark.parametrize("bytes_", [4, 8])
+def test_c_abi_relabel_of_one_array(cabi, oracle, n, bytes_):
+    """shmt_relabel (one id array, no concatenation) through raw pointers, on both sides of the
+    size up to which one workgroup does all passes."""
+    lib = cabi.load()
+    rng = np.random.default_rng(n + bytes_)
+    ids = rng.integers(0, max(2, n // 2), size=n).astype(np.int32 if bytes_ == 4 else np.int64)
+    if bytes_ == 8:
+        ids[::3] += 2**33                                  # ids beyond 32 bits
+        ids[1::11] = -ids[1::11] - 2                       # and negative ones (-1 is the reserved value)
+    total = torch.from_numpy(ids).cuda()
+    unique, labels = torch.empty_like(total), torch.empty_like(total)
+    sbytes = lib.shmt_relabel_scratch_bytes(n)
+    scratch = torch.empty(sbytes, dtype=torch.uint8).cuda()
+    count = torch.full((1,), -1, dtype=torch.int64).cuda()
+    cabi.check(lib.shmt_relabel(total.data_ptr(), n, bytes_, scratch.data_ptr(), sbytes, unique.data_ptr(),
+                                labels.data_ptr(), count.data_ptr(), cabi.current_stream()))
+    torch.cuda.synchronize()
+    eu, (el,) = oracle.relabel([ids])
+    assert int(count.item()) == eu.size
+    assert np.array_equal(unique[:eu.size].cpu().numpy(), eu) and np.array_equal(labels.cpu().numpy(), el)
