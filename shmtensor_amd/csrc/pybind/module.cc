@@ -766,7 +766,7 @@ BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<in
 }
 
 // Multi-hop sampling of several independent seed batches. Every batch is a
-// chain of short, latency-bound kernels with two host reads of a size per hop,
+// chain of short, latency-bound kernels with a host read of the sizes at its end,
 // so one batch alone leaves most of the GPU idle. Here up to `max_in_flight`
 // batches advance at the same time: each is driven by its own host thread on
 // its own stream (default priority, the same streams every call), so both the

@@ -108,3 +108,54 @@ def test_fused_hop_replays_in_a_hip_graph(capi, cabi):
         assert nnz == want[1].numel() and u == want[2].numel(), it
         assert torch.equal(buf["sp"], want[0]) and torch.equal(buf["si"][:nnz], want[1]), it
         assert torch.equal(buf["unique"][:u], want[2]) and torch.equal(buf["labels"][S:S + nnz], want[3]), it
+
+
+def test_a_whole_batch_of_chained_hops_replays_in_a_hip_graph(capi, cabi):
+    """Three hops chained on the device (each takes its seeds and their number from the hop before) are
+    captured as ONE graph and replayed on new seed batches; every replay equals sample_blocks run eagerly."""
+    from shmtensor_amd.synthetic import rmat_csr
+    lib = cabi.load()
+    indptr, indices = rmat_csr(13, 12, seed=5)
+    n = indptr.numel() - 1
+    S, picks = 500, (3, 4, 6)
+    seeds = torch.zeros(S, dtype=torch.int64, device="cuda")
+    hops, s_max = [], S
+    for k in picks:
+        n_max = s_max + s_max * k
+        hops.append(dict(s_max=s_max, k=k,
+                         sp=torch.empty(s_max + 1, dtype=torch.int64, device="cuda"),
+                         si=torch.empty(s_max * k, dtype=indices.dtype, device="cuda"),
+                         plan=torch.empty(lib.shmt_sample_plan_bytes(s_max), dtype=torch.uint8, device="cuda"),
+                         total=torch.empty(n_max, dtype=torch.int64, device="cuda"),
+                         unique=torch.empty(n_max, dtype=torch.int64, device="cuda"),
+                         labels=torch.empty(n_max, dtype=torch.int64, device="cuda"),
+                         scratch=torch.empty(lib.shmt_relabel_scratch_bytes(n_max), dtype=torch.uint8, device="cuda"),
+                         nnz=torch.zeros(1, dtype=torch.int64, device="cuda"), count=torch.zeros(1, dtype=torch.int64, device="cuda"),
+                         count_dev=torch.zeros(1, dtype=torch.int64, device="cuda")))
+        s_max = n_max
+    ib = indices.element_size()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        src, src_len = seeds, None
+        for hop, b in enumerate(hops):
+            cabi.check(lib.shmt_sample_hop_chained(
+                indptr.data_ptr(), 8, indices.data_ptr(), ib, None, None, None, src.data_ptr(), 8, b["s_max"], src_len,
+                b["k"], 0, 77, hop, b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(), b["plan"].numel(), 8,
+                b["total"].data_ptr(), b["scratch"].data_ptr(), b["scratch"].numel(), b["unique"].data_ptr(),
+                b["labels"].data_ptr(), b["nnz"].data_ptr(), b["count"].data_ptr(), b["count_dev"].data_ptr(),
+                cabi.current_stream()))
+            src, src_len = b["unique"], b["count_dev"].data_ptr()
+    g = torch.Generator().manual_seed(3)
+    for it in range(4):
+        seeds.copy_(torch.randperm(n, generator=g)[:S])
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = capi.sample_blocks(indptr, indices, None, None, None, [seeds], list(picks), False, seeds_rng=[77])[0]
+        s_now = S
+        for b, (sp, si, uniq, rel) in zip(hops, want):
+            nnz, u = int(b["nnz"].item()), int(b["count"].item())
+            assert (nnz, u) == (si.numel(), uniq.numel()), it
+            assert torch.equal(b["sp"][:s_now + 1], sp) and torch.equal(b["si"][:nnz], si), it
+            assert torch.equal(b["unique"][:u], uniq) and torch.equal(b["labels"][s_now:s_now + nnz], rel), it
+            s_now = u
