@@ -276,7 +276,9 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices,
  * out for the true number of seeds S': sub_indptr has S' + 1 entries,
  * total_out / labels_out hold the S' seeds followed by the sampled ids.
  * count_dev_out (device memory, may be NULL) receives the number of
- * distinct ids like count_out does.                                        */
+ * distinct ids like count_out does. rng_seed_dev (device memory, may be
+ * NULL) overrides rng_seed with a value read by the kernels, so that a
+ * captured launch sequence can be replayed with another seed.              */
 int shmt_sample_hop_chained(const void *indptr, int ptr_bytes,
                             const void *indices, int idx_bytes,
                             const void *cache_indptr,
@@ -284,14 +286,36 @@ int shmt_sample_hop_chained(const void *indptr, int ptr_bytes,
                             const shmt_hashmap_t *map, const void *seeds,
                             int seed_bytes, int64_t max_seeds,
                             const int64_t *seeds_len, int64_t k, int replace,
-                            uint64_t rng_seed, uint32_t rng_stream,
-                            void *sub_indptr, void *sub_indices, void *plan,
+                            uint64_t rng_seed, const uint64_t *rng_seed_dev,
+                            uint32_t rng_stream, void *sub_indptr,
+                            void *sub_indices, void *plan,
                             int64_t plan_bytes, int elem_bytes,
                             void *total_out, void *scratch,
                             int64_t scratch_bytes, void *unique_out,
                             void *labels_out, int64_t *nnz_out,
                             int64_t *count_out, int64_t *count_dev_out,
                             void *stream);
+
+/* Replaying a mini-batch. The hops of a batch, queued with
+ * shmt_sample_hop_chained on fixed buffers, never wait for the host, so the
+ * whole sequence can be captured once as a HIP graph and replayed for every
+ * further batch with one launch instead of one per kernel (the reference
+ * issues each kernel of each hop from the host and waits in between,
+ * python/shmtensor/sampling.py:128-143). shmt_capture_begin starts recording
+ * what is queued on `stream` (not the null stream); shmt_capture_end stops and
+ * returns an executable graph; shmt_graph_launch replays it on a stream;
+ * shmt_graph_destroy frees it. shmt_stage_seeds is the eager step before a
+ * replay: it copies the n seeds of the next batch into the captured
+ * sequence's input buffer (`staged`, widened from seed_bytes to staged_bytes)
+ * and stores n and the batch's RNG seed where the captured kernels read them
+ * (seeds_len / rng_seed_dev of the first / every hop).                      */
+int shmt_capture_begin(void *stream);
+int shmt_capture_end(void *stream, void **graph_exec_out);
+int shmt_graph_launch(void *graph_exec, void *stream);
+void shmt_graph_destroy(void *graph_exec);
+int shmt_stage_seeds(const void *seeds, int seed_bytes, int64_t n, void *staged,
+                     int staged_bytes, int64_t *len_out, uint64_t rng_seed,
+                     uint64_t *rng_seed_out, void *stream);
 
 /* Cached sub-CSR: CreateCacheCSR, src/cache_graph_sampling.cu:455-492
  * (CSRIndicesCopyKernel :428-453). Step 1 writes

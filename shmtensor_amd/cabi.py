@@ -44,8 +44,13 @@ SIGNATURES = {
     "shmt_sample_hop": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int, _i64, _i64, _int, _c.c_uint64,
                                _c.c_uint32, _vp, _vp, _vp, _i64, _int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "shmt_sample_hop_chained": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int, _i64, _vp, _i64, _int,
-                                       _c.c_uint64, _c.c_uint32, _vp, _vp, _vp, _i64, _int, _vp, _vp, _i64, _vp,
-                                       _vp, _vp, _vp, _vp, _vp]),
+                                       _c.c_uint64, _vp, _c.c_uint32, _vp, _vp, _vp, _i64, _int, _vp, _vp, _i64,
+                                       _vp, _vp, _vp, _vp, _vp, _vp]),
+    "shmt_capture_begin": (_int, [_vp]),
+    "shmt_capture_end": (_int, [_vp, _c.POINTER(_vp)]),
+    "shmt_graph_launch": (_int, [_vp, _vp]),
+    "shmt_graph_destroy": (None, [_vp]),
+    "shmt_stage_seeds": (_int, [_vp, _int, _i64, _vp, _int, _vp, _c.c_uint64, _vp, _vp]),
     "shmt_subcsr_plan": (_int, [_vp, _int, _vp, _int, _i64, _vp, _vp, _i64, _vp, _vp]),
     "shmt_subcsr_copy": (_int, [_vp, _vp, _int, _int, _vp, _int, _i64, _vp, _i64, _vp, _vp]),
 }

@@ -204,6 +204,7 @@ struct PickArgs {
   void *sub_indptr_rw;          // tile-local offsets in, final offsets out
   const uint64_t *tile_prefix;  // scanned totals of the 1024-seed tiles, or null when offsets are final
   const int64_t *S_len;         // optional: true number of seeds in device memory, S is then its bound
+  const uint64_t *rng_seed_dev; // optional: the RNG seed lives in device memory (replayed launch sequences)
   void *copy_out;               // second copy of every sampled id, widened to copy_bytes, at
   int copy_bytes;               // copy_out[number of seeds + offset]: the relabel input after the seeds
   uint4 *clear;                 // clear_n 16-byte words set to all ones (the relabel table)
@@ -267,6 +268,7 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
   const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
   const int k = static_cast<int>(a.k);
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
+  const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
 
   for (int64_t s0 = wave * groups_per_wave; s0 < S; s0 += nwaves * groups_per_wave) {
     const int64_t s = s0 + (lane >> a.log2_group);
@@ -278,7 +280,7 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
     if (a.replace) {
       if (gl < k) {
         const int64_t node = load_int(a.seeds, s, a.seed_bytes);
-        const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
+        const uint64_t r = sample_draw(rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
         pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
       const int64_t node = load_int(a.seeds, s, a.seed_bytes);
       int64_t t = 0;
       if (gl < k)
-        t = static_cast<int64_t>(sample_draw(a.rng_seed, a.rng_stream, node, gl,
+        t = static_cast<int64_t>(sample_draw(rng_seed, a.rng_stream, node, gl,
                                              static_cast<uint64_t>(deg - k + gl + 1)));
       int64_t mine = -1;
       for (int step = 0; step < k; ++step) {
@@ -313,6 +315,7 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
   const int lane = threadIdx.x;
   const int64_t k = a.k;
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
+  const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
   for (int64_t s = blockIdx.x; s < S; s += gridDim.x) {
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
@@ -321,7 +324,7 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
     const int64_t node = load_int(a.seeds, s, a.seed_bytes);
     if (a.replace) {
       for (int64_t j = lane; j < k; j += kWave) {
-        const uint64_t r = sample_draw(a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(j),
+        const uint64_t r = sample_draw(rng_seed, a.rng_stream, node, static_cast<uint32_t>(j),
                                        static_cast<uint64_t>(deg));
         pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
@@ -331,7 +334,7 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
       for (int64_t step = 0; step < k; ++step) {
         const int64_t J = deg - k + step;
         const int64_t t = static_cast<int64_t>(sample_draw(
-            a.rng_seed, a.rng_stream, node, static_cast<uint32_t>(step), static_cast<uint64_t>(J + 1)));
+            rng_seed, a.rng_stream, node, static_cast<uint32_t>(step), static_cast<uint64_t>(J + 1)));
         bool taken = false;
         for (int64_t q = lane; q < step; q += kWave) {
           const int64_t c = IN_LDS ? chosen_lds[q] : load_int(a.out, optr + q, a.idx_bytes);
@@ -546,6 +549,7 @@ struct PickHopExtras {
   void *sub_indptr_rw;
   const uint64_t *tile_prefix;
   const int64_t *S_len;
+  const uint64_t *rng_seed_dev;
   void *copy_out;
   int copy_bytes;
   uint4 *clear;
@@ -613,6 +617,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.sub_indptr_rw = nullptr;
   a.tile_prefix = nullptr;
   a.S_len = nullptr;
+  a.rng_seed_dev = nullptr;
   a.copy_out = nullptr;
   a.copy_bytes = 8;
   a.clear = nullptr;
@@ -624,6 +629,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.sub_indptr_rw = hop->sub_indptr_rw;
   a.tile_prefix = hop->tile_prefix;
   a.S_len = hop->S_len;
+  a.rng_seed_dev = hop->rng_seed_dev;
   a.copy_out = hop->copy_out;
   a.copy_bytes = hop->copy_bytes;
   a.clear = hop->clear;
@@ -644,7 +650,8 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
 static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
                     const void *cache_indptr, const void *cache_indices, const shmt_hashmap_t *map,
                     const void *seeds, int seed_bytes, int64_t S, const int64_t *S_len, int64_t k,
-                    int replace, uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr,
+                    int replace, uint64_t rng_seed, const uint64_t *rng_seed_dev, uint32_t rng_stream,
+                    void *sub_indptr,
                     void *sub_indices, void *plan, int64_t plan_bytes, int elem_bytes, void *total_out,
                     void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
                     int64_t *nnz_out, int64_t *count_out, int64_t *count_copy, void *stream) {
@@ -664,7 +671,7 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
                  plan_bytes, nnz_out, stream, &plan_hop);
   if (rc) return rc;
-  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, S_len, total_out, elem_bytes,
+  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, S_len, rng_seed_dev, total_out, elem_bytes,
                                static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                  plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
@@ -684,7 +691,7 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
                     int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *nnz_out,
                     int64_t *count_out, void *stream) {
   return hop_impl(indptr, ptr_bytes, indices, idx_bytes, cache_indptr, cache_indices, map, seeds, seed_bytes,
-                  S, nullptr, k, replace, rng_seed, rng_stream, sub_indptr, sub_indices, plan, plan_bytes,
+                  S, nullptr, k, replace, rng_seed, nullptr, rng_stream, sub_indptr, sub_indices, plan, plan_bytes,
                   elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out, count_out,
                   nullptr, stream);
 }
@@ -693,12 +700,14 @@ int shmt_sample_hop_chained(const void *indptr, int ptr_bytes, const void *indic
                             const void *cache_indptr, const void *cache_indices,
                             const shmt_hashmap_t *map, const void *seeds, int seed_bytes,
                             int64_t max_seeds, const int64_t *seeds_len, int64_t k, int replace,
-                            uint64_t rng_seed, uint32_t rng_stream, void *sub_indptr, void *sub_indices,
+                            uint64_t rng_seed, const uint64_t *rng_seed_dev, uint32_t rng_stream,
+                            void *sub_indptr, void *sub_indices,
                             void *plan, int64_t plan_bytes, int elem_bytes, void *total_out,
                             void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
                             int64_t *nnz_out, int64_t *count_out, int64_t *count_dev_out, void *stream) {
   return hop_impl(indptr, ptr_bytes, indices, idx_bytes, cache_indptr, cache_indices, map, seeds, seed_bytes,
-                  max_seeds, seeds_len, k, replace, rng_seed, rng_stream, sub_indptr, sub_indices, plan,
+                  max_seeds, seeds_len, k, replace, rng_seed, rng_seed_dev, rng_stream, sub_indptr, sub_indices,
+                  plan,
                   plan_bytes, elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out,
                   count_out, count_dev_out, stream);
 }

@@ -419,7 +419,7 @@ def test_c_abi_chained_hops_need_no_host_wait(cabi, cached, S, picks, replace):
     chained, seeds, s_max, s_len = [], seeds0, S, None
     for hop, k in enumerate(picks):
         b = buffers(s_max, k)
-        cabi.check(lib.shmt_sample_hop_chained(*graph_args(), seeds.data_ptr(), 8, s_max, s_len, k, replace, 42, hop,
+        cabi.check(lib.shmt_sample_hop_chained(*graph_args(), seeds.data_ptr(), 8, s_max, s_len, k, replace, 42, None, hop,
                                                b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(),
                                                b["plan"].numel(), 8, b["total"].data_ptr(), b["scratch"].data_ptr(),
                                                b["scratch"].numel(), b["unique"].data_ptr(), b["labels"].data_ptr(),
@@ -449,3 +449,83 @@ def test_c_abi_chained_hops_need_no_host_wait(cabi, cached, S, picks, replace):
         seeds = b["unique"][:u].clone()
     if hnd is not None:
         lib.shmt_hashmap_destroy(hnd)
+
+
+def _chains_equal(got, want):
+    assert len(got) == len(want)
+    for a, b in zip(got, want):
+        assert len(a) == len(b)
+        for x, y in zip(a, b):
+            _same(x, y)
+
+
+@pytest.mark.parametrize("seeded", [True, False])
+@pytest.mark.parametrize("seed_dt", [torch.int64, torch.int32])
+def test_batch_sampler_replays_a_recorded_batch(capi, seeded, seed_dt):
+    """BatchSampler records the chained hops of one batch as a HIP graph and replays it per batch:
+    same results as sample_blocks, for full, ragged and empty batches, with results of earlier
+    calls still intact while later ones run, and lanes reused once results are dropped."""
+    import gc
+    indptr, indices = _graph(scale=14, idx_dt=torch.int32)
+    indptr_h, indices_h = indptr.cpu().pin_memory(), indices.cpu().pin_memory()
+    n = indptr.numel() - 1
+    hot = torch.randperm(n, generator=torch.Generator().manual_seed(1))[: n // 3].cuda()
+    gp, gi = capi.create_subcsr(indptr_h, indices_h, hot)
+    h = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel()).cuda(), 0.8)
+    picks = [4, 6, 3]
+    sampler = capi.BatchSampler(indptr_h, indices_h, gp, gi, h, 512, picks, False,
+                                seed_bytes=torch.empty(0, dtype=seed_dt).element_size())
+    g = torch.Generator().manual_seed(9)
+    sizes = [512, 100, 512, 1, 0, 511, 512, 37, 512]
+    batches = [torch.randperm(n, generator=g)[:s].to(seed_dt).cuda() for s in sizes]
+    rng = [300 + b for b in range(len(batches))] if seeded else None
+    want = capi.sample_blocks(indptr_h, indices_h, gp, gi, h, batches, picks, False, seeds_rng=rng)
+    kept = []
+    for repeat in range(3):
+        got = sampler.sample(batches, seeds_rng=rng, max_in_flight=3)
+        _chains_equal(got, want)
+        kept.append(got)                       # earlier results stay alive ...
+        for earlier in kept:
+            _chains_equal(earlier, want)       # ... and intact
+    lanes_held = sampler.lanes()
+    assert lanes_held >= 3 * (len(sizes) - 1)  # every non-empty batch still held owns a lane
+    del kept, got, earlier
+    gc.collect()
+    for repeat in range(3):                    # dropped results hand their lanes back: no new ones
+        _chains_equal(sampler.sample(batches, seeds_rng=rng, max_in_flight=2), want)
+        gc.collect()
+    assert sampler.lanes() == lanes_held
+    # the same through submit / collect, collected out of order
+    tickets = [sampler.submit(b, rng[i] if seeded else None) for i, b in enumerate(batches[:4])]
+    for i in (2, 0, 3, 1):
+        _chains_equal([sampler.collect(tickets[i])], [want[i]])
+    with pytest.raises(RuntimeError):
+        sampler.collect(tickets[0])            # a ticket is good for one collect
+    one = sampler.sample([batches[0]], seeds_rng=[300] if seeded else None)
+    del sampler                                # results outlive the sampler object
+    gc.collect()
+    _chains_equal(one, [want[0]])
+
+
+def test_batch_sampler_arguments(capi):
+    indptr = torch.tensor([0, 3, 3, 4]).cuda()
+    indices = torch.tensor([2, 1, 0, 2]).cuda()
+    sampler = capi.BatchSampler(indptr, indices, None, None, None, 2, [5, 2], True)
+    seeds = [torch.tensor([0, 2]).cuda(), torch.tensor([1]).cuda()]
+    _chains_equal(sampler.sample(seeds), capi.sample_blocks(indptr, indices, None, None, None, seeds, [5, 2], True))
+    assert sampler.sample([]) == []
+    with pytest.raises(RuntimeError):          # more seeds than the recorded batch holds
+        sampler.sample([torch.tensor([0, 1, 2]).cuda()])
+    with pytest.raises(RuntimeError):          # other id width than the sampler was built for
+        sampler.sample([torch.tensor([0], dtype=torch.int32).cuda()])
+    with pytest.raises(RuntimeError):
+        sampler.sample(seeds, seeds_rng=[1])
+    with pytest.raises(RuntimeError):          # a hop without picks cannot be recorded
+        capi.BatchSampler(indptr, indices, None, None, None, 2, [5, 0], False)
+    with pytest.raises(RuntimeError):          # bounds beyond what a recorded batch may allocate
+        capi.BatchSampler(indptr, indices, None, None, None, 4096, [25, 15, 10], False)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):              # called with a non-default current stream
+        got = sampler.sample(seeds, seeds_rng=[4, 5])
+    side.synchronize()
+    _chains_equal(got, capi.sample_blocks(indptr, indices, None, None, None, seeds, [5, 2], True, seeds_rng=[4, 5]))

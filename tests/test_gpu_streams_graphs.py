@@ -140,7 +140,7 @@ def test_a_whole_batch_of_chained_hops_replays_in_a_hip_graph(capi, cabi):
         for hop, b in enumerate(hops):
             cabi.check(lib.shmt_sample_hop_chained(
                 indptr.data_ptr(), 8, indices.data_ptr(), ib, None, None, None, src.data_ptr(), 8, b["s_max"], src_len,
-                b["k"], 0, 77, hop, b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(), b["plan"].numel(), 8,
+                b["k"], 0, 77, None, hop, b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(), b["plan"].numel(), 8,
                 b["total"].data_ptr(), b["scratch"].data_ptr(), b["scratch"].numel(), b["unique"].data_ptr(),
                 b["labels"].data_ptr(), b["nnz"].data_ptr(), b["count"].data_ptr(), b["count_dev"].data_ptr(),
                 cabi.current_stream()))
