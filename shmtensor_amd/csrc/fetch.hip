@@ -90,8 +90,7 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
     const int64_t counted = *a.count;
     if (counted < Q) Q = counted;
     if (a.count_seen && blockIdx.x == 0 && threadIdx.x == 0) {
-      *a.count_seen = counted;
-      __threadfence_system();
+      publish_size(a.count_seen, counted);
     }
   }
 

@@ -67,7 +67,7 @@ void *device_address(const torch::Tensor &t, const char *name) {
 // Totals whose value only the GPU knows (nnz of a sample, number of unique
 // ids) come back through int64 slots in pinned host memory. The host marks a
 // slot pending before the launches and the kernel overwrites it with the
-// total (always >= 0) followed by a system-scope fence; the host then watches
+// total (always >= 0) in one store that bypasses the caches; the host then watches
 // the slot instead of synchronising the stream, so it learns the total as
 // soon as the kernel that computes it has run, while later kernels of the
 // same operator are still queued or running. If the value does not show up

@@ -329,8 +329,7 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
   const int64_t last_tile = N > 0 ? (N - 1) / kRlTile : 0;
   if (static_cast<int64_t>(blockIdx.x) == last_tile && threadIdx.x == 0) {
     if (count_copy) *count_copy = static_cast<int64_t>(tile_prefix + tile_total);
-    *count_out = static_cast<int64_t>(tile_prefix + tile_total);
-    __threadfence_system();
+    publish_size(count_out, static_cast<int64_t>(tile_prefix + tile_total));
   }
 }
 
@@ -488,15 +487,13 @@ __global__ __launch_bounds__(kRlSmallBlock) void rl_small_kernel(const void *tot
   }
   if (t == 0) {
     if (count_copy) *count_copy = static_cast<int64_t>(below);
-    *count_out = static_cast<int64_t>(below);
-    __threadfence_system();
+    publish_size(count_out, static_cast<int64_t>(below));
   }
 }
 
 __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
   if (count_copy) *count_copy = 0;
-  *count_out = 0;
-  __threadfence_system();
+  publish_size(count_out, 0);
 }
 
 // A value no earlier call has used (and that uninitialised memory is unlikely to hold).

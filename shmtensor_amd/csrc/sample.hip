@@ -114,8 +114,7 @@ __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
   if (threadIdx.x == 0) {
     store_int(a.sub_indptr, S, a.ptr_bytes, static_cast<int64_t>(carry));
     if (a.total_word) *a.total_word = carry;
-    *a.nnz_out = static_cast<int64_t>(carry);
-    __threadfence_system();
+    publish_size(a.nnz_out, static_cast<int64_t>(carry));
   }
 }
 
@@ -150,8 +149,7 @@ __global__ __launch_bounds__(256) void add_tile_offsets_kernel(void *data, int e
     } else {
       const int64_t t = static_cast<int64_t>(partials[nb]);
       store_int(data, n, eb, t);
-      *total_out = t;
-      __threadfence_system();
+      publish_size(total_out, t);
     }
   }
 }
@@ -177,8 +175,7 @@ __global__ __launch_bounds__(1024) void plan_totals_kernel(uint64_t *partials, i
   if (threadIdx.x == 0) {
     partials[nb] = carry;
     store_int(sub_indptr, S, ptr_bytes, static_cast<int64_t>(carry));
-    *nnz_out = static_cast<int64_t>(carry);
-    __threadfence_system();
+    publish_size(nnz_out, static_cast<int64_t>(carry));
   }
 }
 
@@ -379,8 +376,7 @@ __global__ __launch_bounds__(256) void subcsr_degree_kernel(const void *indptr, 
 }
 
 __global__ void copy_total_kernel(const void *data, int eb, int64_t n, int64_t *total_out) {
-  *total_out = load_int(data, n, eb);
-  __threadfence_system();
+  publish_size(total_out, load_int(data, n, eb));
 }
 
 // Last row r in [lo, hi] with offsets[r] <= e.

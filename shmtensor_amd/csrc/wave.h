@@ -32,6 +32,16 @@ __device__ __host__ __forceinline__ uint32_t reduce_range(uint32_t h, uint32_t n
 // ---- width-switched integer access --------------------------------------
 // Ids, offsets and masks arrive as 4- or 8-byte signed integers; the width is
 // uniform across the launch, so the branch is scalar.
+// A result size the host is polling for (int64 in pinned host memory, or in
+// device memory that the host copies later): one store that bypasses the
+// caches, visible to the host as soon as it lands. Not a fence: nothing else
+// the kernel wrote is meant to be read by the host before it synchronises, and
+// a system-scope fence would write the whole L2 back to make this one word
+// visible.
+__device__ __forceinline__ void publish_size(int64_t *slot, int64_t value) {
+  __hip_atomic_store(slot, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 __device__ __forceinline__ int64_t load_int(const void *p, int64_t i, int bytes) {
   return bytes == 8 ? static_cast<const int64_t *>(p)[i]
                     : static_cast<int64_t>(static_cast<const int32_t *>(p)[i]);
