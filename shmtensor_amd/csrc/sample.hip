@@ -5,9 +5,12 @@
 // plan:  probe the cache map for 64 consecutive seeds per wave (8 cooperative
 //        probes at a time), read the two row offsets from the cached or the
 //        cold indptr, derive the output count and prefix-sum the counts in the
-//        same kernel. Up to kPlanSingleMax (1,024) seeds run in one workgroup (one
-//        launch); beyond that each 1024-seed tile scans locally and two short
-//        kernels add the tile offsets.
+//        same kernel. Tiles of kPlanBlock (256) seeds: cold row offsets are
+//        host-link reads and one compute unit keeps only so many in flight,
+//        so small tiles on many units beat one large workgroup. Up to one tile
+//        is one launch; beyond that each tile scans locally and the tile
+//        offsets are added by two short kernels (or, in the fused hop, by the
+//        pick kernel itself).
 // pick:  a sub-wave group of G >= k lanes owns a seed. Rows with deg <= k are
 //        copied in CSR order. Otherwise the k draws of Floyd's subset
 //        algorithm are generated in parallel (one Philox block per lane) and
@@ -18,8 +21,9 @@
 // hop:   shmt_sample_hop queues plan, pick and the relabel passes of
 //        {seeds, sampled ids} as one sequence. The HOP forms of the kernels
 //        do the relabel's preparation on the side: plan writes the seeds into
-//        the relabel input, pick adds the tile offsets itself (one short
-//        totals kernel instead of two passes over sub_indptr), writes every
+//        the relabel input, pick adds the tile offsets itself (every wave sums
+//        the tile totals below its tile; a totals kernel only beyond 1,024
+//        tiles) and publishes the total, writes every
 //        sampled id into the relabel input too, empties the relabel table and
 //        marks whether any id falls outside 32 bits. The number of seeds may
 //        itself live in device memory (the count a previous hop produced):
@@ -35,9 +39,10 @@
 
 namespace shmt {
 
-constexpr int kPlanBlock = 1024;
-constexpr int64_t kPlanSingleMax = 1024;
+constexpr int kPlanBlock = 256;
+constexpr int64_t kPlanSingleMax = 256;
 constexpr int64_t kCachedTag = 1ll << 62;  // plan.begin carries the source in bit 62
+constexpr int64_t kPickSumsTiles = 1024;  // up to this many plan tiles the fused hop needs no totals kernel
 constexpr int kWideMaxPicks = 8192;  // chosen set of 8 B entries must fit 64 KiB of LDS
 
 struct SeedPlan {
@@ -199,7 +204,10 @@ struct PickArgs {
   int log2_group;  // lanes per seed (narrow kernel)
   // fused hop only (HOP kernels):
   void *sub_indptr_rw;          // tile-local offsets in, final offsets out
-  const uint64_t *tile_prefix;  // scanned totals of the 1024-seed tiles, or null when offsets are final
+  const uint64_t *tile_prefix;  // totals of the plan's seed tiles, or null when offsets are final: scanned
+  int64_t raw_tiles;            // (raw_tiles == 0), or that many raw totals which this kernel sums itself,
+  int64_t *nnz_out;             // then also publishing the grand total (sub_indptr[S], total_word, *nnz_out)
+  uint64_t *total_word;
   const int64_t *S_len;         // optional: true number of seeds in device memory, S is then its bound
   const uint64_t *rng_seed_dev; // optional: the RNG seed lives in device memory (replayed launch sequences)
   void *copy_out;               // second copy of every sampled id, widened to copy_bytes, at
@@ -214,15 +222,41 @@ __device__ __forceinline__ void note_wide_id(const PickArgs &a, int64_t id) {
   if (static_cast<uint64_t>(id) >> 32) *a.wide_mark = a.wide_nonce;
 }
 
+// Sum of the first `count` raw tile totals, by a whole wave (all lanes active).
+__device__ __forceinline__ int64_t wave_sum_tiles(const uint64_t *totals, int64_t count) {
+  uint64_t acc = 0;
+  for (int64_t t = lane_id(); t < count; t += kWave) acc += totals[t];
+  return static_cast<int64_t>(wave_last(wave_inclusive_scan(acc)));
+}
+
+// Output offset that precedes the plan tile of seed s (fused hop; wave-uniform s / kPlanBlock,
+// all lanes active): the scanned tile total, or the sum of the raw totals below the tile.
+__device__ __forceinline__ int64_t pick_tile_base(const PickArgs &a, int64_t s) {
+  if (!a.tile_prefix) return 0;
+  const int64_t tile = s / kPlanBlock;
+  return a.raw_tiles ? wave_sum_tiles(a.tile_prefix, tile) : static_cast<int64_t>(a.tile_prefix[tile]);
+}
+
+// With raw tile totals nobody has published the grand total yet: the first wave of the grid does.
+__device__ __forceinline__ void pick_publish_total(const PickArgs &a, int64_t S) {
+  if (!a.raw_tiles || blockIdx.x != 0 || threadIdx.x >= kWave) return;
+  const int64_t total = wave_sum_tiles(a.tile_prefix, a.raw_tiles);
+  if (threadIdx.x == 0) {
+    store_int(a.sub_indptr_rw, S, a.ptr_bytes, total);
+    *a.total_word = static_cast<uint64_t>(total);
+    publish_size(a.nnz_out, total);
+  }
+}
+
 // Output offset of seed s. In the fused hop the plan left tile-local offsets:
-// the tile's prefix is added here and the final value written back by `writer`.
+// the tile's base is added here and the final value written back by `writer`.
 template <bool HOP>
-__device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, bool writer) {
+__device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, int64_t tile_base, bool writer) {
   if (!HOP) return load_int(a.sub_indptr, s, a.ptr_bytes);
   int64_t optr = load_int(a.sub_indptr_rw, s, a.ptr_bytes);
   if (writer) note_wide_id(a, load_int(a.seeds, s, a.seed_bytes));
   if (a.tile_prefix) {
-    optr += static_cast<int64_t>(a.tile_prefix[s / kPlanBlock]);
+    optr += tile_base;
     if (writer) store_int(a.sub_indptr_rw, s, a.ptr_bytes, optr);
   }
   return optr;
@@ -266,13 +300,16 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
   const int k = static_cast<int>(a.k);
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
   const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
+  if (HOP) pick_publish_total(a, S);
 
   for (int64_t s0 = wave * groups_per_wave; s0 < S; s0 += nwaves * groups_per_wave) {
+    // the seeds of a wave share a plan tile (tiles hold a multiple of groups_per_wave seeds)
+    const int64_t tile_base = HOP ? pick_tile_base(a, s0) : 0;
     const int64_t s = s0 + (lane >> a.log2_group);
     if (s >= S) continue;  // uniform within the group
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
-    const int64_t optr = pick_offset<HOP>(a, s, gl == 0);
+    const int64_t optr = pick_offset<HOP>(a, s, tile_base, gl == 0);
     if (deg <= 0) continue;
     if (a.replace) {
       if (gl < k) {
@@ -313,10 +350,11 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
   const int64_t k = a.k;
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
   const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
+  if (HOP) pick_publish_total(a, S);
   for (int64_t s = blockIdx.x; s < S; s += gridDim.x) {
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
-    const int64_t optr = pick_offset<HOP>(a, s, lane == 0);
+    const int64_t optr = pick_offset<HOP>(a, s, HOP ? pick_tile_base(a, s) : 0, lane == 0);
     if (deg <= 0) continue;
     const int64_t node = load_int(a.seeds, s, a.seed_bytes);
     if (a.replace) {
@@ -447,6 +485,7 @@ struct PlanHopExtras {
   const int64_t *S_len;             // true number of seeds in device memory, or null
   const uint64_t *tile_prefix_out;
   const uint64_t *total_out;        // where the kernels leave the total (nnz) in device memory
+  int64_t raw_tiles_out;            // > 0: tile_prefix_out holds that many raw totals, the pick kernel sums them
 };
 
 static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr,
@@ -494,6 +533,7 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   if (hop) {
     hop->tile_prefix_out = nullptr;
     hop->total_out = a.total_word;
+    hop->raw_tiles_out = 0;
   }
   const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
 
@@ -516,10 +556,14 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   }
   SHMT_LAUNCH_CHECK();
   if (hop) {
+    hop->tile_prefix_out = a.partials;
+    if (nb <= kPickSumsTiles) {  // few tiles: every wave of the pick kernel sums the totals below its tile
+      hop->raw_tiles_out = nb;
+      return SHMT_OK;
+    }
     hipLaunchKernelGGL(plan_totals_kernel, dim3(1), dim3(1024), 0, s, a.partials, nb, sub_indptr,
                        ptr_bytes, S, a.S_len, nnz_out);
     SHMT_LAUNCH_CHECK();
-    hop->tile_prefix_out = a.partials;
     return SHMT_OK;
   }
   int rc = launch_scan_partials(a.partials, nb + 1, s);
@@ -544,6 +588,9 @@ int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr
 struct PickHopExtras {
   void *sub_indptr_rw;
   const uint64_t *tile_prefix;
+  int64_t raw_tiles;
+  int64_t *nnz_out;
+  uint64_t *total_word;
   const int64_t *S_len;
   const uint64_t *rng_seed_dev;
   void *copy_out;
@@ -612,6 +659,9 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   }
   a.sub_indptr_rw = nullptr;
   a.tile_prefix = nullptr;
+  a.raw_tiles = 0;
+  a.nnz_out = nullptr;
+  a.total_word = nullptr;
   a.S_len = nullptr;
   a.rng_seed_dev = nullptr;
   a.copy_out = nullptr;
@@ -624,6 +674,9 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   if (!hop) return pick_launch<false>(a, s);
   a.sub_indptr_rw = hop->sub_indptr_rw;
   a.tile_prefix = hop->tile_prefix;
+  a.raw_tiles = hop->raw_tiles;
+  a.nnz_out = hop->nnz_out;
+  a.total_word = hop->total_word;
   a.S_len = hop->S_len;
   a.rng_seed_dev = hop->rng_seed_dev;
   a.copy_out = hop->copy_out;
@@ -663,11 +716,12 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
   RelabelTable table;
   int rc = relabel_table(n_max, scratch, scratch_bytes, &table);
   if (rc) return rc;
-  PlanHopExtras plan_hop{total_out, elem_bytes, S_len, nullptr, nullptr};
+  PlanHopExtras plan_hop{total_out, elem_bytes, S_len, nullptr, nullptr, 0};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
                  plan_bytes, nnz_out, stream, &plan_hop);
   if (rc) return rc;
-  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, S_len, rng_seed_dev, total_out, elem_bytes,
+  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, plan_hop.raw_tiles_out, nnz_out,
+                               const_cast<uint64_t *>(plan_hop.total_out), S_len, rng_seed_dev, total_out, elem_bytes,
                                static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                  plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
