@@ -605,14 +605,21 @@ template <bool HOP>
 static int pick_launch(const PickArgs &a, hipStream_t s) {
   const int64_t S = a.S, k = a.k;
   if (k <= kWave) {
-    const int seeds_per_block = 4 * (kWave >> a.log2_group);
+    // Few seeds: one wave per workgroup, so that the cold rows' host-link reads come from as many
+    // compute units as possible (a unit keeps only so many of them in flight).
+    const int seeds_per_wave = kWave >> a.log2_group;
+    int threads = 256;
+    int64_t blocks = (S + 4 * seeds_per_wave - 1) / (4 * seeds_per_wave);
+    if (blocks < 512) {
+      threads = kWave;
+      blocks = (S + seeds_per_wave - 1) / seeds_per_wave;
+    }
     // the fused form also clears the relabel table: enough threads for that even when S is small
-    int64_t blocks = (S + seeds_per_block - 1) / seeds_per_block;
     if (HOP) {
-      const int64_t for_clear = (a.clear_n + 256 * 4 - 1) / (256 * 4);
+      const int64_t for_clear = (a.clear_n + threads * 4 - 1) / (threads * 4);
       if (blocks < for_clear) blocks = for_clear;
     }
-    hipLaunchKernelGGL(pick_narrow_kernel<HOP>, dim3(grid_for(blocks, 1)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(pick_narrow_kernel<HOP>, dim3(grid_for(blocks, 1)), dim3(threads), 0, s, a);
   } else if (k <= kWideMaxPicks) {
     hipLaunchKernelGGL((pick_wide_kernel<true, HOP>), dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
                        static_cast<size_t>(k) * sizeof(int64_t), s, a);
