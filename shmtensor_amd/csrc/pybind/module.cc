@@ -982,6 +982,13 @@ class SamplerState : public std::enable_shared_from_this<SamplerState> {
     }
   }
 
+  // A lane that was acquired but whose batch could not be queued.
+  void give_back(Lane *lane) {
+    lane->release_unordered = true;  // whatever did get queued is waited for before the next use
+    std::lock_guard<std::mutex> lock(mutex_);
+    free_.push_back(lane);
+  }
+
   // Stage the batch and replay the lane's graph on the lane's stream.
   void launch(Lane *lane, const torch::Tensor &seeds, uint64_t rng_seed,
               c10::hip::HIPStreamMasqueradingAsCUDA caller) {
@@ -1187,7 +1194,12 @@ class BatchSampler {
       p.ready = run_hops(st.graph(), seeds, st.picks(), st.replace(), seed_rng, nullptr).hops;
     } else {
       p.lane = st.acquire(seed_rng.has_value());
-      st.launch(p.lane, seeds, seed_rng ? static_cast<uint64_t>(*seed_rng) : kDefaultSeed, *p.caller);
+      try {
+        st.launch(p.lane, seeds, seed_rng ? static_cast<uint64_t>(*seed_rng) : kDefaultSeed, *p.caller);
+      } catch (...) {
+        st.give_back(p.lane);
+        throw;
+      }
     }
     std::lock_guard<std::mutex> lock(mutex_);
     const int64_t ticket = next_ticket_++;
