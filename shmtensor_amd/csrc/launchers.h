@@ -27,11 +27,11 @@ struct RelabelTable {
   uint64_t *wide_mark;  // where the earlier kernels store `nonce` when an id lies outside [0, 2^32)
   uint64_t nonce;
 };
-int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable *out);
+int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scratch_bytes, RelabelTable *out);
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const int64_t *n_fixed_dev,
                           const void *n_extra_dev, int n_extra_bytes, int elem_bytes, void *scratch,
                           int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
-                          int64_t *count_copy, uint64_t nonce, hipStream_t stream);
+                          int64_t *count_copy, const RelabelTable &table, hipStream_t stream);
 uint64_t relabel_nonce();
 
 }  // namespace shmt

@@ -522,7 +522,8 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
 static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
                         int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
                         void *labels_out, int64_t *count_out, void *stream, bool prepared = false,
-                        uint64_t prepared_nonce = 0, int64_t *count_copy = nullptr) {
+                        uint64_t prepared_nonce = 0, int64_t *count_copy = nullptr,
+                        int64_t prepared_slots = 0) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
@@ -547,7 +548,8 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   uint32_t *rank_of = reinterpret_cast<uint32_t *>(base + l.rank_off);
   uint64_t *partials = reinterpret_cast<uint64_t *>(base + l.partial_off);
   const int64_t nb = (N + kRlTile - 1) / kRlTile;
-  const uint32_t cap = static_cast<uint32_t>(l.cap);
+  // a caller that emptied the table itself says how much of it (relabel_table)
+  const uint32_t cap = static_cast<uint32_t>(prepared && prepared_slots > 0 ? prepared_slots : l.cap);
   // 4-byte ids always fit the packed table; 8-byte ids use it when an earlier kernel vouches for them
   // (plain shmt_relabel has no kernel that sees the ids before the insert pass: 16-byte slots)
   uint64_t *wide_mark = reinterpret_cast<uint64_t *>(base + l.flag_off);
@@ -604,7 +606,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
 
 namespace shmt {
 
-int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable *out) {
+int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scratch_bytes, RelabelTable *out) {
   SHMT_REQUIRE(N >= 1 && N < (1ll << 31), "relabel: N must be in [1, 2^31)");
   const RlLayout l = rl_layout(N);
   if (scratch == nullptr || scratch_bytes < l.total) {
@@ -614,7 +616,11 @@ int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable 
   }
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "relabel: scratch must be 16-byte aligned");
   out->slots = static_cast<char *>(scratch) + l.table_off;
-  out->n16 = N <= kRlSmallMax ? 0 : l.cap;  // small inputs are relabelled in LDS: nothing to empty
+  // Small inputs are relabelled in LDS: nothing to empty. When N is a loose bound of the id count (a
+  // chained hop sized for every seed the hop before could have produced, typically three times what
+  // it did produce) half the slots are used: still one 16-byte slot per id in the worst case, and
+  // half as much to empty.
+  out->n16 = N <= kRlSmallMax ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
   out->wide_mark = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + l.flag_off);
   out->nonce = relabel_nonce();
   return SHMT_OK;
@@ -623,11 +629,11 @@ int relabel_table(int64_t N, void *scratch, int64_t scratch_bytes, RelabelTable 
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const int64_t *n_fixed_dev,
                           const void *n_extra_dev, int n_extra_bytes, int elem_bytes, void *scratch,
                           int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
-                          int64_t *count_copy, uint64_t nonce, hipStream_t stream) {
+                          int64_t *count_copy, const RelabelTable &table, hipStream_t stream) {
   return relabel_impl(total, nullptr, n_bound,
                       RlCount{n_fixed, n_fixed_dev, n_extra_dev, n_extra_bytes, n_bound}, elem_bytes,
-                      scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true, nonce,
-                      count_copy);
+                      scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true, table.nonce,
+                      count_copy, table.n16);
 }
 
 }  // namespace shmt

@@ -721,7 +721,7 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
                "shmt_sample_hop: null buffer");
   const int64_t n_max = S + S * k;
   RelabelTable table;
-  int rc = relabel_table(n_max, scratch, scratch_bytes, &table);
+  int rc = relabel_table(n_max, S_len != nullptr, scratch, scratch_bytes, &table);
   if (rc) return rc;
   PlanHopExtras plan_hop{total_out, elem_bytes, S_len, nullptr, nullptr, 0};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
@@ -736,7 +736,7 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
   // [seeds, sub_indices] is in total_out and the table is empty: the relabel passes follow, with the
   // number of sampled ids (and of seeds, when it is a device-side figure) read from device memory
   return launch_relabel_passes(total_out, n_max, S, S_len, plan_hop.total_out, 8, elem_bytes, scratch,
-                               scratch_bytes, unique_out, labels_out, count_out, count_copy, table.nonce,
+                               scratch_bytes, unique_out, labels_out, count_out, count_copy, table,
                                as_stream(stream));
 }
 
