@@ -231,6 +231,22 @@ int shmt_sample_pick(const void *indices, const void *cache_indices,
                      int ptr_bytes, const void *plan, void *sub_indices,
                      uint64_t rng_seed, uint32_t rng_stream, void *stream);
 
+/* Both steps for callers that can give sub_indices room for the bound S * k
+ * (the first *nnz_out entries are the result): plan and pick are then two
+ * launches whatever the number of seeds, queued back to back, because the
+ * pick kernel adds the tile offsets of the plan itself and publishes the
+ * total; nothing needs *nnz_out before the pick is queued. Same results as
+ * shmt_sample_plan + shmt_sample_pick (CSRWiseSampling / CSRWiseCacheSampling,
+ * src/cache_graph_sampling.cu:179-220, :382-426, which read nnz on the host
+ * between the two steps, :195, :403). Requires S >= 1, k >= 1.             */
+int shmt_sample(const void *indptr, int ptr_bytes, const void *indices,
+                int idx_bytes, const void *cache_indptr,
+                const void *cache_indices, const shmt_hashmap_t *map,
+                const void *seeds, int seed_bytes, int64_t S, int64_t k,
+                int replace, uint64_t rng_seed, uint32_t rng_stream,
+                void *sub_indptr, void *sub_indices, void *plan,
+                int64_t plan_bytes, int64_t *nnz_out, void *stream);
+
 /* One hop of mini-batch sampling as one launch sequence: the body of the
  * dataloader's loop, python/shmtensor/sampling.py:128-143, i.e.
  * CSRWise[Cache]Sampling (src/cache_graph_sampling.cu:179-220, :382-426)

@@ -41,6 +41,8 @@ SIGNATURES = {
     "shmt_sample_plan": (_int, [_vp, _int, _vp, _vp, _vp, _int, _i64, _i64, _int, _vp, _vp, _i64, _vp, _vp]),
     "shmt_sample_pick": (_int, [_vp, _vp, _int, _vp, _int, _i64, _i64, _int, _vp, _int, _vp, _vp,
                                 _c.c_uint64, _c.c_uint32, _vp]),
+    "shmt_sample": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int, _i64, _i64, _int, _c.c_uint64,
+                           _c.c_uint32, _vp, _vp, _vp, _i64, _vp, _vp]),
     "shmt_sample_hop": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int, _i64, _i64, _int, _c.c_uint64,
                                _c.c_uint32, _vp, _vp, _vp, _i64, _int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "shmt_sample_hop_chained": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int, _i64, _vp, _i64, _int,

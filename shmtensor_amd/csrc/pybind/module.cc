@@ -372,32 +372,32 @@ std::tuple<torch::Tensor, torch::Tensor> sample_impl(const torch::Tensor &indptr
   torch::Tensor plan = device_bytes(plan_bytes);
   const Readback::Slot total = readback().acquire();
   void *stream = current_stream();
-  check(shmt_sample_plan(device_address(indptr, "indptr"), pb,
-                         map ? gpu_indptr->data_ptr() : nullptr, map ? map->handle() : nullptr,
-                         seeds.data_ptr(), static_cast<int>(seeds.element_size()), S, num_picks,
-                         replace, sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, total.dev,
-                         stream));
+  void *const indptr_dev = device_address(indptr, "indptr");
+  void *const indices_dev = device_address(indices, "indices");
+  const int sb = static_cast<int>(seeds.element_size());
+  const uint64_t rng_seed = static_cast<uint64_t>(seed.value_or(kDefaultSeed));
   // Output size is data dependent. When the bound S*k is modest, sample into a
-  // buffer of that size and pick up the total afterwards (both kernels are
-  // queued back to back); otherwise wait for the total first and allocate exactly.
+  // buffer of that size and pick up the total afterwards (plan and pick are
+  // queued back to back, two launches); otherwise plan, wait for the total,
+  // allocate exactly, pick.
   const bool eager = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
-  int64_t nnz = -1;
   torch::Tensor sub_indices;
   if (eager) {
     sub_indices = torch::empty({S * num_picks}, indices.options().device(dev));
+    check(shmt_sample(indptr_dev, pb, indices_dev, ib, map ? gpu_indptr->data_ptr() : nullptr,
+                      map ? gpu_indices->data_ptr() : nullptr, map ? map->handle() : nullptr, seeds.data_ptr(),
+                      sb, S, num_picks, replace, rng_seed, static_cast<uint32_t>(stream_id),
+                      sub_indptr.data_ptr(), sub_indices.data_ptr(), plan.data_ptr(), plan_bytes, total.dev,
+                      stream));
+    sub_indices = sub_indices.narrow(0, 0, Readback::wait(total));
   } else {
-    nnz = Readback::wait(total);
-    sub_indices = torch::empty({nnz}, indices.options().device(dev));
-  }
-  check(shmt_sample_pick(device_address(indices, "indices"),
-                         map ? gpu_indices->data_ptr() : nullptr, ib, seeds.data_ptr(),
-                         static_cast<int>(seeds.element_size()), S, num_picks, replace,
-                         sub_indptr.data_ptr(), pb, plan.data_ptr(), sub_indices.data_ptr(),
-                         static_cast<uint64_t>(seed.value_or(kDefaultSeed)),
-                         static_cast<uint32_t>(stream_id), stream));
-  if (eager) {
-    nnz = Readback::wait(total);
-    sub_indices = sub_indices.narrow(0, 0, nnz);
+    check(shmt_sample_plan(indptr_dev, pb, map ? gpu_indptr->data_ptr() : nullptr,
+                           map ? map->handle() : nullptr, seeds.data_ptr(), sb, S, num_picks, replace,
+                           sub_indptr.data_ptr(), plan.data_ptr(), plan_bytes, total.dev, stream));
+    sub_indices = torch::empty({Readback::wait(total)}, indices.options().device(dev));
+    check(shmt_sample_pick(indices_dev, map ? gpu_indices->data_ptr() : nullptr, ib, seeds.data_ptr(), sb, S,
+                           num_picks, replace, sub_indptr.data_ptr(), pb, plan.data_ptr(),
+                           sub_indices.data_ptr(), rng_seed, static_cast<uint32_t>(stream_id), stream));
   }
   return std::make_tuple(sub_indptr, sub_indices);
 }

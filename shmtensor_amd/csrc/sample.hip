@@ -219,7 +219,7 @@ struct PickArgs {
 };
 
 __device__ __forceinline__ void note_wide_id(const PickArgs &a, int64_t id) {
-  if (static_cast<uint64_t>(id) >> 32) *a.wide_mark = a.wide_nonce;
+  if (a.wide_mark && (static_cast<uint64_t>(id) >> 32)) *a.wide_mark = a.wide_nonce;
 }
 
 // Sum of the first `count` raw tile totals, by a whole wave (all lanes active).
@@ -254,7 +254,7 @@ template <bool HOP>
 __device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, int64_t tile_base, bool writer) {
   if (!HOP) return load_int(a.sub_indptr, s, a.ptr_bytes);
   int64_t optr = load_int(a.sub_indptr_rw, s, a.ptr_bytes);
-  if (writer) note_wide_id(a, load_int(a.seeds, s, a.seed_bytes));
+  if (writer && a.wide_mark) note_wide_id(a, load_int(a.seeds, s, a.seed_bytes));
   if (a.tile_prefix) {
     optr += tile_base;
     if (writer) store_int(a.sub_indptr_rw, s, a.ptr_bytes, optr);
@@ -265,7 +265,7 @@ __device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, int
 template <bool HOP>
 __device__ __forceinline__ void pick_store(const PickArgs &a, int64_t S, int64_t pos, int64_t v) {
   store_int(a.out, pos, a.idx_bytes, v);
-  if (HOP) {
+  if (HOP && a.copy_out) {
     store_int(a.copy_out, S + pos, a.copy_bytes, v);
     note_wide_id(a, v);
   }
@@ -701,6 +701,25 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
                      uint64_t rng_seed, uint32_t rng_stream, void *stream) {
   return pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr,
                    ptr_bytes, plan, sub_indices, rng_seed, rng_stream, stream, nullptr);
+}
+
+int shmt_sample(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
+                const void *cache_indptr, const void *cache_indices, const shmt_hashmap_t *map,
+                const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace, uint64_t rng_seed,
+                uint32_t rng_stream, void *sub_indptr, void *sub_indices, void *plan, int64_t plan_bytes,
+                int64_t *nnz_out, void *stream) {
+  SHMT_REQUIRE(S >= 1 && k >= 1, "shmt_sample: S and num_picks must be >= 1");
+  // the fused-hop forms of the kernels without their relabel extras: the pick kernel adds the tile
+  // offsets and publishes the total, so plan + pick are two launches whatever the number of seeds
+  PlanHopExtras plan_hop{nullptr, 8, nullptr, nullptr, nullptr, 0};
+  int rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
+                     plan_bytes, nnz_out, stream, &plan_hop);
+  if (rc) return rc;
+  const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, plan_hop.raw_tiles_out, nnz_out,
+                               const_cast<uint64_t *>(plan_hop.total_out), nullptr, nullptr, nullptr, 8,
+                               nullptr, 0, nullptr, 0};
+  return pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
+                   plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
 }
 
 static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,

@@ -529,3 +529,35 @@ def test_batch_sampler_arguments(capi):
         got = sampler.sample(seeds, seeds_rng=[4, 5])
     side.synchronize()
     _chains_equal(got, capi.sample_blocks(indptr, indices, None, None, None, seeds, [5, 2], True, seeds_rng=[4, 5]))
+
+
+@pytest.mark.parametrize("S,k,replace", [(1, 3, 0), (256, 5, 0), (257, 5, 1), (3000, 20, 0), (50, 70, 0),
+                                         (300000, 2, 0)])
+def test_c_abi_sample_in_two_launches_matches_plan_then_pick(cabi, S, k, replace):
+    """shmt_sample (bound-sized output, the pick kernel adds the tile offsets) against
+    shmt_sample_plan + shmt_sample_pick with the total read by the host in between."""
+    lib = cabi.load()
+    indptr, indices = _graph(scale=13, ptr_dt=torch.int64, idx_dt=torch.int32)
+    indptr, indices = indptr.cuda(), indices.cuda()
+    n = indptr.numel() - 1
+    stream = cabi.current_stream()
+    seeds = torch.randint(0, n, (S,), generator=torch.Generator().manual_seed(S)).cuda()
+
+    def buffers():
+        return dict(sp=torch.full((S + 1,), -1, dtype=torch.int64).cuda(), si=torch.empty(S * k, dtype=torch.int32).cuda(),
+                    plan=torch.empty(lib.shmt_sample_plan_bytes(S), dtype=torch.uint8).cuda(),
+                    nnz=torch.full((1,), -1, dtype=torch.int64).cuda())
+    a, b = buffers(), buffers()
+    cabi.check(lib.shmt_sample(indptr.data_ptr(), 8, indices.data_ptr(), 4, None, None, None, seeds.data_ptr(), 8, S, k,
+                               replace, 11, 3, a["sp"].data_ptr(), a["si"].data_ptr(), a["plan"].data_ptr(),
+                               a["plan"].numel(), a["nnz"].data_ptr(), stream))
+    cabi.check(lib.shmt_sample_plan(indptr.data_ptr(), 8, None, None, seeds.data_ptr(), 8, S, k, replace,
+                                    b["sp"].data_ptr(), b["plan"].data_ptr(), b["plan"].numel(), b["nnz"].data_ptr(), stream))
+    cabi.check(lib.shmt_sample_pick(indices.data_ptr(), None, 4, seeds.data_ptr(), 8, S, k, replace, b["sp"].data_ptr(), 8,
+                                    b["plan"].data_ptr(), b["si"].data_ptr(), 11, 3, stream))
+    torch.cuda.synchronize()
+    nnz = int(b["nnz"].item())
+    assert int(a["nnz"].item()) == nnz
+    assert torch.equal(a["sp"], b["sp"]) and torch.equal(a["si"][:nnz], b["si"][:nnz])
+    assert lib.shmt_sample(indptr.data_ptr(), 8, indices.data_ptr(), 4, None, None, None, seeds.data_ptr(), 8, 0, k,
+                           replace, 11, 3, None, None, None, 0, None, stream) == -1
