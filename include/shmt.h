@@ -259,7 +259,7 @@ int shmt_sample(const void *indptr, int ptr_bytes, const void *indices,
  * writes the seeds to total_out[0..S), the pick kernel also writes every
  * sampled id to total_out[S + offset], adds the tile offsets and empties the
  * relabel table, and the relabel passes read the sampled count from
- * sub_indptr[S] on the device.
+ * device memory (a word of the plan buffer).
  * Requires S >= 1, k >= 1 and S * (k + 1) < 2^31. Buffers: sub_indptr S + 1
  * entries (ptr_bytes); sub_indices S * k entries (idx_bytes; the first nnz are
  * the result); plan >= shmt_sample_plan_bytes(S); total_out, unique_out,
