@@ -312,6 +312,48 @@ int shmt_sample_hop_chained(const void *indptr, int ptr_bytes,
                             int64_t *count_out, int64_t *count_dev_out,
                             void *stream);
 
+/* Several independent chained hops at once (the same hop of several
+ * mini-batches): every job is one shmt_sample_hop_chained call, the fields
+ * are its parameters. Jobs that run the same kernels (same cache mode,
+ * fan-out class and size class) share their launches: one launch per kernel
+ * for up to 8 jobs, the job being a grid dimension, instead of one per job;
+ * other jobs are issued one after the other. Results are those of the
+ * individual calls. With several mini-batches in flight the host's launch
+ * rate, not the GPU, bounds the sampler; the reference issues every kernel of
+ * every hop of every batch separately (python/shmtensor/sampling.py:128-143). */
+typedef struct shmt_hop_job {
+  const void *indptr;
+  int ptr_bytes;
+  const void *indices;
+  int idx_bytes;
+  const void *cache_indptr;
+  const void *cache_indices;
+  const shmt_hashmap_t *map;
+  const void *seeds;
+  int seed_bytes;
+  int64_t max_seeds;
+  const int64_t *seeds_len;
+  int64_t k;
+  int replace;
+  uint64_t rng_seed;
+  const uint64_t *rng_seed_dev;
+  uint32_t rng_stream;
+  void *sub_indptr;
+  void *sub_indices;
+  void *plan;
+  int64_t plan_bytes;
+  int elem_bytes;
+  void *total_out;
+  void *scratch;
+  int64_t scratch_bytes;
+  void *unique_out;
+  void *labels_out;
+  int64_t *nnz_out;
+  int64_t *count_out;
+  int64_t *count_dev_out;
+} shmt_hop_job;
+int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream);
+
 /* Replaying a mini-batch. The hops of a batch, queued with
  * shmt_sample_hop_chained on fixed buffers, never wait for the host, so the
  * whole sequence can be captured once as a HIP graph and replayed for every

@@ -48,6 +48,7 @@ SIGNATURES = {
     "shmt_sample_hop_chained": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _vp, _int, _i64, _vp, _i64, _int,
                                        _c.c_uint64, _vp, _c.c_uint32, _vp, _vp, _vp, _i64, _int, _vp, _vp, _i64,
                                        _vp, _vp, _vp, _vp, _vp, _vp]),
+    "shmt_sample_hops_chained": (_int, [_vp, _int, _vp]),
     "shmt_capture_begin": (_int, [_vp]),
     "shmt_capture_end": (_int, [_vp, _c.POINTER(_vp)]),
     "shmt_graph_launch": (_int, [_vp, _vp]),
@@ -56,6 +57,18 @@ SIGNATURES = {
     "shmt_subcsr_plan": (_int, [_vp, _int, _vp, _int, _i64, _vp, _vp, _i64, _vp, _vp]),
     "shmt_subcsr_copy": (_int, [_vp, _vp, _int, _int, _vp, _int, _i64, _vp, _i64, _vp, _vp]),
 }
+
+class HopJob(_c.Structure):
+    """shmt_hop_job of include/shmt.h: the parameters of one shmt_sample_hop_chained call."""
+    _fields_ = [("indptr", _vp), ("ptr_bytes", _int), ("indices", _vp), ("idx_bytes", _int),
+                ("cache_indptr", _vp), ("cache_indices", _vp), ("map", _vp), ("seeds", _vp),
+                ("seed_bytes", _int), ("max_seeds", _i64), ("seeds_len", _vp), ("k", _i64), ("replace", _int),
+                ("rng_seed", _c.c_uint64), ("rng_seed_dev", _vp), ("rng_stream", _c.c_uint32),
+                ("sub_indptr", _vp), ("sub_indices", _vp), ("plan", _vp), ("plan_bytes", _i64),
+                ("elem_bytes", _int), ("total_out", _vp), ("scratch", _vp), ("scratch_bytes", _i64),
+                ("unique_out", _vp), ("labels_out", _vp), ("nnz_out", _vp), ("count_out", _vp),
+                ("count_dev_out", _vp)]
+
 
 _lib = None
 

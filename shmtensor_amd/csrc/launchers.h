@@ -3,7 +3,86 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <string.h>
+
 namespace shmt {
+
+// ---- merged launches ----------------------------------------------------------
+// Several independent jobs that run the same kernel sequence (the hops of
+// several mini-batches) can share their launches: instead of being issued, a
+// job's launches are recorded as stages, and stage i of all jobs then goes out
+// as ONE launch whose blockIdx.y selects the job. The kernels are the same
+// device code either way; a sequence that contains a launch without a merged
+// form is marked so and the caller issues the jobs one by one instead.
+constexpr int kMaxJobs = 8;
+constexpr int kStageArgBytes = 256;
+constexpr int kMaxStages = 12;
+
+enum StageKind : int {
+  kStagePlanSingle = 0,  // + map mode (0: no cache, 1: wide map, 2: narrow map)
+  kStagePlanTile = 3,    // + map mode
+  kStagePickNarrowHop = 6,
+  kStageRlSmall = 7,
+  kStageRlInsert = 8,
+  kStageRlFirst = 9,
+  kStageRlUnique = 10,
+  kStageRlLabels = 11,
+};
+
+struct Stage {
+  int kind;
+  unsigned blocks, threads;
+  alignas(16) unsigned char args[kStageArgBytes];
+};
+
+struct StageList {
+  int n = 0;
+  bool mergeable = true;
+  Stage stage[kMaxStages];
+};
+
+// Where a launch goes: to the stream at once, or (defer != nullptr) into a stage list.
+struct Launcher {
+  hipStream_t stream;
+  StageList *defer;
+};
+
+template <typename Args>
+inline void stage_push(StageList *list, int kind, unsigned blocks, unsigned threads, const Args &a) {
+  static_assert(sizeof(Args) <= kStageArgBytes, "kernel arguments do not fit a stage record");
+  if (list->n >= kMaxStages) {
+    list->mergeable = false;
+    return;
+  }
+  Stage &s = list->stage[list->n++];
+  s.kind = kind;
+  s.blocks = blocks;
+  s.threads = threads;
+  memcpy(s.args, &a, sizeof(Args));
+}
+
+// Arguments of `n_jobs` recorded launches of one kernel, as the merged kernel takes them.
+template <typename Args>
+struct Jobs {
+  Args a[kMaxJobs];
+  unsigned blocks[kMaxJobs];
+};
+
+template <typename Args>
+inline unsigned jobs_from_stages(int n_jobs, const Stage *const *stages, Jobs<Args> *out) {
+  unsigned max_blocks = 1;
+  for (int j = 0; j < kMaxJobs; ++j) {
+    const Stage *s = stages[j < n_jobs ? j : 0];
+    memcpy(&out->a[j], s->args, sizeof(Args));
+    out->blocks[j] = j < n_jobs ? s->blocks : 0;
+    if (j < n_jobs && s->blocks > max_blocks) max_blocks = s->blocks;
+  }
+  return max_blocks;
+}
+
+// One merged launch for stage `stages[j]` of jobs j < n_jobs (all of the same kind and block size).
+int launch_merged_sampling_stage(int n_jobs, const Stage *const *stages, hipStream_t s);  // sample.hip
+int launch_merged_relabel_stage(int n_jobs, const Stage *const *stages, hipStream_t s);   // relabel.hip
 
 // Set n16 consecutive 16-byte words at p (16-byte aligned) to all-ones, i.e.
 // every integer field to -1 / its unsigned maximum.
@@ -31,7 +110,7 @@ int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scrat
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const int64_t *n_fixed_dev,
                           const void *n_extra_dev, int n_extra_bytes, int elem_bytes, void *scratch,
                           int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
-                          int64_t *count_copy, const RelabelTable &table, hipStream_t stream);
+                          int64_t *count_copy, const RelabelTable &table, Launcher launcher);
 uint64_t relabel_nonce();
 
 }  // namespace shmt

@@ -546,15 +546,19 @@ struct PendingHop {
 // then holds an unknown number of ids, at most seeds.numel(), and the kernels
 // read the true number there (the count_dev of the hop before, whose unique
 // buffer is `seeds`); every buffer is sized for the bound.
+// With `job` the fused hop is not queued: its launch parameters are written
+// there, for a caller that queues several hops together
+// (shmt_sample_hops_chained); the hop must then be a fused one.
 PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds_len, int64_t num_picks,
-                     bool replace, std::optional<int64_t> seed, int64_t stream_id) {
+                     bool replace, std::optional<int64_t> seed, int64_t stream_id,
+                     shmt_hop_job *job = nullptr) {
   PendingHop h;
   seeds = cuda_ids(seeds, "seeds");
   TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0");
   const int64_t S = seeds.numel();
   const bool fused = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
   if (!fused) {  // degenerate or very large bound: the two operators one after the other
-    TORCH_CHECK(seeds_len == nullptr, "internal: a chained hop must be a fused one");
+    TORCH_CHECK(seeds_len == nullptr && job == nullptr, "internal: a chained hop must be a fused one");
     auto sampled = sample_impl(g.indptr, g.indices, g.cached() ? &*g.gpu_indptr : nullptr,
                                g.cached() ? &*g.gpu_indices : nullptr, g.hashmap, seeds, num_picks,
                                replace, seed, stream_id);
@@ -600,14 +604,40 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds
   char *const scratch_ptr = total_ptr + aligned(total_bytes);
   h.nnz_slot = readback().acquire();
   h.count_slot = readback().acquire();
-  check(shmt_sample_hop_chained(
-      g.indptr_dev, pb, g.indices_dev, ib, g.cached() ? g.gpu_indptr->data_ptr() : nullptr,
-      g.cached() ? g.gpu_indices->data_ptr() : nullptr, g.cached() ? g.hashmap->handle() : nullptr,
-      seeds.data_ptr(), sb, S, seeds_len, num_picks, replace,
-      static_cast<uint64_t>(seed.value_or(kDefaultSeed)), nullptr, static_cast<uint32_t>(stream_id),
-      h.sub_indptr.data_ptr(), h.sub_indices.data_ptr(), plan_ptr, plan_bytes, eb, total_ptr, scratch_ptr,
-      scratch_bytes, h.unique.data_ptr(), h.labels.data_ptr(), h.nnz_slot.dev, h.count_slot.dev, h.count_dev,
-      stream));
+  shmt_hop_job j{};
+  j.indptr = g.indptr_dev;
+  j.ptr_bytes = pb;
+  j.indices = g.indices_dev;
+  j.idx_bytes = ib;
+  j.cache_indptr = g.cached() ? g.gpu_indptr->data_ptr() : nullptr;
+  j.cache_indices = g.cached() ? g.gpu_indices->data_ptr() : nullptr;
+  j.map = g.cached() ? g.hashmap->handle() : nullptr;
+  j.seeds = seeds.data_ptr();
+  j.seed_bytes = sb;
+  j.max_seeds = S;
+  j.seeds_len = seeds_len;
+  j.k = num_picks;
+  j.replace = replace;
+  j.rng_seed = static_cast<uint64_t>(seed.value_or(kDefaultSeed));
+  j.rng_seed_dev = nullptr;
+  j.rng_stream = static_cast<uint32_t>(stream_id);
+  j.sub_indptr = h.sub_indptr.data_ptr();
+  j.sub_indices = h.sub_indices.data_ptr();
+  j.plan = plan_ptr;
+  j.plan_bytes = plan_bytes;
+  j.elem_bytes = eb;
+  j.total_out = total_ptr;
+  j.scratch = scratch_ptr;
+  j.scratch_bytes = scratch_bytes;
+  j.unique_out = h.unique.data_ptr();
+  j.labels_out = h.labels.data_ptr();
+  j.nnz_out = h.nnz_slot.dev;
+  j.count_out = h.count_slot.dev;
+  j.count_dev_out = h.count_dev;
+  if (job)
+    *job = j;
+  else
+    check(shmt_sample_hops_chained(&j, 1, stream));
   return h;
 }
 
@@ -768,6 +798,159 @@ BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<in
   return batch;
 }
 
+// True when every hop of a batch of S seeds can be queued without a host wait
+// (all hops fused, every hop after the first within the chaining bound).
+bool chains_entirely(int64_t S, const std::vector<int64_t> &num_picks) {
+  if (S <= 0 || num_picks.empty()) return false;
+  int64_t bound = S;
+  for (size_t hop = 0; hop < num_picks.size(); ++hop) {
+    const int64_t k = num_picks[hop];
+    if (k <= 0 || k > kEagerOutputLimit / bound) return false;
+    if (hop > 0 && bound > kChainLimit / (k + 1)) return false;
+    bound += bound * k;
+  }
+  return true;
+}
+
+// The hops of several batches in lockstep on the current stream: hop h of all
+// batches goes out in ONE call whose launches are shared between the batches
+// (shmt_sample_hops_chained), then hop h + 1, chained on the device; the sizes
+// of all of them are read at the end. Every batch must chain entirely, so all
+// bounds are known up front: a batch gets one allocation for the results of
+// all its hops and one for their scratch, and result tensors are made once,
+// when the sizes are in (with several batches per launch the host's own
+// bookkeeping, not the GPU, is what bounds the rate).
+struct TogetherHop {
+  int64_t s_max, n_max;
+  int64_t off_sp, off_si, off_unique, off_labels, off_count;  // bytes into the batch's results
+  Readback::Slot nnz, count;
+};
+struct TogetherBatch {
+  torch::Tensor seeds, results, workspace;
+  std::vector<TogetherHop> hops;
+  int sb, eb;
+};
+
+// Queue all hops of the group; finish_together() reads the sizes and makes the results.
+std::vector<TogetherBatch> issue_together(const CsrArgs &g, const std::vector<torch::Tensor> &seeds,
+                                          const std::vector<int64_t> &num_picks, bool replace,
+                                          const std::vector<std::optional<int64_t>> &rng) {
+  using Hop = TogetherHop;
+  using Batch = TogetherBatch;
+  const size_t B = seeds.size(), H = num_picks.size();
+  const int pb = static_cast<int>(g.indptr.element_size());
+  const int ib = static_cast<int>(g.indices.element_size());
+  auto aligned = [](int64_t bytes) { return (bytes + 255) & ~int64_t{255}; };
+  void *stream = current_stream();
+  std::vector<Batch> batches(B);
+  std::vector<std::vector<shmt_hop_job>> jobs(H, std::vector<shmt_hop_job>(B));
+  for (size_t b = 0; b < B; ++b) {
+    Batch &bt = batches[b];
+    bt.seeds = cuda_ids(seeds[b], "seeds");
+    bt.sb = static_cast<int>(bt.seeds.element_size());
+    bt.eb = std::max(bt.sb, ib);
+    bt.hops.resize(H);
+    int64_t results_bytes = 0, work_bytes = 0, s_max = bt.seeds.numel();
+    std::vector<int64_t> off_plan(H), off_total(H), off_scratch(H), plan_bytes(H), scratch_bytes(H);
+    for (size_t h = 0; h < H; ++h) {
+      Hop &hp = bt.hops[h];
+      const int64_t k = num_picks[h];
+      hp.s_max = s_max;
+      hp.n_max = s_max + s_max * k;
+      hp.off_sp = results_bytes;
+      results_bytes += aligned((s_max + 1) * pb);
+      hp.off_si = results_bytes;
+      results_bytes += aligned(s_max * k * ib);
+      hp.off_unique = results_bytes;
+      results_bytes += aligned(hp.n_max * bt.eb);
+      hp.off_labels = results_bytes;
+      results_bytes += aligned(hp.n_max * bt.eb);
+      hp.off_count = results_bytes;
+      results_bytes += 256;
+      plan_bytes[h] = shmt_sample_plan_bytes(s_max);
+      scratch_bytes[h] = shmt_relabel_scratch_bytes(hp.n_max);
+      off_plan[h] = work_bytes;
+      work_bytes += aligned(plan_bytes[h]);
+      off_total[h] = work_bytes;
+      work_bytes += aligned(hp.n_max * bt.eb);
+      off_scratch[h] = work_bytes;
+      work_bytes += aligned(scratch_bytes[h]);
+      s_max = hp.n_max;
+    }
+    bt.results = device_bytes(results_bytes);
+    bt.workspace = device_bytes(work_bytes);
+    char *const r = static_cast<char *>(bt.results.data_ptr());
+    char *const w = static_cast<char *>(bt.workspace.data_ptr());
+    for (size_t h = 0; h < H; ++h) {
+      Hop &hp = bt.hops[h];
+      hp.nnz = readback().acquire();
+      hp.count = readback().acquire();
+      shmt_hop_job &j = jobs[h][b];
+      j = shmt_hop_job{};
+      j.indptr = g.indptr_dev;
+      j.ptr_bytes = pb;
+      j.indices = g.indices_dev;
+      j.idx_bytes = ib;
+      j.cache_indptr = g.cached() ? g.gpu_indptr->data_ptr() : nullptr;
+      j.cache_indices = g.cached() ? g.gpu_indices->data_ptr() : nullptr;
+      j.map = g.cached() ? g.hashmap->handle() : nullptr;
+      j.seeds = h == 0 ? bt.seeds.data_ptr() : static_cast<void *>(r + bt.hops[h - 1].off_unique);
+      j.seed_bytes = h == 0 ? bt.sb : bt.eb;
+      j.max_seeds = hp.s_max;
+      j.seeds_len = h == 0 ? nullptr : reinterpret_cast<const int64_t *>(r + bt.hops[h - 1].off_count);
+      j.k = num_picks[h];
+      j.replace = replace;
+      j.rng_seed = static_cast<uint64_t>(rng[b].value_or(kDefaultSeed));
+      j.rng_seed_dev = nullptr;
+      j.rng_stream = static_cast<uint32_t>(rng[b].has_value() ? h : 0);
+      j.sub_indptr = r + hp.off_sp;
+      j.sub_indices = r + hp.off_si;
+      j.plan = w + off_plan[h];
+      j.plan_bytes = plan_bytes[h];
+      j.elem_bytes = bt.eb;
+      j.total_out = w + off_total[h];
+      j.scratch = w + off_scratch[h];
+      j.scratch_bytes = scratch_bytes[h];
+      j.unique_out = r + hp.off_unique;
+      j.labels_out = r + hp.off_labels;
+      j.nnz_out = hp.nnz.dev;
+      j.count_out = hp.count.dev;
+      j.count_dev_out = reinterpret_cast<int64_t *>(r + hp.off_count);
+    }
+  }
+  for (size_t h = 0; h < H; ++h)
+    check(shmt_sample_hops_chained(jobs[h].data(), static_cast<int>(B), stream));
+  return batches;
+}
+
+// Must run with the stream of issue_together current.
+std::vector<BatchResult> finish_together(const CsrArgs &g, std::vector<TogetherBatch> &batches) {
+  const size_t B = batches.size();
+  const int pb = static_cast<int>(g.indptr.element_size());
+  const int ib = static_cast<int>(g.indices.element_size());
+  // sizes in, batch by batch; typed views of the results buffer are made from two typed aliases of it
+  std::vector<BatchResult> out(B);
+  for (size_t b = 0; b < B; ++b) {
+    TogetherBatch &bt = batches[b];
+    const size_t H = bt.hops.size();
+    const torch::Tensor as32 = bt.results.view(torch::kInt32), as64 = bt.results.view(torch::kInt64);
+    auto typed = [&](int64_t off, int64_t first, int64_t count, int elem) {
+      return (elem == 8 ? as64 : as32).narrow(0, off / elem + first, count);
+    };
+    int64_t s_now = bt.seeds.numel();
+    out[b].hops.reserve(H);
+    for (size_t h = 0; h < H; ++h) {
+      const TogetherHop &hp = bt.hops[h];
+      const int64_t nnz = Readback::wait(hp.nnz);
+      const int64_t U = Readback::wait(hp.count);
+      out[b].hops.emplace_back(typed(hp.off_sp, 0, s_now + 1, pb), typed(hp.off_si, 0, nnz, ib),
+                               typed(hp.off_unique, 0, U, bt.eb), typed(hp.off_labels, s_now, nnz, bt.eb));
+      s_now = U;
+    }
+  }
+  return out;
+}
+
 // Multi-hop sampling of several independent seed batches. Every batch is a
 // chain of short, latency-bound kernels with a host read of the sizes at its end,
 // so one batch alone leaves most of the GPU idle. Here up to `max_in_flight`
@@ -798,6 +981,48 @@ std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch
     py::gil_scoped_release no_gil;  // lets a Python thread that prefetches batches run beside the caller
     for (int64_t b = 0; b < B; ++b) out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b), features);
     return out;
+  }
+  if (!features) {
+    // Batches whose hops all chain on the device advance in lockstep and share their launches:
+    // up to 8 of them per kernel launch, on the caller's stream, without helper threads.
+    bool any = false;
+    for (int64_t b = 0; b < B; ++b) any = any || chains_entirely(seeds[b].numel(), num_picks);
+    if (any) {
+      py::gil_scoped_release no_gil;
+      const size_t group_size = static_cast<size_t>(std::min<int64_t>(K, 8));
+      std::vector<int64_t> group;
+      // one group is queued ahead of the one whose sizes are being read, so the GPU never waits
+      // for the host's bookkeeping
+      std::deque<std::pair<std::vector<int64_t>, std::vector<TogetherBatch>>> queued;
+      auto finish_oldest = [&]() {
+        std::vector<BatchResult> done = finish_together(g, queued.front().second);
+        for (size_t i = 0; i < done.size(); ++i) out[queued.front().first[i]] = std::move(done[i]);
+        queued.pop_front();
+      };
+      auto flush = [&]() {
+        if (group.empty()) return;
+        std::vector<torch::Tensor> group_seeds;
+        std::vector<std::optional<int64_t>> group_rng;
+        for (int64_t b : group) {
+          group_seeds.push_back(seeds[b]);
+          group_rng.push_back(rng_of(b));
+        }
+        queued.emplace_back(group, issue_together(g, group_seeds, num_picks, replace, group_rng));
+        group.clear();
+        if (queued.size() > 1) finish_oldest();
+      };
+      for (int64_t b = 0; b < B; ++b) {
+        if (chains_entirely(seeds[b].numel(), num_picks)) {
+          group.push_back(b);
+          if (group.size() == group_size) flush();
+        } else {
+          out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b), nullptr);
+        }
+      }
+      flush();
+      while (!queued.empty()) finish_oldest();
+      return out;
+    }
   }
   const auto caller = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
   const c10::DeviceIndex device = caller.device_index();

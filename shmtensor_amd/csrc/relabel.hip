@@ -177,15 +177,28 @@ constexpr int kRlLdsSlots = 2 * kRlInsertTile;   // per-workgroup staging table,
 // de-duplicates its 256 ids in an LDS table (key -> smallest index among
 // them) and sends one global insert per distinct id, issued by the thread that
 // holds the id's smallest index: at most one global probe chain per thread.
-__global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32_t cap,
-                                                             const void *total, int eb, RlCount n,
-                                                             RlPath path) {
-  const int64_t N = rl_count(n);
-  const bool packed = rl_packed(path);
+struct RlInsertArgs {
+  RlSlot *tbl;
+  uint32_t cap;
+  const void *total;
+  int eb;
+  RlCount n;
+  RlPath path;
+};
+
+// (bx, gx): this workgroup's index and the number of workgroups of its job:
+// blockIdx.x / gridDim.x of a plain launch, the job's share of a merged one.
+__device__ __forceinline__ void rl_insert_body(unsigned bx, unsigned gx, const RlInsertArgs &a) {
+  RlSlot *const tbl = a.tbl;
+  const uint32_t cap = a.cap;
+  const void *const total = a.total;
+  const int eb = a.eb;
+  const int64_t N = rl_count(a.n);
+  const bool packed = rl_packed(a.path);
   __shared__ unsigned long long lkey[kRlLdsSlots];
   __shared__ uint32_t lfirst[kRlLdsSlots];
   const int64_t ntiles = (N + kRlInsertTile - 1) / kRlInsertTile;
-  for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+  for (int64_t tile = bx; tile < ntiles; tile += gx) {
     for (int t = threadIdx.x; t < kRlLdsSlots; t += kRlBlock) {
       lkey[t] = ~0ull;
       lfirst[t] = 0xFFFFFFFFu;
@@ -222,6 +235,14 @@ __global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlSlot *tbl, uint32
   }
 }
 
+__global__ __launch_bounds__(kRlBlock) void rl_insert_kernel(RlInsertArgs a) {
+  rl_insert_body(blockIdx.x, gridDim.x, a);
+}
+
+__global__ __launch_bounds__(kRlBlock) void rl_insert_jobs(Jobs<RlInsertArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rl_insert_body(blockIdx.x, j.blocks[blockIdx.y], j.a[blockIdx.y]);
+}
+
 // First-occurrence index of every element: one id per thread, a workgroup of
 // kRlTile threads per tile (the tile whose count of first occurrences the
 // unique pass ranks). One id per thread keeps every value in registers and
@@ -254,47 +275,79 @@ __device__ __forceinline__ uint32_t rl_first_of(const RlSlot *tbl, uint32_t cap,
   return 0xFFFFFFFFu;
 }
 
-__global__ __launch_bounds__(kRlTile) void rl_first_kernel(const RlSlot *tbl, uint32_t cap,
-                                                           const void *total, int eb, RlCount n,
-                                                           void *labels, uint64_t *partials,
-                                                           RlPath path) {
-  const int64_t N = rl_count(n);
+struct RlFirstArgs {
+  const RlSlot *tbl;
+  uint32_t cap;
+  const void *total;
+  int eb;
+  RlCount n;
+  void *labels;
+  uint64_t *partials;
+  RlPath path;
+};
+
+__device__ __forceinline__ void rl_first_body(unsigned bx, const RlFirstArgs &a) {
+  const int64_t N = rl_count(a.n);
+  // launched for a bound of N: tiles past the ids have nothing to do, and nobody reads their count
+  if (static_cast<int64_t>(bx) * kRlTile >= N) return;
   __shared__ uint64_t lds[kRlTile / kWave];
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kRlTile + threadIdx.x;
+  const int64_t i = static_cast<int64_t>(bx) * kRlTile + threadIdx.x;
   uint64_t cnt = 0;
   if (i < N) {
-    const int64_t key = load_int(total, i, eb);
-    const uint32_t f = rl_packed(path) ? rl_first_of<true>(tbl, cap, key) : rl_first_of<false>(tbl, cap, key);
-    store_int(labels, i, eb, static_cast<int64_t>(f));
+    const int64_t key = load_int(a.total, i, a.eb);
+    const uint32_t f = rl_packed(a.path) ? rl_first_of<true>(a.tbl, a.cap, key) : rl_first_of<false>(a.tbl, a.cap, key);
+    store_int(a.labels, i, a.eb, static_cast<int64_t>(f));
     cnt = (f == static_cast<uint32_t>(i));
   }
   uint64_t tile_total;
   block_exclusive_scan<uint64_t, kRlTile>(cnt, lds, &tile_total);
-  if (threadIdx.x == 0) partials[blockIdx.x] = tile_total;
+  if (threadIdx.x == 0) a.partials[bx] = tile_total;
 }
 
-__global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, int eb, RlCount n,
-                                                             const void *labels,
-                                                             const uint64_t *partials,
-                                                             void *unique_out, uint32_t *rank_of,
-                                                             int64_t *count_out, int64_t *count_copy,
-                                                             int scanned) {
-  const int64_t N = rl_count(n);
+__global__ __launch_bounds__(kRlTile) void rl_first_kernel(RlFirstArgs a) { rl_first_body(blockIdx.x, a); }
+
+__global__ __launch_bounds__(kRlTile) void rl_first_jobs(Jobs<RlFirstArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rl_first_body(blockIdx.x, j.a[blockIdx.y]);
+}
+
+struct RlUniqueArgs {
+  const void *total;
+  int eb;
+  RlCount n;
+  const void *labels;
+  const uint64_t *partials;
+  void *unique_out;
+  uint32_t *rank_of;
+  int64_t *count_out;
+  int64_t *count_copy;
+  int scanned;
+};
+
+__device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &a) {
+  const void *const total = a.total;
+  const int eb = a.eb;
+  const void *const labels = a.labels;
+  const uint64_t *const partials = a.partials;
+  void *const unique_out = a.unique_out;
+  uint32_t *const rank_of = a.rank_of;
+  const int64_t N = rl_count(a.n);
+  // launched for a bound of N: only the tiles that hold ids work (tile 0 reports N = 0)
+  if (bx > 0 && static_cast<int64_t>(bx) * kRlTile >= N) return;
   __shared__ uint32_t lds[kRlBlock / kWave];
   __shared__ uint64_t lds64[kRlBlock / kWave];
   // Tile prefix: either already scanned by a separate launch, or (few tiles)
   // summed here from the raw per-tile counts.
   uint64_t tile_prefix;
-  if (scanned) {
-    tile_prefix = partials[blockIdx.x];
+  if (a.scanned) {
+    tile_prefix = partials[bx];
   } else {
     uint64_t part = 0;
-    for (int t = threadIdx.x; t < static_cast<int>(blockIdx.x); t += kRlBlock) part += partials[t];
+    for (int t = threadIdx.x; t < static_cast<int>(bx); t += kRlBlock) part += partials[t];
     uint64_t below;
     block_exclusive_scan<uint64_t, kRlBlock>(part, lds64, &below);
     tile_prefix = below;
   }
-  const int64_t first_i = static_cast<int64_t>(blockIdx.x) * kRlTile +
+  const int64_t first_i = static_cast<int64_t>(bx) * kRlTile +
                           static_cast<int64_t>(threadIdx.x) * kRlItems;
   bool win[kRlItems], ok[kRlItems];
   int64_t idx[kRlItems], lab[kRlItems], val[kRlItems];
@@ -327,21 +380,41 @@ __global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(const void *total, 
   }
   // the workgroup holding the last id reports the number of distinct ids
   const int64_t last_tile = N > 0 ? (N - 1) / kRlTile : 0;
-  if (static_cast<int64_t>(blockIdx.x) == last_tile && threadIdx.x == 0) {
-    if (count_copy) *count_copy = static_cast<int64_t>(tile_prefix + tile_total);
-    publish_size(count_out, static_cast<int64_t>(tile_prefix + tile_total));
+  if (static_cast<int64_t>(bx) == last_tile && threadIdx.x == 0) {
+    if (a.count_copy) *a.count_copy = static_cast<int64_t>(tile_prefix + tile_total);
+    publish_size(a.count_out, static_cast<int64_t>(tile_prefix + tile_total));
   }
 }
 
-__global__ __launch_bounds__(256) void rl_labels_kernel(void *labels, int eb, RlCount n,
-                                                        const uint32_t *rank_of) {
-  const int64_t N = rl_count(n);
-  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+__global__ __launch_bounds__(kRlBlock) void rl_unique_kernel(RlUniqueArgs a) { rl_unique_body(blockIdx.x, a); }
+
+__global__ __launch_bounds__(kRlBlock) void rl_unique_jobs(Jobs<RlUniqueArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rl_unique_body(blockIdx.x, j.a[blockIdx.y]);
+}
+
+struct RlLabelsArgs {
+  void *labels;
+  int eb;
+  RlCount n;
+  const uint32_t *rank_of;
+};
+
+__device__ __forceinline__ void rl_labels_body(unsigned bx, unsigned gx, const RlLabelsArgs &a) {
+  const int64_t N = rl_count(a.n);
+  int64_t i = static_cast<int64_t>(bx) * blockDim.x + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gx) * blockDim.x;
   for (; i < N; i += stride) {
-    const int64_t f = load_int(labels, i, eb);
-    store_int(labels, i, eb, static_cast<int64_t>(rank_of[f]));
+    const int64_t f = load_int(a.labels, i, a.eb);
+    store_int(a.labels, i, a.eb, static_cast<int64_t>(a.rank_of[f]));
   }
+}
+
+__global__ __launch_bounds__(256) void rl_labels_kernel(RlLabelsArgs a) {
+  rl_labels_body(blockIdx.x, gridDim.x, a);
+}
+
+__global__ __launch_bounds__(256) void rl_labels_jobs(Jobs<RlLabelsArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rl_labels_body(blockIdx.x, j.blocks[blockIdx.y], j.a[blockIdx.y]);
 }
 
 struct RlSegments {
@@ -386,11 +459,27 @@ constexpr int kRlSmallItems = kRlSmallMax / kRlSmallBlock;
 constexpr int kRlSmallSlots = 2 * kRlSmallMax;
 static_assert(kRlSmallItems == 8, "the rank scan packs eight 16-bit counters into two words");
 
+struct RlSmallArgs {
+  const void *total_in;  // the ids (SEGS = false)
+  void *total_out;       // receives the concatenated ids (SEGS = true)
+  int eb;
+  RlCount n;
+  void *unique_out;
+  void *labels_out;
+  int64_t *count_out;
+  int64_t *count_copy;
+};
+
 template <bool SEGS>
-__global__ __launch_bounds__(kRlSmallBlock) void rl_small_kernel(const void *total_in, RlSegments segs,
-                                                                 void *total_out, int eb, RlCount n,
-                                                                 void *unique_out, void *labels_out,
-                                                                 int64_t *count_out, int64_t *count_copy) {
+__device__ __forceinline__ void rl_small_body(const RlSmallArgs &a, const RlSegments &segs) {
+  const void *const total_in = a.total_in;
+  void *const total_out = a.total_out;
+  const int eb = a.eb;
+  const RlCount n = a.n;
+  void *const unique_out = a.unique_out;
+  void *const labels_out = a.labels_out;
+  int64_t *const count_out = a.count_out;
+  int64_t *const count_copy = a.count_copy;
   __shared__ int64_t keys[kRlSmallMax];
   __shared__ uint32_t tbl[kRlSmallSlots];
   __shared__ uint64_t scan_lds[kRlSmallBlock / kWave];
@@ -491,6 +580,18 @@ __global__ __launch_bounds__(kRlSmallBlock) void rl_small_kernel(const void *tot
   }
 }
 
+__global__ __launch_bounds__(kRlSmallBlock) void rl_small_segments_kernel(RlSmallArgs a, RlSegments segs) {
+  rl_small_body<true>(a, segs);
+}
+
+__global__ __launch_bounds__(kRlSmallBlock) void rl_small_kernel(RlSmallArgs a) {
+  rl_small_body<false>(a, RlSegments{});
+}
+
+__global__ __launch_bounds__(kRlSmallBlock) void rl_small_jobs(Jobs<RlSmallArgs> j) {
+  rl_small_body<false>(j.a[blockIdx.y], RlSegments{});
+}
+
 __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
   if (count_copy) *count_copy = 0;
   publish_size(count_out, 0);
@@ -521,15 +622,20 @@ int64_t shmt_relabel_scratch_bytes(int64_t N) {
 // kernels work on the true count.
 static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, RlCount n,
                         int elem_bytes, void *scratch, int64_t scratch_bytes, void *unique_out,
-                        void *labels_out, int64_t *count_out, void *stream, bool prepared = false,
+                        void *labels_out, int64_t *count_out, Launcher launcher, bool prepared = false,
                         uint64_t prepared_nonce = 0, int64_t *count_copy = nullptr,
                         int64_t prepared_slots = 0) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
   SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
   SHMT_REQUIRE(count_out != nullptr, "shmt_relabel: count_out is null");
-  hipStream_t s = as_stream(stream);
+  hipStream_t s = launcher.stream;
+  StageList *const defer = launcher.defer;  // only the fused hop (prepared) records its launches
   if (N == 0) {
+    if (defer) {
+      defer->mergeable = false;
+      return SHMT_OK;
+    }
     hipLaunchKernelGGL(rl_zero_count_kernel, dim3(1), dim3(1), 0, s, count_out, count_copy);
     SHMT_LAUNCH_CHECK();
     return SHMT_OK;
@@ -557,18 +663,39 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   RlPath path{elem_bytes == 4 ? 1 : ((prepared || segs) ? 2 : 0), wide_mark, nonce};
 
   if (N <= kRlSmallMax) {
+    const RlSmallArgs a{segs ? nullptr : total, segs ? const_cast<void *>(total) : nullptr, elem_bytes, n,
+                        unique_out, labels_out, count_out, count_copy};
+    if (defer) {
+      if (segs) defer->mergeable = false; else stage_push(defer, kStageRlSmall, 1, kRlSmallBlock, a);
+      return SHMT_OK;
+    }
     if (segs)
-      hipLaunchKernelGGL(rl_small_kernel<true>, dim3(1), dim3(kRlSmallBlock), 0, s, nullptr, *segs,
-                         const_cast<void *>(total), elem_bytes, n, unique_out, labels_out, count_out,
-                         count_copy);
+      hipLaunchKernelGGL(rl_small_segments_kernel, dim3(1), dim3(kRlSmallBlock), 0, s, a, *segs);
     else
-      hipLaunchKernelGGL(rl_small_kernel<false>, dim3(1), dim3(kRlSmallBlock), 0, s, total, RlSegments{},
-                         nullptr, elem_bytes, n, unique_out, labels_out, count_out, count_copy);
+      hipLaunchKernelGGL(rl_small_kernel, dim3(1), dim3(kRlSmallBlock), 0, s, a);
     SHMT_LAUNCH_CHECK();
     return SHMT_OK;
   }
 
   int rc = SHMT_OK;
+  const int scanned = nb > kRlSelfPrefixTiles;
+  const RlInsertArgs ins{tbl, cap, total, elem_bytes, n, path};
+  const RlFirstArgs fst{tbl, cap, total, elem_bytes, n, labels_out, partials, path};
+  const RlUniqueArgs unq{total, elem_bytes, n, labels_out, partials, unique_out, rank_of, count_out, count_copy,
+                         scanned};
+  const RlLabelsArgs lab{labels_out, elem_bytes, n, rank_of};
+  const unsigned ins_blocks = grid_for(N, kRlInsertTile, 256 * 32), lab_blocks = grid_for(N, 256);
+  if (defer) {
+    if (!prepared || scanned) {
+      defer->mergeable = false;
+      return SHMT_OK;
+    }
+    stage_push(defer, kStageRlInsert, ins_blocks, kRlBlock, ins);
+    stage_push(defer, kStageRlFirst, static_cast<unsigned>(nb), kRlTile, fst);
+    stage_push(defer, kStageRlUnique, static_cast<unsigned>(nb), kRlBlock, unq);
+    stage_push(defer, kStageRlLabels, lab_blocks, 256, lab);
+    return SHMT_OK;
+  }
   if (prepared) {
     // the caller's earlier kernels on this stream emptied the table and wrote `total`
   } else if (segs) {
@@ -581,23 +708,17 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     rc = launch_fill_ones(tbl, l.cap, s);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(rl_insert_kernel, dim3(grid_for(N, kRlInsertTile, 256 * 32)), dim3(kRlBlock), 0,
-                     s, tbl, cap, total, elem_bytes, n, path);
+  hipLaunchKernelGGL(rl_insert_kernel, dim3(ins_blocks), dim3(kRlBlock), 0, s, ins);
   SHMT_LAUNCH_CHECK();
-  hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlTile), 0, s, tbl,
-                     cap, total, elem_bytes, n, labels_out, partials, path);
+  hipLaunchKernelGGL(rl_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlTile), 0, s, fst);
   SHMT_LAUNCH_CHECK();
-  const int scanned = nb > kRlSelfPrefixTiles;
   if (scanned) {
     rc = launch_scan_partials(partials, nb, s);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s,
-                     total, elem_bytes, n, labels_out, partials, unique_out, rank_of, count_out,
-                     count_copy, scanned);
+  hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, unq);
   SHMT_LAUNCH_CHECK();
-  hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, labels_out,
-                     elem_bytes, n, rank_of);
+  hipLaunchKernelGGL(rl_labels_kernel, dim3(lab_blocks), dim3(256), 0, s, lab);
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;
 }
@@ -629,11 +750,52 @@ int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scrat
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const int64_t *n_fixed_dev,
                           const void *n_extra_dev, int n_extra_bytes, int elem_bytes, void *scratch,
                           int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
-                          int64_t *count_copy, const RelabelTable &table, hipStream_t stream) {
+                          int64_t *count_copy, const RelabelTable &table, Launcher launcher) {
   return relabel_impl(total, nullptr, n_bound,
                       RlCount{n_fixed, n_fixed_dev, n_extra_dev, n_extra_bytes, n_bound}, elem_bytes,
-                      scratch, scratch_bytes, unique_out, labels_out, count_out, stream, true, table.nonce,
+                      scratch, scratch_bytes, unique_out, labels_out, count_out, launcher, true, table.nonce,
                       count_copy, table.n16);
+}
+
+int launch_merged_relabel_stage(int n_jobs, const Stage *const *stages, hipStream_t s) {
+  const unsigned threads = stages[0]->threads;
+  switch (stages[0]->kind) {
+    case kStageRlSmall: {
+      Jobs<RlSmallArgs> j;
+      jobs_from_stages(n_jobs, stages, &j);
+      hipLaunchKernelGGL(rl_small_jobs, dim3(1, n_jobs), dim3(threads), 0, s, j);
+      break;
+    }
+    case kStageRlInsert: {
+      Jobs<RlInsertArgs> j;
+      const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+      hipLaunchKernelGGL(rl_insert_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
+      break;
+    }
+    case kStageRlFirst: {
+      Jobs<RlFirstArgs> j;
+      const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+      hipLaunchKernelGGL(rl_first_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
+      break;
+    }
+    case kStageRlUnique: {
+      Jobs<RlUniqueArgs> j;
+      const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+      hipLaunchKernelGGL(rl_unique_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
+      break;
+    }
+    case kStageRlLabels: {
+      Jobs<RlLabelsArgs> j;
+      const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+      hipLaunchKernelGGL(rl_labels_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
+      break;
+    }
+    default:
+      set_error("internal: stage kind %d has no merged relabel launch", stages[0]->kind);
+      return SHMT_EINVAL;
+  }
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
 }
 
 }  // namespace shmt
@@ -644,7 +806,7 @@ int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,
                  void *stream) {
   return relabel_impl(total, nullptr, N, RlCount{N, nullptr, nullptr, 8, N}, elem_bytes, scratch, scratch_bytes,
-                      unique_out, labels_out, count_out, stream);
+                      unique_out, labels_out, count_out, Launcher{as_stream(stream), nullptr});
 }
 
 int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, const int *seg_bytes,
@@ -683,7 +845,7 @@ int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, 
     n.extra_bytes = last_len_bytes;
   }
   return relabel_impl(total_out, &segs, N, n, elem_bytes, scratch, scratch_bytes, unique_out,
-                      labels_out, count_out, stream);
+                      labels_out, count_out, Launcher{as_stream(stream), nullptr});
 }
 
 }  // extern "C"

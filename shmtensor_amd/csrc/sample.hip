@@ -104,7 +104,7 @@ __device__ __forceinline__ int64_t plan_one(const PlanArgs &a, int64_t S, int64_
 
 // One workgroup walks all seeds with a running carry and writes final offsets.
 template <int MODE>
-__global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
+__device__ __forceinline__ void plan_single_body(const PlanArgs &a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
   const int64_t S = seed_count(a.S, a.S_len);
   uint64_t carry = 0;
@@ -123,20 +123,46 @@ __global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
   }
 }
 
-// Multi-workgroup form: tile-local offsets + one total per tile.
 template <int MODE>
-__global__ __launch_bounds__(kPlanBlock) void plan_tile_kernel(PlanArgs a) {
+__global__ __launch_bounds__(kPlanBlock) void plan_single_kernel(PlanArgs a) {
+  plan_single_body<MODE>(a);
+}
+
+// Merged form (see launchers.h): blockIdx.y selects the job.
+template <int MODE>
+__global__ __launch_bounds__(kPlanBlock) void plan_single_jobs(Jobs<PlanArgs> j) {
+  plan_single_body<MODE>(j.a[blockIdx.y]);
+}
+
+// Multi-workgroup form: tile-local offsets + one total per tile. (bx, gx):
+// this workgroup's index and the number of workgroups of its job.
+template <int MODE>
+__device__ __forceinline__ void plan_tile_body(unsigned bx, unsigned gx, const PlanArgs &a) {
   __shared__ uint64_t lds[kPlanBlock / kWave];
   const int64_t S = seed_count(a.S, a.S_len);
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kPlanBlock + threadIdx.x;
+  if (bx > 0 && static_cast<int64_t>(bx) * kPlanBlock >= S) {  // launched for a bound of S: an empty tile
+    if (threadIdx.x == 0) a.partials[bx] = 0;
+    return;
+  }
+  const int64_t i = static_cast<int64_t>(bx) * kPlanBlock + threadIdx.x;
   const uint64_t cnt = static_cast<uint64_t>(plan_one<MODE>(a, S, i));
   uint64_t total;
   const uint64_t ex = block_exclusive_scan<uint64_t, kPlanBlock>(cnt, lds, &total);
   if (i < S) store_int(a.sub_indptr, i, a.ptr_bytes, static_cast<int64_t>(ex));
   if (threadIdx.x == 0) {
-    a.partials[blockIdx.x] = total;
-    if (blockIdx.x == 0) a.partials[gridDim.x] = 0;  // becomes the grand total after the scan
+    a.partials[bx] = total;
+    if (bx == 0) a.partials[gx] = 0;  // becomes the grand total after the scan
   }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kPlanBlock) void plan_tile_kernel(PlanArgs a) {
+  plan_tile_body<MODE>(blockIdx.x, gridDim.x, a);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kPlanBlock) void plan_tile_jobs(Jobs<PlanArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) plan_tile_body<MODE>(blockIdx.x, j.blocks[blockIdx.y], j.a[blockIdx.y]);
 }
 
 // Adds the scanned tile offsets to the tile-local offsets. partials holds
@@ -238,8 +264,8 @@ __device__ __forceinline__ int64_t pick_tile_base(const PickArgs &a, int64_t s) 
 }
 
 // With raw tile totals nobody has published the grand total yet: the first wave of the grid does.
-__device__ __forceinline__ void pick_publish_total(const PickArgs &a, int64_t S) {
-  if (!a.raw_tiles || blockIdx.x != 0 || threadIdx.x >= kWave) return;
+__device__ __forceinline__ void pick_publish_total(const PickArgs &a, int64_t S, unsigned bx) {
+  if (!a.raw_tiles || bx != 0 || threadIdx.x >= kWave) return;
   const int64_t total = wave_sum_tiles(a.tile_prefix, a.raw_tiles);
   if (threadIdx.x == 0) {
     store_int(a.sub_indptr_rw, S, a.ptr_bytes, total);
@@ -272,11 +298,11 @@ __device__ __forceinline__ void pick_store(const PickArgs &a, int64_t S, int64_t
 }
 
 template <bool HOP>
-__device__ __forceinline__ void pick_clear(const PickArgs &a) {
+__device__ __forceinline__ void pick_clear(const PickArgs &a, unsigned bx, unsigned gx) {
   if (!HOP) return;
   const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.clear_n; i += stride)
+  const int64_t stride = static_cast<int64_t>(gx) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(bx) * blockDim.x + threadIdx.x; i < a.clear_n; i += stride)
     a.clear[i] = ones;
 }
 
@@ -285,22 +311,23 @@ __device__ __forceinline__ int64_t load_adj(const PickArgs &a, int64_t begin_tag
   return load_int(base, (begin_tagged & ~kCachedTag) + pos, a.idx_bytes);
 }
 
-// k <= 64: group of G = 2^log2_group >= k lanes per seed.
+// k <= 64: group of G = 2^log2_group >= k lanes per seed. (bx, gx): this
+// workgroup's index and the number of workgroups of its job.
 template <bool HOP>
-__global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
-  pick_clear<HOP>(a);
+__device__ __forceinline__ void pick_narrow_body(unsigned bx, unsigned gx, const PickArgs &a) {
+  pick_clear<HOP>(a, bx, gx);
   const int lane = lane_id();
   const int G = 1 << a.log2_group;
   const int gl = lane & (G - 1);
   const int gbase = lane & ~(G - 1);
   const int groups_per_wave = kWave >> a.log2_group;
   const int64_t waves_per_block = blockDim.x / kWave;
-  const int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + threadIdx.x / kWave;
-  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
+  const int64_t wave = static_cast<int64_t>(bx) * waves_per_block + threadIdx.x / kWave;
+  const int64_t nwaves = static_cast<int64_t>(gx) * waves_per_block;
   const int k = static_cast<int>(a.k);
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
   const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
-  if (HOP) pick_publish_total(a, S);
+  if (HOP) pick_publish_total(a, S, bx);
 
   for (int64_t s0 = wave * groups_per_wave; s0 < S; s0 += nwaves * groups_per_wave) {
     // the seeds of a wave share a plan tile (tiles hold a multiple of groups_per_wave seeds)
@@ -338,6 +365,15 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
   }
 }
 
+template <bool HOP>
+__global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
+  pick_narrow_body<HOP>(blockIdx.x, gridDim.x, a);
+}
+
+__global__ __launch_bounds__(256) void pick_narrow_hop_jobs(Jobs<PickArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) pick_narrow_body<true>(blockIdx.x, j.blocks[blockIdx.y], j.a[blockIdx.y]);
+}
+
 // k > 64: one wave (= one 64-thread workgroup) per seed. The chosen positions
 // are staged in LDS when k fits (IN_LDS), otherwise in the seed's own output
 // segment, which is overwritten by the gathered neighbours at the end
@@ -345,12 +381,12 @@ __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
 template <bool IN_LDS, bool HOP>
 __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
   extern __shared__ int64_t chosen_lds[];
-  pick_clear<HOP>(a);
+  pick_clear<HOP>(a, blockIdx.x, gridDim.x);
   const int lane = threadIdx.x;
   const int64_t k = a.k;
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
   const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
-  if (HOP) pick_publish_total(a, S);
+  if (HOP) pick_publish_total(a, S, blockIdx.x);
   for (int64_t s = blockIdx.x; s < S; s += gridDim.x) {
     const SeedPlan p = a.plan[s];
     const int64_t deg = p.deg;
@@ -491,7 +527,7 @@ struct PlanHopExtras {
 static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr,
                      const shmt_hashmap_t *map, const void *seeds, int seed_bytes, int64_t S,
                      int64_t k, int replace, void *sub_indptr, void *plan, int64_t plan_bytes,
-                     int64_t *nnz_out, void *stream, PlanHopExtras *hop) {
+                     int64_t *nnz_out, Launcher launcher, PlanHopExtras *hop) {
   SHMT_REQUIRE(S >= 0, "shmt_sample_plan: S must be >= 0");
   SHMT_REQUIRE(k >= 0, "shmt_sample_plan: num_picks must be >= 0");
   SHMT_REQUIRE(width_ok(ptr_bytes) && width_ok(seed_bytes),
@@ -509,7 +545,8 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
     SHMT_REQUIRE((reinterpret_cast<uintptr_t>(plan) & 15) == 0,
                  "shmt_sample_plan: plan must be 16-byte aligned");
   }
-  hipStream_t s = as_stream(stream);
+  hipStream_t s = launcher.stream;
+  StageList *const defer = launcher.defer;
   PlanArgs a;
   a.indptr = indptr;
   a.cache_indptr = cache_indptr;
@@ -538,6 +575,10 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   const int mode = map ? (map->fmt == kSlot16 ? 1 : 2) : 0;
 
   if (S <= kPlanSingleMax) {
+    if (defer) {
+      stage_push(defer, kStagePlanSingle + mode, 1, kPlanBlock, a);
+      return SHMT_OK;
+    }
     switch (mode) {
       case 0: hipLaunchKernelGGL(plan_single_kernel<0>, dim3(1), dim3(kPlanBlock), 0, s, a); break;
       case 1: hipLaunchKernelGGL(plan_single_kernel<1>, dim3(1), dim3(kPlanBlock), 0, s, a); break;
@@ -549,6 +590,16 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   const int64_t nb = (S + kPlanBlock - 1) / kPlanBlock;
   SHMT_REQUIRE(nb < (1ll << 31), "shmt_sample_plan: too many seeds");
   const dim3 grid(static_cast<unsigned>(nb));
+  if (defer) {
+    if (!hop || nb > kPickSumsTiles) {
+      defer->mergeable = false;
+      return SHMT_OK;
+    }
+    stage_push(defer, kStagePlanTile + mode, static_cast<unsigned>(nb), kPlanBlock, a);
+    hop->tile_prefix_out = a.partials;
+    hop->raw_tiles_out = nb;
+    return SHMT_OK;
+  }
   switch (mode) {
     case 0: hipLaunchKernelGGL(plan_tile_kernel<0>, grid, dim3(kPlanBlock), 0, s, a); break;
     case 1: hipLaunchKernelGGL(plan_tile_kernel<1>, grid, dim3(kPlanBlock), 0, s, a); break;
@@ -580,7 +631,7 @@ int shmt_sample_plan(const void *indptr, int ptr_bytes, const void *cache_indptr
                      int64_t k, int replace, void *sub_indptr, void *plan, int64_t plan_bytes,
                      int64_t *nnz_out, void *stream) {
   return plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr,
-                   plan, plan_bytes, nnz_out, stream, nullptr);
+                   plan, plan_bytes, nnz_out, Launcher{as_stream(stream), nullptr}, nullptr);
 }
 
 }  // extern "C"
@@ -602,7 +653,9 @@ struct PickHopExtras {
 };
 
 template <bool HOP>
-static int pick_launch(const PickArgs &a, hipStream_t s) {
+static int pick_launch(const PickArgs &a, Launcher launcher) {
+  hipStream_t s = launcher.stream;
+  StageList *const defer = launcher.defer;
   const int64_t S = a.S, k = a.k;
   if (k <= kWave) {
     // Few seeds: one wave per workgroup, so that the cold rows' host-link reads come from as many
@@ -619,7 +672,14 @@ static int pick_launch(const PickArgs &a, hipStream_t s) {
       const int64_t for_clear = (a.clear_n + threads * 4 - 1) / (threads * 4);
       if (blocks < for_clear) blocks = for_clear;
     }
+    if (defer) {
+      if (HOP) stage_push(defer, kStagePickNarrowHop, grid_for(blocks, 1), threads, a); else defer->mergeable = false;
+      return SHMT_OK;
+    }
     hipLaunchKernelGGL(pick_narrow_kernel<HOP>, dim3(grid_for(blocks, 1)), dim3(threads), 0, s, a);
+  } else if (defer) {
+    defer->mergeable = false;  // the one-wave-per-seed forms have no merged launch
+    return SHMT_OK;
   } else if (k <= kWideMaxPicks) {
     hipLaunchKernelGGL((pick_wide_kernel<true, HOP>), dim3(grid_for(S, 1, 256 * 32)), dim3(kWave),
                        static_cast<size_t>(k) * sizeof(int64_t), s, a);
@@ -631,12 +691,43 @@ static int pick_launch(const PickArgs &a, hipStream_t s) {
   return SHMT_OK;
 }
 
+namespace shmt {
+
+int launch_merged_sampling_stage(int n_jobs, const Stage *const *stages, hipStream_t s) {
+  const int kind = stages[0]->kind;
+  const unsigned threads = stages[0]->threads;
+  if (kind == kStagePickNarrowHop) {
+    Jobs<PickArgs> j;
+    const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+    hipLaunchKernelGGL(pick_narrow_hop_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
+  } else if (kind >= kStagePlanSingle && kind < kStagePlanTile + 3) {
+    Jobs<PlanArgs> j;
+    const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+    const dim3 grid(blocks, n_jobs), block(threads);
+    switch (kind) {
+      case kStagePlanSingle + 0: hipLaunchKernelGGL(plan_single_jobs<0>, grid, block, 0, s, j); break;
+      case kStagePlanSingle + 1: hipLaunchKernelGGL(plan_single_jobs<1>, grid, block, 0, s, j); break;
+      case kStagePlanSingle + 2: hipLaunchKernelGGL(plan_single_jobs<2>, grid, block, 0, s, j); break;
+      case kStagePlanTile + 0: hipLaunchKernelGGL(plan_tile_jobs<0>, grid, block, 0, s, j); break;
+      case kStagePlanTile + 1: hipLaunchKernelGGL(plan_tile_jobs<1>, grid, block, 0, s, j); break;
+      default: hipLaunchKernelGGL(plan_tile_jobs<2>, grid, block, 0, s, j); break;
+    }
+  } else {
+    set_error("internal: stage kind %d has no merged sampling launch", kind);
+    return SHMT_EINVAL;
+  }
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
+}  // namespace shmt
+
 extern "C" {
 
 static int pick_impl(const void *indices, const void *cache_indices, int idx_bytes,
                      const void *seeds, int seed_bytes, int64_t S, int64_t k, int replace,
                      const void *sub_indptr, int ptr_bytes, const void *plan, void *sub_indices,
-                     uint64_t rng_seed, uint32_t rng_stream, void *stream, const PickHopExtras *hop) {
+                     uint64_t rng_seed, uint32_t rng_stream, Launcher launcher, const PickHopExtras *hop) {
   SHMT_REQUIRE(S >= 0 && k >= 0, "shmt_sample_pick: S and num_picks must be >= 0");
   SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes),
                "shmt_sample_pick: ID can only be int32 or int64");
@@ -677,8 +768,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.clear_n = 0;
   a.wide_mark = nullptr;
   a.wide_nonce = 0;
-  hipStream_t s = as_stream(stream);
-  if (!hop) return pick_launch<false>(a, s);
+  if (!hop) return pick_launch<false>(a, launcher);
   a.sub_indptr_rw = hop->sub_indptr_rw;
   a.tile_prefix = hop->tile_prefix;
   a.raw_tiles = hop->raw_tiles;
@@ -692,7 +782,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.clear_n = hop->clear_n;
   a.wide_mark = hop->wide_mark;
   a.wide_nonce = hop->wide_nonce;
-  return pick_launch<true>(a, s);
+  return pick_launch<true>(a, launcher);
 }
 
 int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_bytes,
@@ -700,7 +790,7 @@ int shmt_sample_pick(const void *indices, const void *cache_indices, int idx_byt
                      const void *sub_indptr, int ptr_bytes, const void *plan, void *sub_indices,
                      uint64_t rng_seed, uint32_t rng_stream, void *stream) {
   return pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr,
-                   ptr_bytes, plan, sub_indices, rng_seed, rng_stream, stream, nullptr);
+                   ptr_bytes, plan, sub_indices, rng_seed, rng_stream, Launcher{as_stream(stream), nullptr}, nullptr);
 }
 
 int shmt_sample(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
@@ -712,14 +802,15 @@ int shmt_sample(const void *indptr, int ptr_bytes, const void *indices, int idx_
   // the fused-hop forms of the kernels without their relabel extras: the pick kernel adds the tile
   // offsets and publishes the total, so plan + pick are two launches whatever the number of seeds
   PlanHopExtras plan_hop{nullptr, 8, nullptr, nullptr, nullptr, 0};
+  const Launcher launcher{as_stream(stream), nullptr};
   int rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
-                     plan_bytes, nnz_out, stream, &plan_hop);
+                     plan_bytes, nnz_out, launcher, &plan_hop);
   if (rc) return rc;
   const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, plan_hop.raw_tiles_out, nnz_out,
                                const_cast<uint64_t *>(plan_hop.total_out), nullptr, nullptr, nullptr, 8,
                                nullptr, 0, nullptr, 0};
   return pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
-                   plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
+                   plan, sub_indices, rng_seed, rng_stream, launcher, &pick_hop);
 }
 
 static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
@@ -729,7 +820,7 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
                     void *sub_indptr,
                     void *sub_indices, void *plan, int64_t plan_bytes, int elem_bytes, void *total_out,
                     void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
-                    int64_t *nnz_out, int64_t *count_out, int64_t *count_copy, void *stream) {
+                    int64_t *nnz_out, int64_t *count_out, int64_t *count_copy, Launcher launcher) {
   SHMT_REQUIRE(S >= 1 && k >= 1, "shmt_sample_hop: S and num_picks must be >= 1");
   SHMT_REQUIRE(k <= ((1ll << 31) - 1 - S) / S, "shmt_sample_hop: S * (num_picks + 1) must be < 2^31");
   SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes) && width_ok(elem_bytes),
@@ -744,19 +835,18 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
   if (rc) return rc;
   PlanHopExtras plan_hop{total_out, elem_bytes, S_len, nullptr, nullptr, 0};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
-                 plan_bytes, nnz_out, stream, &plan_hop);
+                 plan_bytes, nnz_out, launcher, &plan_hop);
   if (rc) return rc;
   const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, plan_hop.raw_tiles_out, nnz_out,
                                const_cast<uint64_t *>(plan_hop.total_out), S_len, rng_seed_dev, total_out, elem_bytes,
                                static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
-                 plan, sub_indices, rng_seed, rng_stream, stream, &pick_hop);
+                 plan, sub_indices, rng_seed, rng_stream, launcher, &pick_hop);
   if (rc) return rc;
   // [seeds, sub_indices] is in total_out and the table is empty: the relabel passes follow, with the
   // number of sampled ids (and of seeds, when it is a device-side figure) read from device memory
   return launch_relabel_passes(total_out, n_max, S, S_len, plan_hop.total_out, 8, elem_bytes, scratch,
-                               scratch_bytes, unique_out, labels_out, count_out, count_copy, table,
-                               as_stream(stream));
+                               scratch_bytes, unique_out, labels_out, count_out, count_copy, table, launcher);
 }
 
 int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
@@ -769,7 +859,7 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
   return hop_impl(indptr, ptr_bytes, indices, idx_bytes, cache_indptr, cache_indices, map, seeds, seed_bytes,
                   S, nullptr, k, replace, rng_seed, nullptr, rng_stream, sub_indptr, sub_indices, plan, plan_bytes,
                   elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out, count_out,
-                  nullptr, stream);
+                  nullptr, Launcher{as_stream(stream), nullptr});
 }
 
 int shmt_sample_hop_chained(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
@@ -785,7 +875,49 @@ int shmt_sample_hop_chained(const void *indptr, int ptr_bytes, const void *indic
                   max_seeds, seeds_len, k, replace, rng_seed, rng_seed_dev, rng_stream, sub_indptr, sub_indices,
                   plan,
                   plan_bytes, elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out,
-                  count_out, count_dev_out, stream);
+                  count_out, count_dev_out, Launcher{as_stream(stream), nullptr});
+}
+
+static int hop_job(const shmt_hop_job &j, Launcher launcher) {
+  return hop_impl(j.indptr, j.ptr_bytes, j.indices, j.idx_bytes, j.cache_indptr, j.cache_indices, j.map, j.seeds,
+                  j.seed_bytes, j.max_seeds, j.seeds_len, j.k, j.replace, j.rng_seed, j.rng_seed_dev, j.rng_stream,
+                  j.sub_indptr, j.sub_indices, j.plan, j.plan_bytes, j.elem_bytes, j.total_out, j.scratch,
+                  j.scratch_bytes, j.unique_out, j.labels_out, j.nnz_out, j.count_out, j.count_dev_out, launcher);
+}
+
+int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream) {
+  SHMT_REQUIRE(n_jobs >= 0, "shmt_sample_hops_chained: n_jobs must be >= 0");
+  SHMT_REQUIRE(n_jobs == 0 || jobs != nullptr, "shmt_sample_hops_chained: jobs is null");
+  hipStream_t s = as_stream(stream);
+  for (int first = 0; first < n_jobs; first += kMaxJobs) {
+    const int n = n_jobs - first < kMaxJobs ? n_jobs - first : kMaxJobs;
+    // record every job's launches; merge them when all jobs run the same kernels stage by stage
+    StageList lists[kMaxJobs];
+    bool merge = n > 1;
+    for (int j = 0; j < n && merge; ++j) {
+      const int rc = hop_job(jobs[first + j], Launcher{s, &lists[j]});
+      if (rc) return rc;
+      merge = lists[j].mergeable && lists[j].n == lists[0].n;
+      for (int i = 0; merge && i < lists[j].n; ++i)
+        merge = lists[j].stage[i].kind == lists[0].stage[i].kind &&
+                lists[j].stage[i].threads == lists[0].stage[i].threads;
+    }
+    if (!merge) {
+      for (int j = 0; j < n; ++j) {
+        const int rc = hop_job(jobs[first + j], Launcher{s, nullptr});
+        if (rc) return rc;
+      }
+      continue;
+    }
+    for (int i = 0; i < lists[0].n; ++i) {
+      const Stage *stages[kMaxJobs];
+      for (int j = 0; j < n; ++j) stages[j] = &lists[j].stage[i];
+      const int rc = stages[0]->kind >= kStageRlSmall ? launch_merged_relabel_stage(n, stages, s)
+                                                      : launch_merged_sampling_stage(n, stages, s);
+      if (rc) return rc;
+    }
+  }
+  return SHMT_OK;
 }
 
 int shmt_subcsr_plan(const void *indptr, int ptr_bytes, const void *seeds, int seed_bytes,

@@ -561,3 +561,81 @@ def test_c_abi_sample_in_two_launches_matches_plan_then_pick(cabi, S, k, replace
     assert torch.equal(a["sp"], b["sp"]) and torch.equal(a["si"][:nnz], b["si"][:nnz])
     assert lib.shmt_sample(indptr.data_ptr(), 8, indices.data_ptr(), 4, None, None, None, seeds.data_ptr(), 8, 0, k,
                            replace, 11, 3, None, None, None, 0, None, stream) == -1
+
+
+@pytest.mark.parametrize("cached", [False, True])
+@pytest.mark.parametrize("sizes,picks", [([300, 300, 300], (4, 5)), ([1000, 1000, 1000, 1000, 1000], (6, 3, 2)),
+                                         ([100, 1000, 200], (3, 3)), ([50] * 11, (8, 2)), ([40, 40], (70, 2))])
+def test_c_abi_merged_jobs_equal_separate_chained_hops(cabi, cached, sizes, picks):
+    """shmt_sample_hops_chained: the same hop of several batches in one call (launches merged when
+    the jobs run the same kernels, issued one by one otherwise: unequal sizes, more than 8 jobs, a
+    fan-out without merged form) gives what one shmt_sample_hop_chained call per batch gives."""
+    lib = cabi.load()
+    indptr, indices = _graph(scale=13, ptr_dt=torch.int64, idx_dt=torch.int32)
+    indptr, indices = indptr.cuda(), indices.cuda()
+    n = indptr.numel() - 1
+    stream = cabi.current_stream()
+    gp = gi = hnd = None
+    keep = []
+    if cached:
+        hot = torch.randperm(n, generator=torch.Generator().manual_seed(2))[: n // 2].cuda()
+        deg = indptr[hot + 1] - indptr[hot]
+        gp = torch.cat([torch.zeros(1, dtype=torch.int64).cuda(), torch.cumsum(deg, 0)])
+        gi = torch.cat([indices[indptr[v]:indptr[v + 1]] for v in hot.tolist()])
+        nbytes = lib.shmt_hashmap_table_bytes(hot.numel(), 0.8, 8, 8)
+        keep.append(torch.empty(nbytes, dtype=torch.uint8).cuda())
+        hnd = ctypes.c_void_p()
+        cabi.check(lib.shmt_hashmap_create(ctypes.byref(hnd), hot.data_ptr(), torch.arange(hot.numel()).cuda().data_ptr(),
+                                           hot.numel(), 8, 8, 0.8, keep[0].data_ptr(), nbytes, stream))
+    g = torch.Generator().manual_seed(len(sizes))
+    seed_sets = [torch.randperm(n, generator=g)[:s].cuda() for s in sizes]
+
+    def buffers(s_max, k):
+        n_max = s_max + s_max * k
+        return dict(s_max=s_max, k=k, sp=torch.full((s_max + 1,), -1, dtype=torch.int64).cuda(),
+                    si=torch.empty(s_max * k, dtype=torch.int32).cuda(),
+                    plan=torch.empty(lib.shmt_sample_plan_bytes(s_max), dtype=torch.uint8).cuda(),
+                    total=torch.empty(n_max, dtype=torch.int64).cuda(), unique=torch.empty(n_max, dtype=torch.int64).cuda(),
+                    labels=torch.empty(n_max, dtype=torch.int64).cuda(),
+                    scratch=torch.empty(lib.shmt_relabel_scratch_bytes(n_max), dtype=torch.uint8).cuda(),
+                    nnz=torch.full((1,), -1, dtype=torch.int64).cuda(), count=torch.full((1,), -1, dtype=torch.int64).cuda(),
+                    count_dev=torch.full((1,), -1, dtype=torch.int64).cuda())
+
+    def job(b, seeds_ptr, s_len, hop, rng):
+        return cabi.HopJob(indptr.data_ptr(), 8, indices.data_ptr(), 4, gp.data_ptr() if cached else None,
+                           gi.data_ptr() if cached else None, hnd, seeds_ptr, 8, b["s_max"], s_len, b["k"], 0, rng,
+                           None, hop, b["sp"].data_ptr(), b["si"].data_ptr(), b["plan"].data_ptr(), b["plan"].numel(), 8,
+                           b["total"].data_ptr(), b["scratch"].data_ptr(), b["scratch"].numel(), b["unique"].data_ptr(),
+                           b["labels"].data_ptr(), b["nnz"].data_ptr(), b["count"].data_ptr(), b["count_dev"].data_ptr())
+
+    def run(merged):
+        chains = [[] for _ in sizes]
+        src = [(s.data_ptr(), None, s.numel()) for s in seed_sets]
+        for hop, k in enumerate(picks):
+            jobs = []
+            for j, (ptr, s_len, s_max) in enumerate(src):
+                b = buffers(s_max, k)
+                chains[j].append(b)
+                jobs.append(job(b, ptr, s_len, hop, 90 + j))
+                src[j] = (b["unique"].data_ptr(), b["count_dev"].data_ptr(), s_max + s_max * k)
+            if merged:
+                cabi.check(lib.shmt_sample_hops_chained((cabi.HopJob * len(jobs))(*jobs), len(jobs), stream))
+            else:
+                for one in jobs:
+                    cabi.check(lib.shmt_sample_hops_chained(ctypes.byref(one), 1, stream))
+        torch.cuda.synchronize()
+        return chains
+
+    got, want = run(True), run(False)
+    for j in range(len(sizes)):
+        s_now = sizes[j]
+        for a, b in zip(got[j], want[j]):
+            nnz, u = int(b["nnz"].item()), int(b["count"].item())
+            assert (int(a["nnz"].item()), int(a["count"].item()), int(a["count_dev"].item())) == (nnz, u, u)
+            assert torch.equal(a["sp"][:s_now + 1], b["sp"][:s_now + 1]) and torch.equal(a["si"][:nnz], b["si"][:nnz])
+            assert torch.equal(a["unique"][:u], b["unique"][:u])
+            assert torch.equal(a["labels"][:s_now + nnz], b["labels"][:s_now + nnz])
+            s_now = u
+    assert lib.shmt_sample_hops_chained(None, 0, stream) == 0 and lib.shmt_sample_hops_chained(None, 2, stream) == -1
+    if hnd is not None:
+        lib.shmt_hashmap_destroy(hnd)
