@@ -953,10 +953,13 @@ std::vector<BatchResult> finish_together(const CsrArgs &g, std::vector<TogetherB
 
 // Multi-hop sampling of several independent seed batches. Every batch is a
 // chain of short, latency-bound kernels with a host read of the sizes at its end,
-// so one batch alone leaves most of the GPU idle. Here up to `max_in_flight`
-// batches advance at the same time: each is driven by its own host thread on
-// its own stream (default priority, the same streams every call), so both the
-// launches and the kernels of different batches overlap. Results are those of
+// so one batch alone leaves most of the GPU idle. Batches whose hops all chain
+// on the device advance in lockstep, `min(max_in_flight, 8)` at a time, and
+// share their kernel launches (issue_together). Otherwise (a hop too large to
+// chain, or features to fetch) up to `max_in_flight` batches advance at the
+// same time, each driven by its own host thread on its own stream (default
+// priority, the same streams every call), so that both the launches and the
+// kernels of different batches overlap. Results are those of
 // sample_hop called hop by hop, batch by batch (`seeds_rng[b]` is the RNG seed
 // of batch b, RNG stream = hop number; without seeds_rng every hop uses the
 // default seed and stream 0); they are ordered after the calling
