@@ -546,19 +546,15 @@ struct PendingHop {
 // then holds an unknown number of ids, at most seeds.numel(), and the kernels
 // read the true number there (the count_dev of the hop before, whose unique
 // buffer is `seeds`); every buffer is sized for the bound.
-// With `job` the fused hop is not queued: its launch parameters are written
-// there, for a caller that queues several hops together
-// (shmt_sample_hops_chained); the hop must then be a fused one.
 PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds_len, int64_t num_picks,
-                     bool replace, std::optional<int64_t> seed, int64_t stream_id,
-                     shmt_hop_job *job = nullptr) {
+                     bool replace, std::optional<int64_t> seed, int64_t stream_id) {
   PendingHop h;
   seeds = cuda_ids(seeds, "seeds");
   TORCH_CHECK(num_picks >= 0, "num_picks must be >= 0");
   const int64_t S = seeds.numel();
   const bool fused = S > 0 && num_picks > 0 && num_picks <= kEagerOutputLimit / S;
   if (!fused) {  // degenerate or very large bound: the two operators one after the other
-    TORCH_CHECK(seeds_len == nullptr && job == nullptr, "internal: a chained hop must be a fused one");
+    TORCH_CHECK(seeds_len == nullptr, "internal: a chained hop must be a fused one");
     auto sampled = sample_impl(g.indptr, g.indices, g.cached() ? &*g.gpu_indptr : nullptr,
                                g.cached() ? &*g.gpu_indices : nullptr, g.hashmap, seeds, num_picks,
                                replace, seed, stream_id);
@@ -634,10 +630,7 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds
   j.nnz_out = h.nnz_slot.dev;
   j.count_out = h.count_slot.dev;
   j.count_dev_out = h.count_dev;
-  if (job)
-    *job = j;
-  else
-    check(shmt_sample_hops_chained(&j, 1, stream));
+  check(shmt_sample_hops_chained(&j, 1, stream));
   return h;
 }
 
