@@ -639,3 +639,25 @@ def test_c_abi_merged_jobs_equal_separate_chained_hops(cabi, cached, sizes, pick
     assert lib.shmt_sample_hops_chained(None, 0, stream) == 0 and lib.shmt_sample_hops_chained(None, 2, stream) == -1
     if hnd is not None:
         lib.shmt_hashmap_destroy(hnd)
+
+
+@pytest.mark.parametrize("picks", [[10, 10, 30], [5, 0, 3], [40, 40], [3, 3, 3, 70]])
+@pytest.mark.parametrize("in_flight", [1, 4])
+def test_sample_blocks_with_hops_too_large_to_chain(capi, picks, in_flight):
+    """Fan-outs whose bounds outgrow what a chained hop may allocate (the sizes are then read before
+    that hop), a hop without picks in the middle, and a fan-out above 64 at the end: same results
+    as one sample_hop call per hop and batch."""
+    indptr, indices = _graph(scale=14)
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(17)
+    sizes = [1000, 1000, 999, 1, 1000, 0, 1000]
+    batches = [torch.randperm(n, generator=g)[:s].cuda() for s in sizes]
+    rng = [7 + b for b in range(len(batches))]
+    got = capi.sample_blocks(indptr, indices, None, None, None, batches, picks, False, seeds_rng=rng,
+                             max_in_flight=in_flight)
+    for b, seeds in enumerate(batches):
+        assert len(got[b]) == len(picks)
+        for hop, k in enumerate(picks):
+            want = capi.sample_hop(indptr, indices, None, None, None, seeds, k, False, seed=rng[b], stream_id=hop)
+            _same(got[b][hop], want)
+            seeds = want[2]
