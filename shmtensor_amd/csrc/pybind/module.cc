@@ -75,6 +75,7 @@ void *device_address(const torch::Tensor &t, const char *name) {
 // to a stream synchronisation, which surfaces the error.
 class Readback {
  public:
+  static constexpr int kSlots = 4096;  // a ring: more than all operators together keep pending at once
   struct Slot {
     volatile int64_t *host;
     int64_t *dev;
@@ -112,7 +113,6 @@ class Readback {
   }
 
  private:
-  static constexpr int kSlots = 256;  // more than any operator keeps pending at once
   static constexpr int64_t kPending = INT64_MIN;
   static constexpr int kSpinBudgetMs = 200;
   std::mutex mutex_;  // operators may run on several host threads (sample_blocks)
@@ -985,7 +985,9 @@ std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch
     for (int64_t b = 0; b < B; ++b) any = any || chains_entirely(seeds[b].numel(), num_picks);
     if (any) {
       py::gil_scoped_release no_gil;
-      const size_t group_size = static_cast<size_t>(std::min<int64_t>(K, 8));
+      // (two groups are queued at a time, each holding two size slots per hop and batch)
+      const int64_t by_slots = Readback::kSlots / 8 / static_cast<int64_t>(std::max<size_t>(num_picks.size(), 1));
+      const size_t group_size = static_cast<size_t>(std::max<int64_t>(1, std::min<int64_t>({K, 8, by_slots})));
       std::vector<int64_t> group;
       // one group is queued ahead of the one whose sizes are being read, so the GPU never waits
       // for the host's bookkeeping
