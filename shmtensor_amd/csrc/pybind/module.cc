@@ -975,7 +975,15 @@ std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch
   const int64_t K = std::min<int64_t>({max_in_flight, kMaxBatchesInFlight, B});
   if (K <= 1) {
     py::gil_scoped_release no_gil;  // lets a Python thread that prefetches batches run beside the caller
-    for (int64_t b = 0; b < B; ++b) out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b), features);
+    for (int64_t b = 0; b < B; ++b) {
+      if (!features && chains_entirely(seeds[b].numel(), num_picks)) {
+        // all bounds known up front: two allocations and one set of result tensors for the batch
+        std::vector<TogetherBatch> one = issue_together(g, {seeds[b]}, num_picks, replace, {rng_of(b)});
+        out[b] = std::move(finish_together(g, one)[0]);
+      } else {
+        out[b] = run_hops(g, seeds[b], num_picks, replace, rng_of(b), features);
+      }
+    }
     return out;
   }
   if (!features) {
