@@ -26,7 +26,7 @@ HIP_SOURCES = ["hashmap.hip", "fetch.hip", "scan.hip", "relabel.hip", "sample.hi
 # Packed-FP32 instruction selection is switched off for every HIP translation
 # unit (the kernels here do no floating-point arithmetic at all, rows are
 # moved as raw bytes).
-HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
+HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument"]
 
@@ -47,9 +47,20 @@ def hipcc():
 
 
 def build_lib():
+    """One object per translation unit (compiled side by side), then one link."""
+    from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    _run([hipcc()] + HIPCC_FLAGS + ["-I" + INCLUDE, "-I" + CSRC] + srcs + ["-o", LIB_PATH])
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    objs = [os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in HIP_SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        _run([hipcc()] + HIPCC_FLAGS + ["-I" + INCLUDE, "-I" + CSRC, "-c", os.path.join(CSRC, src), "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=min(8, len(objs))) as pool:
+        list(pool.map(compile_one, zip(HIP_SOURCES, objs)))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB_PATH])
     return LIB_PATH
 
 
