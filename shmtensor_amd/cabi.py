@@ -33,6 +33,7 @@ SIGNATURES = {
     "shmt_scan_tmp_bytes": (_i64, [_i64]),
     "shmt_exclusive_scan": (_int, [_vp, _i64, _int, _vp, _i64, _vp]),
     "shmt_inclusive_scan_i32": (_int, [_vp, _i64, _vp, _i64, _vp]),
+    "shmt_exclusive_scan_noalloc": (_int, [_vp, _i64, _int, _vp]),
     "shmt_relabel_scratch_bytes": (_i64, [_i64]),
     "shmt_relabel": (_int, [_vp, _i64, _int, _vp, _i64, _vp, _vp, _vp, _vp]),
     "shmt_relabel_segments": (_int, [_c.POINTER(_vp), _c.POINTER(_i64), _c.POINTER(_int), _int, _vp, _int, _int,

@@ -8,6 +8,8 @@
 // scanned by one 1024-thread workgroup that walks the array with a running
 // carry (one launch); larger inputs use reduce -> scan-of-partials -> apply,
 // three launches with no inter-workgroup waiting.
+#include <mutex>
+
 #include "common.h"
 #include "launchers.h"
 #include "scan_dev.h"
@@ -100,6 +102,36 @@ static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, hipS
   return SHMT_OK;
 }
 
+// ---- scan without a caller-provided workspace -------------------------------
+// The tile partials of shmt_exclusive_scan_noalloc live in this array, which
+// is part of the loaded code object: every GPU the library runs on holds its
+// own copy, at its own address, until the process ends. The name below is a
+// host-side handle only; kernels are given the device address that
+// hipGetSymbolAddress returns for the current device.
+constexpr int64_t kStaticScanPartials = 1 << 17;                       // 1 MiB
+constexpr int64_t kStaticScanMaxLen = kStaticScanPartials * kScanTile;  // 268,435,456 elements
+static __device__ __align__(256) uint64_t scratch[kStaticScanPartials];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static uint64_t *g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device ordinal
+
+// Device address of this GPU's copy of `scratch` (looked up once per device).
+static int static_scan_scratch(uint64_t **out) {
+  int dev = -1;
+  SHMT_HIP(hipGetDevice(&dev));
+  SHMT_REQUIRE(dev >= 0 && dev < kMaxDevices, "shmt_exclusive_scan_noalloc: device ordinal %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    SHMT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SHMT_REQUIRE(p != nullptr, "shmt_exclusive_scan_noalloc: no device address for the static workspace");
+    g_scratch_ptr[dev] = static_cast<uint64_t *>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return SHMT_OK;
+}
+
 }  // namespace shmt
 
 using namespace shmt;
@@ -121,6 +153,29 @@ int shmt_exclusive_scan(void *data, int64_t len, int elem_bytes, void *tmp, int6
     return scan_inplace<uint64_t, false>(static_cast<uint64_t *>(data), len, tmp, tmp_bytes,
                                          as_stream(stream));
   return scan_inplace<uint32_t, false>(static_cast<uint32_t *>(data), len, tmp, tmp_bytes,
+                                       as_stream(stream));
+}
+
+int shmt_exclusive_scan_noalloc(void *data, int64_t len, int elem_bytes, void *stream) {
+  SHMT_REQUIRE(len >= 0, "shmt_exclusive_scan_noalloc: len must be >= 0");
+  SHMT_REQUIRE(width_ok(elem_bytes), "shmt_exclusive_scan_noalloc: ID can only be int32 or int64");
+  SHMT_REQUIRE(len <= kStaticScanMaxLen,
+               "shmt_exclusive_scan_noalloc: len %lld exceeds the static workspace (at most %lld elements); "
+               "use shmt_exclusive_scan with a caller-provided workspace",
+               static_cast<long long>(len), static_cast<long long>(kStaticScanMaxLen));
+  SHMT_REQUIRE(len == 0 || data != nullptr, "shmt_exclusive_scan_noalloc: data is null");
+  // also for len == 0, so that an empty call can serve as the set-up call
+  uint64_t *partials = nullptr;
+  int rc = static_scan_scratch(&partials);
+  if (rc) return rc;
+  if (len == 0) return SHMT_OK;
+  // Every partial a launch reads was written by the reduce kernel of the same
+  // call, so nothing in the workspace needs clearing between calls.
+  const int64_t tmp_bytes = kStaticScanPartials * static_cast<int64_t>(sizeof(uint64_t));
+  if (elem_bytes == 8)
+    return scan_inplace<uint64_t, false>(static_cast<uint64_t *>(data), len, partials, tmp_bytes,
+                                         as_stream(stream));
+  return scan_inplace<uint32_t, false>(static_cast<uint32_t *>(data), len, partials, tmp_bytes,
                                        as_stream(stream));
 }
 
