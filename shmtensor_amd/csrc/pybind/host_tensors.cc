@@ -23,9 +23,20 @@ namespace py = pybind11;
 
 namespace {
 
-void pin_range(void *ptr, int64_t size, const char *what) {
-  TORCH_CHECK(shmt_host_register(ptr, size) == SHMT_OK, what, ": cannot pin the mapping (",
-              shmt_last_error(), ")");
+// Registers a fresh mapping for GPU access. Some drivers refuse to register
+// memory that already exists; the mapping is then taken down again (and the
+// segment this call created removed) before the error is raised, so a refused
+// request leaves nothing behind.
+void pin_range(void *ptr, int64_t size, int fd, const char *what, const char *unlink_name) {
+  if (shmt_host_register(ptr, size) == SHMT_OK) return;
+  const std::string why = shmt_last_error();
+  munmap(ptr, static_cast<size_t>(size));
+  close(fd);
+  if (unlink_name != nullptr) shm_unlink(unlink_name);
+  TORCH_CHECK(false, what, "(pin_memory=True): this driver does not register an existing mapping for GPU access (",
+              why, "). Open it with pin_memory=False and hand the GPU operators a staging copy in pinned "
+              "memory instead: `staged = obj.pinned()` on a ShmTensor / DiskTensor (`obj.flush()` copies it "
+              "back into the mapping), or `tensor.pin_memory()` on the plain tensor.");
 }
 
 void *map_fd(int fd, int64_t size, const std::string &name) {
@@ -51,7 +62,7 @@ std::tuple<int64_t, int64_t> create_shared_mem(const std::string &name, int64_t 
     TORCH_CHECK(false, "Failed to truncate the file. ", strerror(err));
   }
   void *ptr = map_fd(fd, size, name);
-  if (pin_memory) pin_range(ptr, size, "create_shared_mem");
+  if (pin_memory) pin_range(ptr, size, fd, "create_shared_mem", name.c_str());
   return std::make_tuple(reinterpret_cast<int64_t>(ptr), static_cast<int64_t>(fd));
 }
 
@@ -62,7 +73,7 @@ std::tuple<int64_t, int64_t> open_shared_mem(const std::string &name, int64_t si
   const int fd = shm_open(name.c_str(), O_RDWR, S_IRUSR | S_IWUSR);
   TORCH_CHECK(fd != -1, "fail to open ", name, ": ", strerror(errno));
   void *ptr = map_fd(fd, size, name);
-  if (pin_memory) pin_range(ptr, size, "open_shared_mem");
+  if (pin_memory) pin_range(ptr, size, fd, "open_shared_mem", nullptr);
   return std::make_tuple(reinterpret_cast<int64_t>(ptr), static_cast<int64_t>(fd));
 }
 
@@ -189,10 +200,10 @@ std::tuple<torch::Tensor, int64_t, int64_t, int64_t> open_mmap_tensor(const std:
     TORCH_CHECK(false, fname, ": file is shorter than its header says");
   }
   void *ptr = map_fd(fd, file_size, fname);
+  // the whole file is registered, the tensor starts at ptr + offset (src/mmap_tensor.cc:39-45)
+  if (pin_memory) pin_range(ptr, file_size, fd, "open_mmap_tensor", nullptr);
   torch::Tensor tensor = torch::from_blob(static_cast<char *>(ptr) + h.offset, h.shape,
                                           torch::TensorOptions().dtype(h.dtype));
-  // the whole file is registered, the tensor starts at ptr + offset (src/mmap_tensor.cc:39-45)
-  if (pin_memory) pin_range(ptr, file_size, "open_mmap_tensor");
   return std::make_tuple(tensor, file_size, reinterpret_cast<int64_t>(ptr), static_cast<int64_t>(fd));
 }
 

@@ -11,6 +11,8 @@
 #include <torch/extension.h>
 
 #include <atomic>
+#include <cstdlib>
+#include <cstring>
 #include <chrono>
 #include <cstdint>
 #include <deque>
@@ -89,7 +91,8 @@ class Readback {
       check(shmt_host_devptr(host_.data_ptr(), &d));
       dev_ = static_cast<int64_t *>(d);
     }
-    const int i = next_++ % kSlots;
+    const uint32_t i = next_;
+    next_ = (next_ + 1) % kSlots;  // stays in [0, kSlots): nothing counts up without bound
     Slot s{host_.data_ptr<int64_t>() + i, dev_ + i};
     *s.host = kPending;
     std::atomic_thread_fence(std::memory_order_seq_cst);
@@ -118,7 +121,7 @@ class Readback {
   std::mutex mutex_;  // operators may run on several host threads (sample_blocks)
   torch::Tensor host_;
   int64_t *dev_ = nullptr;
-  int next_ = 0;
+  uint32_t next_ = 0;
 };
 
 Readback &readback() {
@@ -184,24 +187,65 @@ class StaticHashmap {
 std::mutex g_pin_mutex;
 std::unordered_map<void *, int64_t> g_registered;  // ranges registered in place by pin_memory
 
-// PinMemory, src/cache_feature_fetch.cu:6-9. Registers the tensor's memory in
-// place. Where the driver refuses to register existing memory, the tensor is
-// re-homed instead: its contents move into freshly allocated pinned memory
-// and the same Python tensor object now views that memory.
+// Registering memory that already exists (hipHostRegister) is refused by some
+// drivers, and a refused call can leave its error for the next HIP call to
+// report. It is therefore only tried on request: set_host_register(true) or
+// SHMT_HOST_REGISTER=1 in the environment.
+std::atomic<int> g_host_register{-1};  // -1: not decided yet (read the environment)
+
+bool host_register_enabled() {
+  int v = g_host_register.load();
+  if (v < 0) {
+    const char *e = std::getenv("SHMT_HOST_REGISTER");
+    v = (e != nullptr && e[0] != '\0' && e[0] != '0') ? 1 : 0;
+    g_host_register.store(v);
+  }
+  return v == 1;
+}
+
+void set_host_register(bool on) { g_host_register.store(on ? 1 : 0); }
+
+// PinMemory, src/cache_feature_fetch.cu:6-9: make a CPU tensor's memory
+// addressable by kernels. With in-place registration enabled (see above) the
+// memory is registered where it lies, as in the reference. Otherwise the
+// tensor's STORAGE is re-homed: its bytes move into newly allocated pinned
+// memory and the storage object points there afterwards, so the tensor and
+// every other torch tensor that shares the storage (views, slices, aliases)
+// keep seeing one memory, and later GPU writes (uva_set) reach all of them.
+// What cannot follow is memory that torch does not own: a storage that wraps
+// a numpy array, a shared-memory or file mapping. Re-homing such a storage
+// cuts the tie to that memory, which is reported with a warning.
 void pin_memory(torch::Tensor &data) {
   TORCH_CHECK(!data.is_cuda(), "data must be a CPU tensor");
   if (data.numel() == 0) return;
   TORCH_CHECK(data.is_contiguous(), "data must be contiguous");
   void *dev = nullptr;
   if (shmt_host_devptr(data.data_ptr(), &dev) == SHMT_OK) return;  // already addressable
-  if (shmt_host_register(data.data_ptr(), static_cast<int64_t>(data.nbytes())) == SHMT_OK) {
+  if (host_register_enabled() &&
+      shmt_host_register(data.data_ptr(), static_cast<int64_t>(data.nbytes())) == SHMT_OK) {
     std::lock_guard<std::mutex> lock(g_pin_mutex);
     g_registered[data.data_ptr()] = static_cast<int64_t>(data.nbytes());
     return;
   }
-  torch::Tensor pinned = torch::empty_like(data, data.options().pinned_memory(true));
-  pinned.copy_(data);
-  data.set_data(pinned);
+  c10::Storage storage = data.storage();
+  const size_t nbytes = storage.nbytes();
+  TORCH_CHECK(nbytes > 0 && storage.data() != nullptr, "pin_memory: tensor has no memory");
+  if (!storage.resizable()) {
+    // storages that wrap foreign memory (from_numpy, from_blob) are the non-resizable ones
+    if (PyErr_WarnEx(PyExc_UserWarning,
+                     "pin_memory: the tensor's memory is not owned by torch (a numpy array, a shared-memory or "
+                     "file mapping) and existing memory is not registered in place with the current setting, so "
+                     "its contents were copied into new pinned memory: the tensor now lives there and no longer "
+                     "aliases the original buffer (GPU writes will not reach it). Allocate the data pinned in "
+                     "the first place, or enable in-place registration with set_host_register(True).",
+                     1) < 0)
+      throw py::error_already_set();
+  }
+  at::Allocator *pinned = at::globalContext().getPinnedMemoryAllocator(c10::kCUDA);
+  at::DataPtr fresh = pinned->allocate(nbytes);
+  std::memcpy(fresh.get(), storage.data(), nbytes);
+  // the old memory is released here (or, for foreign memory, handed back to its owner)
+  storage.set_data_ptr_noswap(std::move(fresh));
 }
 
 // UnpinMemory, src/cache_feature_fetch.cu:11-13.
@@ -1512,6 +1556,10 @@ PYBIND11_MODULE(ShmTensorLib, m) {
 
   m.def("thrust_scan", &thrust_scan, py::arg("tensor"));
 
+  m.def("set_host_register", &set_host_register, py::arg("enabled"),
+        "Let pin_memory() try to register existing memory in place (hipHostRegister) before it falls "
+        "back to re-homing the tensor's storage in new pinned memory. Off by default; also switched on "
+        "by SHMT_HOST_REGISTER=1 in the environment.");
   m.def("pin_memory", &pin_memory, py::arg("data"))
       .def("unpin_memory", &unpin_memory, py::arg("data"))
       .def("uva_fetch", &uva_fetch, py::arg("data"), py::arg("indices"))

@@ -60,10 +60,16 @@ class GPUSamplingDataloader:
         self.use_ddp = use_ddp
         self.shuffle = shuffle
         self.drop_last = drop_last
-        # None: every call uses the fixed default seed, as the reference does
-        # (src/cache_graph_sampling.cu:204,407); an int: batch b, hop h draw from
-        # (rng_seed + b, stream h), so epochs and batches differ reproducibly.
+        # A sample here is a pure function of (RNG seed, RNG stream, node id, fanout,
+        # degree); it does not depend on the node's position in the batch (the reference's
+        # draws do: curand_init(7777 + lane, thread id), src/cache_graph_sampling.cu:107,204,
+        # so re-batched or shuffled seeds see other samples there even with its fixed seed).
+        # The loader therefore gives every batch its own seed and every hop its own stream:
+        # batch number b (counted over all epochs) draws from (rng_seed + b, stream = hop).
+        # rng_seed=None takes the base from torch's global seed (torch.initial_seed() when the
+        # loader is built), so torch.manual_seed() makes a run repeatable and unseeded runs differ.
         self.rng_seed = rng_seed
+        self._rng_base = (int(rng_seed) if rng_seed is not None else int(torch.initial_seed())) & ((1 << 62) - 1)
         self._batches_drawn = 0
         # prefetch > 1: that many consecutive batches are sampled together, their
         # kernels overlapping on separate streams (same batches, same order, same
@@ -148,9 +154,7 @@ class GPUSamplingDataloader:
     # ---- one hop / one batch ---------------------------------------------------
 
     def _sample(self, seeds, num_pick, hop, use_cache=True):
-        extra = {}
-        if self.rng_seed is not None:
-            extra = {"seed": int(self.rng_seed) + self._batches_drawn, "stream_id": hop}
+        extra = {"seed": self._rng_base + self._batches_drawn, "stream_id": hop}
         if use_cache and self.has_cache:
             return capi.csr_cache_sampling(self.indptr, self.indices, self.gpu_indptr, self.gpu_indices,
                                            self.hashmap, seeds, num_pick, self.replace, **extra)
@@ -161,9 +165,7 @@ class GPUSamplingDataloader:
         (input_nodes, output_nodes, blocks) per batch."""
         groups = [self.seeds[b * self.batchsize:(b + 1) * self.batchsize]
                   for b in range(first_batch, first_batch + count)]
-        rng = None
-        if self.rng_seed is not None:
-            rng = [int(self.rng_seed) + batches_drawn + j for j in range(count)]
+        rng = [self._rng_base + batches_drawn + j for j in range(count)]
         cached = self.has_cache
         graph = (self.indptr, self.indices, self.gpu_indptr if cached else None,
                  self.gpu_indices if cached else None, self.hashmap if cached else None)
