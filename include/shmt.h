@@ -36,7 +36,7 @@ extern "C" {
 #define SHMT_ENOTPINNED (-3) /* host pointer is not device-accessible        */
 #define SHMT_ENOMEM (-4)  /* caller-provided buffer too small                */
 
-#define SHMT_ABI_VERSION 1
+#define SHMT_ABI_VERSION 2
 
 /* Library identification / error channel (no counterpart in the reference,
  * whose errors are c10 exceptions or exit(): include/common.h:10-27). */
@@ -368,6 +368,14 @@ typedef struct shmt_hop_job {
   int64_t *nnz_out;
   int64_t *count_out;
   int64_t *count_dev_out;
+  /* Coordinate form of the hop's block (create_block_from_coo,
+   * python/shmtensor/sampling.py:21-27): when coo_dst is not NULL the pick kernel
+   * also writes, for every sampled id, the position of the seed it was sampled
+   * for (the destination node of that edge; the source is its label in
+   * labels_out), coo_bytes in {4,8} wide, S * k entries of room. NULL: not
+   * produced.                                                               */
+  void *coo_dst;
+  int coo_bytes;
 } shmt_hop_job;
 int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream);
 
@@ -391,6 +399,15 @@ void shmt_graph_destroy(void *graph_exec);
 int shmt_stage_seeds(const void *seeds, int seed_bytes, int64_t n, void *staged,
                      int staged_bytes, int64_t *len_out, uint64_t rng_seed,
                      uint64_t *rng_seed_out, void *stream);
+
+/* Row coordinate of every element of a CSR / CSC structure:
+ * rows_out[e] = r for offsets[r] <= e < offsets[r + 1], e < nnz = offsets[S]
+ * (given by the caller), out_bytes in {4,8} wide. Turns the (sub_indptr,
+ * labels) pair of a sampled block into the (col, row) pair of
+ * create_block_from_coo (python/shmtensor/sampling.py:21-27) for hops that
+ * did not produce it on the way (shmt_hop_job.coo_dst).                     */
+int shmt_csr_rows(const void *offsets, int ptr_bytes, int64_t S, int64_t nnz,
+                  void *rows_out, int out_bytes, void *stream);
 
 /* Cached sub-CSR: CreateCacheCSR, src/cache_graph_sampling.cu:455-492
  * (CSRIndicesCopyKernel :428-453). Step 1 writes

@@ -55,6 +55,7 @@ SIGNATURES = {
     "shmt_graph_launch": (_int, [_vp, _vp]),
     "shmt_graph_destroy": (None, [_vp]),
     "shmt_stage_seeds": (_int, [_vp, _int, _i64, _vp, _int, _vp, _c.c_uint64, _vp, _vp]),
+    "shmt_csr_rows": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp]),
     "shmt_subcsr_plan": (_int, [_vp, _int, _vp, _int, _i64, _vp, _vp, _i64, _vp, _vp]),
     "shmt_subcsr_copy": (_int, [_vp, _vp, _int, _int, _vp, _int, _i64, _vp, _i64, _vp, _vp]),
 }
@@ -68,7 +69,7 @@ class HopJob(_c.Structure):
                 ("sub_indptr", _vp), ("sub_indices", _vp), ("plan", _vp), ("plan_bytes", _i64),
                 ("elem_bytes", _int), ("total_out", _vp), ("scratch", _vp), ("scratch_bytes", _i64),
                 ("unique_out", _vp), ("labels_out", _vp), ("nnz_out", _vp), ("count_out", _vp),
-                ("count_dev_out", _vp)]
+                ("count_dev_out", _vp), ("coo_dst", _vp), ("coo_bytes", _int)]
 
 
 _lib = None
@@ -91,7 +92,7 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.shmt_abi_version() != 1:
+    if lib.shmt_abi_version() != 2:
         raise ShmtError("libshmt.so ABI version mismatch")
     _lib = lib
     return lib

@@ -544,12 +544,19 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
 // (sub_indptr, sub_indices, unique, relabel_indices): exactly what
 // csr_[cache_]sampling followed by tensor_relabel([seeds, sub_indices]) returns,
 // with relabel_indices = the labels of the sub_indices part.
-using HopResult = std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>;
+// With coordinate output (create_block_from_coo, python/shmtensor/sampling.py:21-27) a fifth
+// tensor follows: coo_dst[e] = position of the seed that sampled id e belongs to, so that
+// (row, col) = (relabel_indices, coo_dst) are the source and destination of every edge of the block.
+struct HopResult {
+  torch::Tensor sub_indptr, sub_indices, unique, relabel_indices;
+  torch::Tensor coo_dst;  // defined only when the coordinate form was asked for
+};
 
 struct CsrArgs {
   torch::Tensor indptr, indices;
   std::optional<torch::Tensor> gpu_indptr, gpu_indices;
   StaticHashmap *hashmap;
+  bool coo = false;  // hops also return the destination position of every sampled id
   // what the kernels dereference for indptr / indices (translated once per call, not once per hop)
   void *indptr_dev = nullptr, *indices_dev = nullptr;
   bool cached() const { return hashmap != nullptr; }
@@ -580,7 +587,7 @@ struct PendingHop {
   HopResult result;                       // valid when finished
   int64_t S = 0;                          // number of seeds the buffers are sized for
   bool counted_seeds = false;             // the kernels took the true number of seeds from device memory
-  torch::Tensor sub_indptr, sub_indices, unique, labels;
+  torch::Tensor sub_indptr, sub_indices, unique, labels, coo_dst;
   torch::Tensor workspace;                // plan + relabel input + relabel scratch, kept until the sizes are in
   Readback::Slot nnz_slot{}, count_slot{};
   int64_t *count_dev = nullptr;           // fused hops: the number of unique ids in device memory as well
@@ -603,8 +610,15 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds
                                g.cached() ? &*g.gpu_indices : nullptr, g.hashmap, seeds, num_picks,
                                replace, seed, stream_id);
     auto relabeled = tensor_relabel({seeds, std::get<1>(sampled)});
-    h.result = std::make_tuple(std::get<0>(sampled), std::get<1>(sampled), std::get<0>(relabeled),
-                               std::get<1>(relabeled)[1]);
+    h.result = HopResult{std::get<0>(sampled), std::get<1>(sampled), std::get<0>(relabeled),
+                         std::get<1>(relabeled)[1], torch::Tensor()};
+    if (g.coo) {
+      const torch::Tensor &sp = h.result.sub_indptr, &labels = h.result.relabel_indices;
+      h.result.coo_dst = torch::empty_like(labels);
+      check(shmt_csr_rows(sp.data_ptr(), static_cast<int>(sp.element_size()), seeds.numel(), labels.numel(),
+                          h.result.coo_dst.data_ptr(), static_cast<int>(labels.element_size()),
+                          current_stream()));
+    }
     h.finished = true;
     return h;
   }
@@ -621,8 +635,8 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds
   auto aligned = [](int64_t bytes) { return (bytes + 255) & ~int64_t{255}; };
   // Two allocations per hop (the allocator is shared by all host threads that drive
   // batches): one for the four results, which are typed views of it, and the count ...
-  torch::Tensor results =
-      device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) + 2 * aligned(n_max * eb) + 256);
+  torch::Tensor results = device_bytes(aligned((S + 1) * pb) + aligned(bound * ib) + 2 * aligned(n_max * eb) +
+                                       (g.coo ? aligned(bound * eb) : 0) + 256);
   int64_t offset = 0;
   auto carve = [&](int64_t count, int elem, torch::ScalarType type) {
     torch::Tensor t = results.narrow(0, offset, count * elem).view(type);
@@ -633,6 +647,7 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds
   h.sub_indices = carve(bound, ib, g.indices.scalar_type());
   h.unique = carve(n_max, eb, id_type);
   h.labels = carve(n_max, eb, id_type);
+  if (g.coo) h.coo_dst = carve(bound, eb, id_type);
   h.count_dev = reinterpret_cast<int64_t *>(static_cast<char *>(results.data_ptr()) + offset);
   // ... and one for everything that does not outlive the hop
   const int64_t plan_bytes = shmt_sample_plan_bytes(S);
@@ -674,6 +689,8 @@ PendingHop hop_issue(const CsrArgs &g, torch::Tensor seeds, const int64_t *seeds
   j.nnz_out = h.nnz_slot.dev;
   j.count_out = h.count_slot.dev;
   j.count_dev_out = h.count_dev;
+  j.coo_dst = g.coo ? h.coo_dst.data_ptr() : nullptr;
+  j.coo_bytes = eb;
   check(shmt_sample_hops_chained(&j, 1, stream));
   return h;
 }
@@ -687,8 +704,9 @@ HopResult hop_finish(PendingHop &h, int64_t true_seeds = -1) {
     TORCH_CHECK(S >= 0 && S <= h.S, "internal: chained hop finished without its seed count");
     const int64_t nnz = Readback::wait(h.nnz_slot);
     const int64_t U = Readback::wait(h.count_slot);
-    h.result = std::make_tuple(h.sub_indptr.narrow(0, 0, S + 1), h.sub_indices.narrow(0, 0, nnz),
-                               h.unique.narrow(0, 0, U), h.labels.narrow(0, S, nnz));
+    h.result = HopResult{h.sub_indptr.narrow(0, 0, S + 1), h.sub_indices.narrow(0, 0, nnz),
+                         h.unique.narrow(0, 0, U), h.labels.narrow(0, S, nnz),
+                         h.coo_dst.defined() ? h.coo_dst.narrow(0, 0, nnz) : torch::Tensor()};
     h.finished = true;
     // scratch goes back to the allocator of its stream; work queued later on
     // that stream is ordered after the kernels that still read it
@@ -736,8 +754,8 @@ torch::Tensor issue_counted_fetch(const PendingHop &h, const FeatureArgs &f, int
 HopResult sample_hop(torch::Tensor indptr, torch::Tensor indices,
                      std::optional<torch::Tensor> gpu_indptr, std::optional<torch::Tensor> gpu_indices,
                      StaticHashmap *hashmap, torch::Tensor seeds, int64_t num_picks, bool replace,
-                     std::optional<int64_t> seed, int64_t stream_id) {
-  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+                     std::optional<int64_t> seed, int64_t stream_id, bool coo) {
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap, coo};
   check_csr(g);
   PendingHop h = hop_issue(g, seeds, nullptr, num_picks, replace, seed, stream_id);
   return hop_finish(h);
@@ -786,7 +804,7 @@ BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<in
   std::vector<PendingHop> chain;  // queued hops whose sizes have not been read yet
   auto finish_chain = [&]() {
     for (PendingHop &h : chain) {
-      const int64_t true_seeds = batch.hops.empty() ? -1 : std::get<2>(batch.hops.back()).numel();
+      const int64_t true_seeds = batch.hops.empty() ? -1 : batch.hops.back().unique.numel();
       batch.hops.push_back(hop_finish(h, true_seeds));
     }
     chain.clear();
@@ -806,7 +824,7 @@ BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<in
         finish_chain();
       }
     }
-    if (chain.empty() && !batch.hops.empty()) seeds = std::get<2>(batch.hops.back());
+    if (chain.empty() && !batch.hops.empty()) seeds = batch.hops.back().unique;
     PendingHop h = hop_issue(g, seeds, seeds_len, k, replace, seed, rng_stream);
     if (h.finished)
       batch.hops.push_back(h.result);  // ran as two separate operators (never a chained hop)
@@ -821,7 +839,7 @@ BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<in
   const bool speculate = f.max_rows != 0 && row_shape(f.uva_data, 0).row_bytes > 0;
   if (chain.empty() || !speculate) {
     finish_chain();
-    batch.features = fetch_rows(f, batch.hops.empty() ? cuda_ids(seeds, "seeds") : std::get<2>(batch.hops.back()));
+    batch.features = fetch_rows(f, batch.hops.empty() ? cuda_ids(seeds, "seeds") : batch.hops.back().unique);
     return batch;
   }
   // the rows of the last hop's unique ids, fetched before the host knows how many there are
@@ -830,7 +848,7 @@ BatchResult run_hops(const CsrArgs &g, torch::Tensor seeds, const std::vector<in
   const int64_t rows = f.max_rows < 0 ? bound : std::min(bound, f.max_rows);
   torch::Tensor out = issue_counted_fetch(last, f, rows);
   finish_chain();
-  const torch::Tensor &nodes = std::get<2>(batch.hops.back());
+  const torch::Tensor &nodes = batch.hops.back().unique;
   batch.features = nodes.numel() <= rows ? out.narrow(0, 0, nodes.numel()) : fetch_rows(f, nodes);
   return batch;
 }
@@ -859,7 +877,7 @@ bool chains_entirely(int64_t S, const std::vector<int64_t> &num_picks) {
 // bookkeeping, not the GPU, is what bounds the rate).
 struct TogetherHop {
   int64_t s_max, n_max;
-  int64_t off_sp, off_si, off_unique, off_labels, off_count;  // bytes into the batch's results
+  int64_t off_sp, off_si, off_unique, off_labels, off_coo, off_count;  // bytes into the batch's results
   Readback::Slot nnz, count;
 };
 struct TogetherBatch {
@@ -902,6 +920,8 @@ std::vector<TogetherBatch> issue_together(const CsrArgs &g, const std::vector<to
       results_bytes += aligned(hp.n_max * bt.eb);
       hp.off_labels = results_bytes;
       results_bytes += aligned(hp.n_max * bt.eb);
+      hp.off_coo = results_bytes;
+      if (g.coo) results_bytes += aligned(s_max * k * bt.eb);
       hp.off_count = results_bytes;
       results_bytes += 256;
       plan_bytes[h] = shmt_sample_plan_bytes(s_max);
@@ -953,6 +973,8 @@ std::vector<TogetherBatch> issue_together(const CsrArgs &g, const std::vector<to
       j.nnz_out = hp.nnz.dev;
       j.count_out = hp.count.dev;
       j.count_dev_out = reinterpret_cast<int64_t *>(r + hp.off_count);
+      j.coo_dst = g.coo ? r + hp.off_coo : nullptr;
+      j.coo_bytes = bt.eb;
     }
   }
   for (size_t h = 0; h < H; ++h)
@@ -980,8 +1002,9 @@ std::vector<BatchResult> finish_together(const CsrArgs &g, std::vector<TogetherB
       const TogetherHop &hp = bt.hops[h];
       const int64_t nnz = Readback::wait(hp.nnz);
       const int64_t U = Readback::wait(hp.count);
-      out[b].hops.emplace_back(typed(hp.off_sp, 0, s_now + 1, pb), typed(hp.off_si, 0, nnz, ib),
-                               typed(hp.off_unique, 0, U, bt.eb), typed(hp.off_labels, s_now, nnz, bt.eb));
+      out[b].hops.push_back(HopResult{typed(hp.off_sp, 0, s_now + 1, pb), typed(hp.off_si, 0, nnz, ib),
+                                      typed(hp.off_unique, 0, U, bt.eb), typed(hp.off_labels, s_now, nnz, bt.eb),
+                                      g.coo ? typed(hp.off_coo, 0, nnz, bt.eb) : torch::Tensor()});
       s_now = U;
     }
   }
@@ -1120,7 +1143,7 @@ std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch
   };
   for (auto &batch : out) {
     for (auto &r : batch.hops)
-      for (const torch::Tensor &t : {std::get<0>(r), std::get<1>(r), std::get<2>(r), std::get<3>(r)})
+      for (const torch::Tensor &t : {r.sub_indptr, r.sub_indices, r.unique, r.relabel_indices, r.coo_dst})
         hand_over(t);
     hand_over(batch.features);
   }
@@ -1131,8 +1154,8 @@ std::vector<std::vector<HopResult>> sample_blocks(
     torch::Tensor indptr, torch::Tensor indices, std::optional<torch::Tensor> gpu_indptr,
     std::optional<torch::Tensor> gpu_indices, StaticHashmap *hashmap, std::vector<torch::Tensor> seeds,
     std::vector<int64_t> num_picks, bool replace, std::optional<std::vector<int64_t>> seeds_rng,
-    int64_t max_in_flight) {
-  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+    int64_t max_in_flight, bool coo) {
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap, coo};
   check_csr(g);
   std::vector<std::vector<HopResult>> out;
   for (BatchResult &b : drive_batches(g, seeds, num_picks, replace, seeds_rng, max_in_flight, nullptr))
@@ -1153,8 +1176,8 @@ std::vector<std::pair<std::vector<HopResult>, torch::Tensor>> sample_blocks_fetc
     std::vector<int64_t> num_picks, bool replace, torch::Tensor uva_data,
     std::optional<torch::Tensor> gpu_data, StaticHashmap *data_hashmap,
     std::optional<std::vector<int64_t>> seeds_rng, int64_t max_in_flight,
-    std::optional<int64_t> max_rows) {
-  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap};
+    std::optional<int64_t> max_rows, bool coo) {
+  CsrArgs g{indptr, indices, gpu_indptr, gpu_indices, hashmap, coo};
   check_csr(g);
   TORCH_CHECK(!max_rows.has_value() || *max_rows >= 0, "max_rows must be >= 0");
   FeatureArgs f{uva_data, gpu_data, data_hashmap, max_rows.value_or(-1)};
@@ -1307,10 +1330,10 @@ class SamplerState : public std::enable_shared_from_this<SamplerState> {
       auto view = [&](int64_t off, int64_t first, int64_t count, int elem, torch::ScalarType type) {
         return blob.narrow(0, off + first * elem, count * elem).view(type);
       };
-      out.emplace_back(view(b.off_sp, 0, s_now + 1, pb_, g_.indptr.scalar_type()),
-                       view(b.off_si, 0, nnz[h], ib_, g_.indices.scalar_type()),
-                       view(b.off_unique, 0, uniq[h], eb_, id_type),
-                       view(b.off_labels, s_now, nnz[h], eb_, id_type));
+      out.push_back(HopResult{view(b.off_sp, 0, s_now + 1, pb_, g_.indptr.scalar_type()),
+                              view(b.off_si, 0, nnz[h], ib_, g_.indices.scalar_type()),
+                              view(b.off_unique, 0, uniq[h], eb_, id_type),
+                              view(b.off_labels, s_now, nnz[h], eb_, id_type), torch::Tensor()});
       s_now = uniq[h];
     }
     return out;
@@ -1550,6 +1573,23 @@ class BatchSampler {
 
 void register_host_tensors(py::module &m);  // host_tensors.cc
 
+namespace pybind11 {
+namespace detail {
+// A hop goes to Python as the tuple (sub_indptr, sub_indices, unique, relabel_indices), with the
+// destination positions as a fifth member when the coordinate form was asked for.
+template <>
+struct type_caster<HopResult> {
+  PYBIND11_TYPE_CASTER(HopResult, const_name("Tuple[Tensor, ...]"));
+  bool load(handle, bool) { return false; }
+  static handle cast(const HopResult &h, return_value_policy, handle) {
+    if (h.coo_dst.defined())
+      return py::make_tuple(h.sub_indptr, h.sub_indices, h.unique, h.relabel_indices, h.coo_dst).release();
+    return py::make_tuple(h.sub_indptr, h.sub_indices, h.unique, h.relabel_indices).release();
+  }
+};
+}  // namespace detail
+}  // namespace pybind11
+
 PYBIND11_MODULE(ShmTensorLib, m) {
   m.doc() = "MI355X-native ShmTensor GPU-cache operators (HIP, gfx950)";
   register_host_tensors(m);
@@ -1584,15 +1624,16 @@ PYBIND11_MODULE(ShmTensorLib, m) {
       .def("tensor_relabel", &tensor_relabel, py::arg("tensors"))
       .def("sample_hop", &sample_hop, py::arg("indptr"), py::arg("indices"), py::arg("gpu_indptr"),
            py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"),
-           py::arg("replace"), py::arg("seed") = py::none(), py::arg("stream_id") = 0)
+           py::arg("replace"), py::arg("seed") = py::none(), py::arg("stream_id") = 0, py::arg("coo") = false)
       .def("sample_blocks", &sample_blocks, py::arg("indptr"), py::arg("indices"), py::arg("gpu_indptr"),
            py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"), py::arg("num_picks"),
-           py::arg("replace"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4)
+           py::arg("replace"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4,
+           py::arg("coo") = false)
       .def("sample_blocks_fetch", &sample_blocks_fetch, py::arg("indptr"), py::arg("indices"),
            py::arg("gpu_indptr"), py::arg("gpu_indices"), py::arg("hashmap"), py::arg("seeds"),
            py::arg("num_picks"), py::arg("replace"), py::arg("uva_data"), py::arg("gpu_data"),
            py::arg("data_hashmap"), py::arg("seeds_rng") = py::none(), py::arg("max_in_flight") = 4,
-           py::arg("max_rows") = py::none());
+           py::arg("max_rows") = py::none(), py::arg("coo") = false);
 
   py::class_<BatchSampler>(m, "BatchSampler")
       .def(py::init<torch::Tensor, torch::Tensor, std::optional<torch::Tensor>, std::optional<torch::Tensor>,

@@ -242,6 +242,8 @@ struct PickArgs {
   int64_t clear_n;
   uint64_t *wide_mark;          // receives wide_nonce when a seed or a sampled id lies outside [0, 2^32)
   uint64_t wide_nonce;
+  void *coo_out;                // optional: position of the seed each sampled id belongs to (the destination
+  int coo_bytes;                // side of the block's edges in coordinate form), coo_bytes wide
 };
 
 __device__ __forceinline__ void note_wide_id(const PickArgs &a, int64_t id) {
@@ -288,13 +290,15 @@ __device__ __forceinline__ int64_t pick_offset(const PickArgs &a, int64_t s, int
   return optr;
 }
 
+// s: position of the seed the id was sampled for.
 template <bool HOP>
-__device__ __forceinline__ void pick_store(const PickArgs &a, int64_t S, int64_t pos, int64_t v) {
+__device__ __forceinline__ void pick_store(const PickArgs &a, int64_t S, int64_t s, int64_t pos, int64_t v) {
   store_int(a.out, pos, a.idx_bytes, v);
   if (HOP && a.copy_out) {
     store_int(a.copy_out, S + pos, a.copy_bytes, v);
     note_wide_id(a, v);
   }
+  if (HOP && a.coo_out) store_int(a.coo_out, pos, a.coo_bytes, s);
 }
 
 template <bool HOP>
@@ -342,10 +346,10 @@ __device__ __forceinline__ void pick_narrow_body(unsigned bx, unsigned gx, const
       if (gl < k) {
         const int64_t node = load_int(a.seeds, s, a.seed_bytes);
         const uint64_t r = sample_draw(rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
-        pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
+        pick_store<HOP>(a, S, s, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
-      if (gl < deg) pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, gl));
+      if (gl < deg) pick_store<HOP>(a, S, s, optr + gl, load_adj(a, p.begin, gl));
     } else {
       // Floyd: for J = deg-k .. deg-1 draw t in [0, J]; take t unless already
       // taken, then take J. Draws in parallel, resolution in k ballot steps.
@@ -360,7 +364,7 @@ __device__ __forceinline__ void pick_narrow_body(unsigned bx, unsigned gx, const
         const bool taken = group_ballot_dyn(gl < step && mine == ts, G) != 0;
         if (gl == step) mine = taken ? (deg - k + step) : ts;
       }
-      if (gl < k) pick_store<HOP>(a, S, optr + gl, load_adj(a, p.begin, mine));
+      if (gl < k) pick_store<HOP>(a, S, s, optr + gl, load_adj(a, p.begin, mine));
     }
   }
 }
@@ -397,10 +401,10 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
       for (int64_t j = lane; j < k; j += kWave) {
         const uint64_t r = sample_draw(rng_seed, a.rng_stream, node, static_cast<uint32_t>(j),
                                        static_cast<uint64_t>(deg));
-        pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, static_cast<int64_t>(r)));
+        pick_store<HOP>(a, S, s, optr + j, load_adj(a, p.begin, static_cast<int64_t>(r)));
       }
     } else if (deg <= k) {
-      for (int64_t j = lane; j < deg; j += kWave) pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, j));
+      for (int64_t j = lane; j < deg; j += kWave) pick_store<HOP>(a, S, s, optr + j, load_adj(a, p.begin, j));
     } else {
       for (int64_t step = 0; step < k; ++step) {
         const int64_t J = deg - k + step;
@@ -425,7 +429,7 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
         int64_t c = 0;
         if (j < k) c = IN_LDS ? chosen_lds[j] : load_int(a.out, optr + j, a.idx_bytes);
         __syncthreads();
-        if (j < k) pick_store<HOP>(a, S, optr + j, load_adj(a, p.begin, c));
+        if (j < k) pick_store<HOP>(a, S, s, optr + j, load_adj(a, p.begin, c));
       }
       __syncthreads();
     }
@@ -494,6 +498,27 @@ __global__ __launch_bounds__(256) void subcsr_copy_kernel(const void *indptr, co
         const int64_t src = load_int(indptr, v, ptr_bytes) + (e - load_int(cache_indptr, r, ptr_bytes));
         store_int(cache_indices, e, idx_bytes, load_int(indices, src, idx_bytes));
       }
+    }
+    __syncthreads();
+  }
+}
+
+// rows_out[e] = the row r with offsets[r] <= e < offsets[r + 1], for every e < nnz: the row
+// coordinate of each element of a CSR / CSC structure. Element-parallel like the copy above.
+__global__ __launch_bounds__(256) void csr_rows_kernel(const void *offsets, int ptr_bytes, int64_t S,
+                                                       int64_t nnz, void *rows_out, int out_bytes) {
+  __shared__ int64_t bracket[2];
+  const int64_t nchunks = (nnz + kCopyChunk - 1) / kCopyChunk;
+  for (int64_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+    const int64_t e0 = c * kCopyChunk;
+    const int64_t e1 = (e0 + kCopyChunk < nnz ? e0 + kCopyChunk : nnz) - 1;
+    if (threadIdx.x < 2)
+      bracket[threadIdx.x] = row_of(offsets, ptr_bytes, 0, S - 1, threadIdx.x == 0 ? e0 : e1);
+    __syncthreads();
+    const int64_t rlo = bracket[0], rhi = bracket[1];
+    for (int j = 0; j < 8; ++j) {
+      const int64_t e = e0 + j * 256 + threadIdx.x;
+      if (e <= e1) store_int(rows_out, e, out_bytes, row_of(offsets, ptr_bytes, rlo, rhi, e));
     }
     __syncthreads();
   }
@@ -650,6 +675,8 @@ struct PickHopExtras {
   int64_t clear_n;
   uint64_t *wide_mark;
   uint64_t wide_nonce;
+  void *coo_out;
+  int coo_bytes;
 };
 
 template <bool HOP>
@@ -768,6 +795,8 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.clear_n = 0;
   a.wide_mark = nullptr;
   a.wide_nonce = 0;
+  a.coo_out = nullptr;
+  a.coo_bytes = 8;
   if (!hop) return pick_launch<false>(a, launcher);
   a.sub_indptr_rw = hop->sub_indptr_rw;
   a.tile_prefix = hop->tile_prefix;
@@ -782,6 +811,8 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.clear_n = hop->clear_n;
   a.wide_mark = hop->wide_mark;
   a.wide_nonce = hop->wide_nonce;
+  a.coo_out = hop->coo_out;
+  a.coo_bytes = hop->coo_bytes;
   return pick_launch<true>(a, launcher);
 }
 
@@ -808,7 +839,7 @@ int shmt_sample(const void *indptr, int ptr_bytes, const void *indices, int idx_
   if (rc) return rc;
   const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, plan_hop.raw_tiles_out, nnz_out,
                                const_cast<uint64_t *>(plan_hop.total_out), nullptr, nullptr, nullptr, 8,
-                               nullptr, 0, nullptr, 0};
+                               nullptr, 0, nullptr, 0, nullptr, 8};
   return pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                    plan, sub_indices, rng_seed, rng_stream, launcher, &pick_hop);
 }
@@ -820,8 +851,10 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
                     void *sub_indptr,
                     void *sub_indices, void *plan, int64_t plan_bytes, int elem_bytes, void *total_out,
                     void *scratch, int64_t scratch_bytes, void *unique_out, void *labels_out,
-                    int64_t *nnz_out, int64_t *count_out, int64_t *count_copy, Launcher launcher) {
+                    int64_t *nnz_out, int64_t *count_out, int64_t *count_copy, void *coo_dst, int coo_bytes,
+                    Launcher launcher) {
   SHMT_REQUIRE(S >= 1 && k >= 1, "shmt_sample_hop: S and num_picks must be >= 1");
+  SHMT_REQUIRE(coo_dst == nullptr || width_ok(coo_bytes), "shmt_sample_hop: coo_bytes must be 4 or 8");
   SHMT_REQUIRE(k <= ((1ll << 31) - 1 - S) / S, "shmt_sample_hop: S * (num_picks + 1) must be < 2^31");
   SHMT_REQUIRE(width_ok(idx_bytes) && width_ok(seed_bytes) && width_ok(ptr_bytes) && width_ok(elem_bytes),
                "shmt_sample_hop: ID can only be int32 or int64");
@@ -839,7 +872,8 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
   if (rc) return rc;
   const PickHopExtras pick_hop{sub_indptr, plan_hop.tile_prefix_out, plan_hop.raw_tiles_out, nnz_out,
                                const_cast<uint64_t *>(plan_hop.total_out), S_len, rng_seed_dev, total_out, elem_bytes,
-                               static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce};
+                               static_cast<uint4 *>(table.slots), table.n16, table.wide_mark, table.nonce,
+                               coo_dst, coo_bytes};
   rc = pick_impl(indices, cache_indices, idx_bytes, seeds, seed_bytes, S, k, replace, sub_indptr, ptr_bytes,
                  plan, sub_indices, rng_seed, rng_stream, launcher, &pick_hop);
   if (rc) return rc;
@@ -859,7 +893,7 @@ int shmt_sample_hop(const void *indptr, int ptr_bytes, const void *indices, int 
   return hop_impl(indptr, ptr_bytes, indices, idx_bytes, cache_indptr, cache_indices, map, seeds, seed_bytes,
                   S, nullptr, k, replace, rng_seed, nullptr, rng_stream, sub_indptr, sub_indices, plan, plan_bytes,
                   elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out, count_out,
-                  nullptr, Launcher{as_stream(stream), nullptr});
+                  nullptr, nullptr, 8, Launcher{as_stream(stream), nullptr});
 }
 
 int shmt_sample_hop_chained(const void *indptr, int ptr_bytes, const void *indices, int idx_bytes,
@@ -875,14 +909,15 @@ int shmt_sample_hop_chained(const void *indptr, int ptr_bytes, const void *indic
                   max_seeds, seeds_len, k, replace, rng_seed, rng_seed_dev, rng_stream, sub_indptr, sub_indices,
                   plan,
                   plan_bytes, elem_bytes, total_out, scratch, scratch_bytes, unique_out, labels_out, nnz_out,
-                  count_out, count_dev_out, Launcher{as_stream(stream), nullptr});
+                  count_out, count_dev_out, nullptr, 8, Launcher{as_stream(stream), nullptr});
 }
 
 static int hop_job(const shmt_hop_job &j, Launcher launcher) {
   return hop_impl(j.indptr, j.ptr_bytes, j.indices, j.idx_bytes, j.cache_indptr, j.cache_indices, j.map, j.seeds,
                   j.seed_bytes, j.max_seeds, j.seeds_len, j.k, j.replace, j.rng_seed, j.rng_seed_dev, j.rng_stream,
                   j.sub_indptr, j.sub_indices, j.plan, j.plan_bytes, j.elem_bytes, j.total_out, j.scratch,
-                  j.scratch_bytes, j.unique_out, j.labels_out, j.nnz_out, j.count_out, j.count_dev_out, launcher);
+                  j.scratch_bytes, j.unique_out, j.labels_out, j.nnz_out, j.count_out, j.count_dev_out, j.coo_dst,
+                  j.coo_bytes, launcher);
 }
 
 int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream) {
@@ -917,6 +952,19 @@ int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream)
       if (rc) return rc;
     }
   }
+  return SHMT_OK;
+}
+
+int shmt_csr_rows(const void *offsets, int ptr_bytes, int64_t S, int64_t nnz, void *rows_out,
+                  int out_bytes, void *stream) {
+  SHMT_REQUIRE(S >= 0 && nnz >= 0, "shmt_csr_rows: S and nnz must be >= 0");
+  SHMT_REQUIRE(width_ok(ptr_bytes) && width_ok(out_bytes), "shmt_csr_rows: ID can only be int32 or int64");
+  if (nnz == 0) return SHMT_OK;
+  SHMT_REQUIRE(S >= 1 && offsets && rows_out, "shmt_csr_rows: null buffer");
+  const int64_t nchunks = (nnz + kCopyChunk - 1) / kCopyChunk;
+  hipLaunchKernelGGL(csr_rows_kernel, dim3(grid_for(nchunks, 1)), dim3(256), 0, as_stream(stream), offsets,
+                     ptr_bytes, S, nnz, rows_out, out_bytes);
+  SHMT_LAUNCH_CHECK();
   return SHMT_OK;
 }
 

@@ -7,8 +7,10 @@ by `tensor_relabel([seeds, sub_indices])`, issued through the fused
 and optionally several batches in flight at once).
 
 Without DGL installed a block is a `CSCBlock` tuple (indptr, indices,
-num_src, num_dst); with DGL it is the DGLBlock the reference builds
-(python/shmtensor/sampling.py:9-18)."""
+num_src, num_dst), or with `block_format="coo"` a `COOBlock` tuple (row, col,
+num_src, num_dst) holding the source and destination of every edge; with DGL
+it is the DGLBlock the reference builds from either form
+(python/shmtensor/sampling.py:9-27)."""
 import collections
 import queue
 import threading
@@ -22,6 +24,9 @@ from .. import install_aliases
 capi = install_aliases()
 
 CSCBlock = collections.namedtuple("CSCBlock", ["indptr", "indices", "num_src", "num_dst"])
+# row[e] / col[e]: source / destination node of edge e, as positions in the block's source /
+# destination node lists (the arguments of create_block_from_coo, sampling.py:21-27)
+COOBlock = collections.namedtuple("COOBlock", ["row", "col", "num_src", "num_dst"])
 
 
 def _dgl():
@@ -42,6 +47,16 @@ def create_block_from_csc(indptr, indices, e_ids, num_src, num_dst):
     return DGLBlock(hgidx, (["_N"], ["_N"]), ["_E"])
 
 
+def create_block_from_coo(row, col, num_src, num_dst):
+    dgl = _dgl()
+    if dgl is None:
+        return COOBlock(row, col, num_src, num_dst)
+    from dgl.heterograph import DGLBlock
+    hgidx = dgl.heterograph_index.create_unitgraph_from_coo(
+        2, num_src, num_dst, row, col, formats=["coo", "csr", "csc"])
+    return DGLBlock(hgidx, (["_N"], ["_N"]), ["_E"])
+
+
 def _unpin(tensor):
     capi.unpin_memory(tensor)
 
@@ -50,7 +65,7 @@ class GPUSamplingDataloader:
 
     def __init__(self, indptr, indices, seeds, batchsize, num_picks, replace=False, use_ddp=False,
                  shuffle=True, drop_last=False, rng_seed=None, prefetch=1, background=False,
-                 indptr_on_device=False, features=None):
+                 indptr_on_device=False, features=None, block_format="csc"):
         self.indptr = indptr
         self.indices = indices
         self.seeds = seeds
@@ -86,6 +101,12 @@ class GPUSamplingDataloader:
         # largest batch seen so far (a batch that outgrows it is fetched after its count is known).
         self.features = features
         self._feature_rows = 0
+        # block_format="coo": blocks are built from (row, col) edge lists, the destination
+        # positions written by the sampling kernel itself; "csc" (the reference loader's
+        # choice, sampling.py:139-141): from (sub_indptr, relabelled indices)
+        if block_format not in ("csc", "coo"):
+            raise ValueError("block_format must be 'csc' or 'coo'")
+        self.block_format = block_format
 
         self.has_cache = False
         self.gpu_indptr = None
@@ -171,24 +192,30 @@ class GPUSamplingDataloader:
                  self.gpu_indices if cached else None, self.hashmap if cached else None)
         # the last fanout is applied to the seed layer (sampling.py:128)
         picks = list(reversed(self.num_picks))
+        coo = self.block_format == "coo"
         if self.features is None:
             chains = capi.sample_blocks(*graph, groups, picks, self.replace, seeds_rng=rng,
-                                        max_in_flight=self.prefetch)
+                                        max_in_flight=self.prefetch, coo=coo)
             rows = [None] * len(groups)
         else:
             uva_data, gpu_data, data_map = self.features
             guess = self._feature_rows + self._feature_rows // 4 + 1024 if self._feature_rows else 0
             fetched = capi.sample_blocks_fetch(*graph, groups, picks, self.replace, uva_data, gpu_data, data_map,
-                                               seeds_rng=rng, max_in_flight=self.prefetch, max_rows=guess)
+                                               seeds_rng=rng, max_in_flight=self.prefetch, max_rows=guess, coo=coo)
             chains = [hops for hops, _ in fetched]
             rows = [x for _, x in fetched]
             self._feature_rows = max([self._feature_rows] + [x.shape[0] for x in rows])
         out = []
         for seeds, chain, x in zip(groups, chains, rows):
             blocks, dst = [], seeds
-            for sub_indptr, _, unique_tensor, relabel_indices in chain:
-                blocks.insert(0, create_block_from_csc(sub_indptr, relabel_indices, torch.Tensor(),
-                                                       unique_tensor.numel(), dst.numel()))
+            for hop in chain:
+                sub_indptr, _, unique_tensor, relabel_indices = hop[:4]
+                if coo:
+                    blocks.insert(0, create_block_from_coo(relabel_indices, hop[4], unique_tensor.numel(),
+                                                           dst.numel()))
+                else:
+                    blocks.insert(0, create_block_from_csc(sub_indptr, relabel_indices, torch.Tensor(),
+                                                           unique_tensor.numel(), dst.numel()))
                 dst = unique_tensor
             out.append((dst, seeds, blocks) if self.features is None else (dst, seeds, blocks, x))
         return out
@@ -247,7 +274,7 @@ class GPUSamplingDataloader:
         current.wait_event(done)
         for item in group:                 # produced on other streams, consumed on this one
             dst, blocks = item[0], item[2]
-            for t in (dst,) + tuple(item[3:]) + tuple(x for blk in blocks if isinstance(blk, CSCBlock)
+            for t in (dst,) + tuple(item[3:]) + tuple(x for blk in blocks if isinstance(blk, (CSCBlock, COOBlock))
                                                       for x in blk[:2]):
                 if t.numel() > 0:
                     t.record_stream(current)

@@ -24,7 +24,7 @@ def test_every_declared_symbol_is_exported(cabi):
 
 def test_size_queries_and_validation(cabi):
     lib = cabi.load()
-    assert lib.shmt_abi_version() == 1
+    assert lib.shmt_abi_version() == 2
     assert lib.shmt_hashmap_capacity(50000, 0.8) == 62500
     assert lib.shmt_hashmap_capacity(3, 0.8) == 4
     # 8 wide slots or 16 narrow slots per 128-byte bucket
