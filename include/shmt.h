@@ -82,6 +82,48 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys,
                         const void *vals, int64_t n, int key_bytes,
                         int val_bytes, double load_factor, void *table_mem,
                         int64_t table_bytes, void *stream);
+/* Build with a layout chosen from the keys. Node ids are small dense
+ * integers, so beside the general bucket table two flat forms exist:
+ *   SHMT_MAP_DIRECT  keys lie in [lo, lo + span) and an int32 table
+ *                    value[key - lo] is no larger than the bucket table would
+ *                    be: one 4-byte load per lookup;
+ *   SHMT_MAP_RANGE   the keys are exactly lo .. lo + span - 1 and every value
+ *                    is key + delta (the cache holds an id range, as in
+ *                    re-numbered graphs): lookups are arithmetic, no table;
+ * and the bucket table uses 8-byte slots whenever all keys and values fit 32
+ * bits, whatever their dtype. Every form answers exactly like the general
+ * table (same contract as the constructor above: include/cuco_hashmap.cuh:
+ * 57-87). shmt_hashmap_plan looks at the keys and values (one sweep, plus a
+ * repeat check for range candidates), SYNCHRONISES the stream once and fills
+ * `layout`, including the table_bytes the caller has to provide;
+ * shmt_hashmap_create_planned then builds that layout (asynchronous).
+ * `scratch` is device memory of shmt_hashmap_plan_scratch_bytes(n) bytes,
+ * 16-byte aligned, free again when plan returns.                            */
+#define SHMT_MAP_BUCKETS 0
+#define SHMT_MAP_DIRECT 1
+#define SHMT_MAP_RANGE 2
+typedef struct shmt_hashmap_layout {
+  int kind;            /* SHMT_MAP_*                                        */
+  int slot_bytes;      /* buckets: 16 or 8; direct: 4; range: 0             */
+  int64_t lo, span;    /* flat forms: id range [lo, lo + span)              */
+  int64_t delta;       /* range: value = key + delta                        */
+  int64_t table_bytes; /* device memory the build needs (128-byte aligned)  */
+} shmt_hashmap_layout;
+int64_t shmt_hashmap_plan_scratch_bytes(int64_t n);
+int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n,
+                      int key_bytes, int val_bytes, double load_factor,
+                      void *scratch, int64_t scratch_bytes,
+                      shmt_hashmap_layout *layout, void *stream);
+int shmt_hashmap_create_planned(shmt_hashmap_t **out,
+                                const shmt_hashmap_layout *layout,
+                                const void *keys, const void *vals, int64_t n,
+                                int key_bytes, int val_bytes,
+                                double load_factor, void *table_mem,
+                                int64_t table_bytes, void *stream);
+/* SHMT_MAP_* of a built map, and the table bytes it actually uses.         */
+int shmt_hashmap_kind(const shmt_hashmap_t *map);
+int64_t shmt_hashmap_used_bytes(const shmt_hashmap_t *map);
+
 /* Bulk lookup (query, src/cuco_hashmap.cu:24-34 + include/cuco_hashmap.cuh:
  * 81-87): requests of width req_bytes in {4,8} are first converted to the
  * key width (two's-complement narrowing / sign extension, as

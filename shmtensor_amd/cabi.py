@@ -21,6 +21,11 @@ SIGNATURES = {
     "shmt_hashmap_capacity": (_i64, [_i64, _dbl]),
     "shmt_hashmap_table_bytes": (_i64, [_i64, _dbl, _int, _int]),
     "shmt_hashmap_create": (_int, [_c.POINTER(_vp), _vp, _vp, _i64, _int, _int, _dbl, _vp, _i64, _vp]),
+    "shmt_hashmap_plan_scratch_bytes": (_i64, [_i64]),
+    "shmt_hashmap_plan": (_int, [_vp, _vp, _i64, _int, _int, _dbl, _vp, _i64, _vp, _vp]),
+    "shmt_hashmap_create_planned": (_int, [_c.POINTER(_vp), _vp, _vp, _vp, _i64, _int, _int, _dbl, _vp, _i64, _vp]),
+    "shmt_hashmap_kind": (_int, [_vp]),
+    "shmt_hashmap_used_bytes": (_i64, [_vp]),
     "shmt_hashmap_query": (_int, [_vp, _vp, _int, _i64, _vp, _vp]),
     "shmt_hashmap_key_bytes": (_int, [_vp]),
     "shmt_hashmap_val_bytes": (_int, [_vp]),
@@ -59,6 +64,12 @@ SIGNATURES = {
     "shmt_subcsr_plan": (_int, [_vp, _int, _vp, _int, _i64, _vp, _vp, _i64, _vp, _vp]),
     "shmt_subcsr_copy": (_int, [_vp, _vp, _int, _int, _vp, _int, _i64, _vp, _i64, _vp, _vp]),
 }
+
+class HashmapLayout(_c.Structure):
+    """shmt_hashmap_layout of include/shmt.h."""
+    _fields_ = [("kind", _int), ("slot_bytes", _int), ("lo", _i64), ("span", _i64), ("delta", _i64),
+                ("table_bytes", _i64)]
+
 
 class HopJob(_c.Structure):
     """shmt_hop_job of include/shmt.h: the parameters of one shmt_sample_hop_chained call."""

@@ -28,7 +28,7 @@
 
 namespace shmt {
 
-enum RouteMode : int { kDirect = 0, kMap16 = 1, kMap8 = 2, kMask = 3 };
+enum RouteMode : int { kDirect = 0, kMap16 = 1, kMap8 = 2, kMask = 3, kMapFlat = 4 };
 
 struct RowArgs {
   char *miss;          // table addressed by id (pinned host alias or device)
@@ -106,6 +106,9 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
       slot = wave_find<kSlot16, kFindBatch>(a.map, live ? map_key(a.map, idx) : -1);
     } else if (MODE == kMap8) {
       slot = wave_find<kSlot8, kFindBatch>(a.map, live ? map_key(a.map, idx) : -1);
+    } else if (MODE == kMapFlat) {
+      // direct or range form of the map: one 4-byte load, or arithmetic only
+      if (live) slot = flat_find(a.map, map_key(a.map, idx));
     }
     const int64_t my_table_row =
         reinterpret_cast<int64_t>(slot >= 0 ? a.cache + slot * R : a.miss + idx * R);
@@ -206,6 +209,9 @@ static void launch_through(int mode, unsigned grid, hipStream_t s, const RowArgs
     case kMap8:
       hipLaunchKernelGGL((rows_kernel<VT, kMap8, true, ONE_VEC, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
+    case kMapFlat:
+      hipLaunchKernelGGL((rows_kernel<VT, kMapFlat, true, ONE_VEC, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
     default:
       hipLaunchKernelGGL((rows_kernel<VT, kMask, true, ONE_VEC, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
@@ -223,6 +229,9 @@ static void launch_mode(int mode, unsigned grid, hipStream_t s, const RowArgs &a
       break;
     case kMap8:
       hipLaunchKernelGGL((rows_kernel<VT, kMap8, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+    case kMapFlat:
+      hipLaunchKernelGGL((rows_kernel<VT, kMapFlat, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
       break;
     default:
       hipLaunchKernelGGL((rows_kernel<VT, kMask, SET, ONE_VEC>), dim3(grid), dim3(kRowsBlock), 0, s, a);
@@ -260,7 +269,7 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   SHMT_REQUIRE(miss != nullptr, "%s: the id-addressed table is null", who);
   int mode = kDirect;
   if (map) {
-    mode = map->fmt == kSlot16 ? kMap16 : kMap8;
+    mode = map->kind != kKindBuckets ? kMapFlat : (map->fmt == kSlot16 ? kMap16 : kMap8);
     // an empty map never yields a slot, so an empty (null) cache table is fine with it
     SHMT_REQUIRE(cache != nullptr || map->n == 0, "%s: cache table is null", who);
   } else if (mask) {
@@ -275,7 +284,7 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   a.dense = static_cast<char *>(dense);
   a.indices = indices;
   a.mask = mask;
-  if (map) a.map = map->view; else a.map = MapView{nullptr, 1, 0};
+  if (map) a.map = map->view; else a.map = empty_map_view();
   a.Q = Q;
   a.count = count;
   a.count_seen = count_seen;

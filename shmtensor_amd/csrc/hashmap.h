@@ -6,7 +6,8 @@
 
 struct shmt_hashmap {
   shmt::MapView view;     // passed by value to kernels
-  int fmt;                // shmt::kSlot16 or shmt::kSlot8
+  int kind;               // shmt::MapKind
+  int fmt;                // bucket table: shmt::kSlot16 or shmt::kSlot8
   int key_bytes;
   int val_bytes;
   int64_t n;              // number of (key, value) pairs given to the build

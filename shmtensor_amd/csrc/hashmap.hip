@@ -144,6 +144,101 @@ __global__ __launch_bounds__(256) void hashmap_insert_kernel(
   }
 }
 
+// ---- what do the keys look like? ---------------------------------------------
+// One sweep over (keys, values): extrema of both, and whether value - key is
+// the same for every pair. The host reads the result and picks the layout.
+struct KeyStats {
+  long long kmin, kmax, vmin, vmax;
+  unsigned long long not_affine;  // != 0: value - key differs between pairs
+  unsigned long long repeats;     // range candidates only: keys seen more than once
+};
+
+__global__ void stats_init_kernel(KeyStats *st) {
+  st->kmin = INT64_MAX;
+  st->kmax = INT64_MIN;
+  st->vmin = INT64_MAX;
+  st->vmax = INT64_MIN;
+  st->not_affine = 0;
+  st->repeats = 0;
+}
+
+__device__ __forceinline__ int64_t wave_min64(int64_t v) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int64_t o = shfl64(v, lane_id() ^ d);
+    v = o < v ? o : v;
+  }
+  return v;
+}
+__device__ __forceinline__ int64_t wave_max64(int64_t v) {
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int64_t o = shfl64(v, lane_id() ^ d);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(256) void key_stats_kernel(const void *keys, const void *vals, int64_t n,
+                                                        int key_bytes, int val_bytes, KeyStats *st) {
+  const int64_t delta0 = load_int(vals, 0, val_bytes) - load_int(keys, 0, key_bytes);
+  int64_t kmin = INT64_MAX, kmax = INT64_MIN, vmin = INT64_MAX, vmax = INT64_MIN;
+  bool off = false;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int64_t k = load_int(keys, i, key_bytes), v = load_int(vals, i, val_bytes);
+    kmin = k < kmin ? k : kmin;
+    kmax = k > kmax ? k : kmax;
+    vmin = v < vmin ? v : vmin;
+    vmax = v > vmax ? v : vmax;
+    off |= (v - k != delta0);
+  }
+  kmin = wave_min64(kmin);
+  kmax = wave_max64(kmax);
+  vmin = wave_min64(vmin);
+  vmax = wave_max64(vmax);
+  const bool any_off = __builtin_amdgcn_ballot_w64(off) != 0;
+  if (lane_id() == 0) {
+    atomicMin(&st->kmin, static_cast<long long>(kmin));
+    atomicMax(&st->kmax, static_cast<long long>(kmax));
+    atomicMin(&st->vmin, static_cast<long long>(vmin));
+    atomicMax(&st->vmax, static_cast<long long>(vmax));
+    if (any_off) atomicOr(&st->not_affine, 1ull);
+  }
+}
+
+// Range candidates (as many pairs as ids between the extrema): every key sets
+// its bit; a bit found set already is a repeated key, and then some id of the
+// range is missing.
+__global__ __launch_bounds__(256) void key_repeats_kernel(const void *keys, int64_t n, int key_bytes,
+                                                          int64_t lo, uint32_t *bits, KeyStats *st) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  bool repeat = false;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint64_t off = static_cast<uint64_t>(load_int(keys, i, key_bytes) - lo);
+    if (off >= static_cast<uint64_t>(n)) continue;  // cannot happen for a true candidate
+    const uint32_t bit = 1u << (off & 31);
+    repeat |= (atomicOr(&bits[off >> 5], bit) & bit) != 0;
+  }
+  if (__builtin_amdgcn_ballot_w64(repeat) != 0 && lane_id() == 0) atomicOr(&st->repeats, 1ull);
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *p, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
+}
+
+// Direct form: value[key - lo] for every pair (the table was filled with -1).
+__global__ __launch_bounds__(256) void direct_build_kernel(int32_t *table, int64_t lo, int64_t span,
+                                                           const void *keys, const void *vals, int64_t n,
+                                                           int key_bytes, int val_bytes) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint64_t off = static_cast<uint64_t>(load_int(keys, i, key_bytes) - lo);
+    if (off < static_cast<uint64_t>(span)) table[off] = static_cast<int32_t>(load_int(vals, i, val_bytes));
+  }
+}
+
 // Bulk query: a wave owns 64 consecutive requests. The eight bucket loads of
 // a probe group (one per step) are all issued before the first is examined,
 // which keeps 8 KiB of table reads in flight per wave; results are gathered
@@ -186,9 +281,161 @@ int64_t shmt_hashmap_table_bytes(int64_t n, double load_factor, int key_bytes, i
   return buckets_for(n, load_factor, format_for(key_bytes, val_bytes)) * kBucketBytes;
 }
 
+int64_t shmt_hashmap_plan_scratch_bytes(int64_t n) {
+  if (n < 0) return -1;
+  return 256 + ((n + 31) / 32) * 4;
+}
+
+int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_bytes, int val_bytes,
+                      double load_factor, void *scratch, int64_t scratch_bytes,
+                      shmt_hashmap_layout *layout, void *stream) {
+  SHMT_REQUIRE(layout != nullptr, "shmt_hashmap_plan: layout is null");
+  SHMT_REQUIRE(n >= 0, "shmt_hashmap_plan: n must be >= 0");
+  SHMT_REQUIRE(width_ok(key_bytes) && width_ok(val_bytes),
+               "shmt_hashmap_plan: ID can only be int32 or int64 (key_bytes=%d, val_bytes=%d)", key_bytes,
+               val_bytes);
+  SHMT_REQUIRE(load_factor > 0.0 && load_factor <= 1.0, "shmt_hashmap_plan: load_factor must be in (0, 1], got %g",
+               load_factor);
+  const int dtype_fmt = format_for(key_bytes, val_bytes);
+  layout->kind = SHMT_MAP_BUCKETS;
+  layout->slot_bytes = dtype_fmt;
+  layout->lo = layout->span = layout->delta = 0;
+  layout->table_bytes = buckets_for(n, load_factor, dtype_fmt) * kBucketBytes;
+  if (n == 0) return SHMT_OK;
+  SHMT_REQUIRE(keys != nullptr && vals != nullptr, "shmt_hashmap_plan: keys/vals are null");
+  if (scratch == nullptr || scratch_bytes < shmt_hashmap_plan_scratch_bytes(n)) {
+    set_error("shmt_hashmap_plan: scratch too small (%lld < %lld bytes)", static_cast<long long>(scratch_bytes),
+              static_cast<long long>(shmt_hashmap_plan_scratch_bytes(n)));
+    return SHMT_ENOMEM;
+  }
+  SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "shmt_hashmap_plan: scratch must be 16-byte aligned");
+  hipStream_t s = as_stream(stream);
+  KeyStats *dev_stats = static_cast<KeyStats *>(scratch);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + 256);
+  hipLaunchKernelGGL(stats_init_kernel, dim3(1), dim3(1), 0, s, dev_stats);
+  hipLaunchKernelGGL(key_stats_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, vals, n,
+                     key_bytes, val_bytes, dev_stats);
+  SHMT_LAUNCH_CHECK();
+  KeyStats st;
+  SHMT_HIP(hipMemcpyAsync(&st, dev_stats, sizeof(st), hipMemcpyDeviceToHost, s));
+  SHMT_HIP(hipStreamSynchronize(s));
+
+  const bool keys32 = st.kmin >= INT32_MIN && st.kmax <= INT32_MAX;
+  const bool vals32 = st.vmin >= INT32_MIN && st.vmax <= INT32_MAX;
+  // narrow slots whenever every key and value fits 32 bits, whatever the dtypes say
+  const int fmt = (keys32 && vals32) ? kSlot8 : kSlot16;
+  layout->slot_bytes = fmt;
+  layout->table_bytes = buckets_for(n, load_factor, fmt) * kBucketBytes;
+  // flat forms need non-negative ids (-1 is the empty key) and a span that can be indexed
+  if (st.kmin < 0 || st.kmax - st.kmin >= (1ll << 40)) return SHMT_OK;
+  const int64_t span = st.kmax - st.kmin + 1;
+  if (span == n && !st.not_affine) {
+    // as many pairs as ids in the range and one offset for all: a range map unless a key repeats
+    const int64_t words = (n + 31) / 32;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(words, 256 * 4)), dim3(256), 0, s, bits, words);
+    hipLaunchKernelGGL(key_repeats_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, n,
+                       key_bytes, static_cast<int64_t>(st.kmin), bits, dev_stats);
+    SHMT_LAUNCH_CHECK();
+    SHMT_HIP(hipMemcpyAsync(&st, dev_stats, sizeof(st), hipMemcpyDeviceToHost, s));
+    SHMT_HIP(hipStreamSynchronize(s));
+    if (!st.repeats) {
+      layout->kind = SHMT_MAP_RANGE;
+      layout->slot_bytes = 0;
+      layout->lo = st.kmin;
+      layout->span = span;
+      layout->delta = st.vmin - st.kmin;  // value - key is one constant, so the minima pair up
+      layout->table_bytes = kBucketBytes;  // nothing is stored; callers still pass a valid pointer
+      return SHMT_OK;
+    }
+  }
+  // direct table when it is no larger than the bucket table would be
+  if (vals32 && span * 4 <= layout->table_bytes) {
+    layout->kind = SHMT_MAP_DIRECT;
+    layout->slot_bytes = 4;
+    layout->lo = st.kmin;
+    layout->span = span;
+    layout->table_bytes = (span * 4 + kBucketBytes - 1) / kBucketBytes * kBucketBytes;
+  }
+  return SHMT_OK;
+}
+
+static int build_buckets(shmt_hashmap_t **out, int fmt, const void *keys, const void *vals, int64_t n,
+                         int key_bytes, int val_bytes, double load_factor, void *table_mem,
+                         int64_t table_bytes, void *stream);
+
+int shmt_hashmap_create_planned(shmt_hashmap_t **out, const shmt_hashmap_layout *layout, const void *keys,
+                                const void *vals, int64_t n, int key_bytes, int val_bytes,
+                                double load_factor, void *table_mem, int64_t table_bytes, void *stream) {
+  SHMT_REQUIRE(out != nullptr && layout != nullptr, "shmt_hashmap_create_planned: null argument");
+  *out = nullptr;
+  SHMT_REQUIRE(n >= 0, "shmt_hashmap_create_planned: n must be >= 0");
+  SHMT_REQUIRE(width_ok(key_bytes) && width_ok(val_bytes),
+               "shmt_hashmap_create_planned: ID can only be int32 or int64 (key_bytes=%d, val_bytes=%d)",
+               key_bytes, val_bytes);
+  SHMT_REQUIRE(load_factor > 0.0 && load_factor <= 1.0,
+               "shmt_hashmap_create_planned: load_factor must be in (0, 1], got %g", load_factor);
+  if (layout->kind == SHMT_MAP_BUCKETS) {
+    SHMT_REQUIRE(layout->slot_bytes == kSlot16 || layout->slot_bytes == kSlot8,
+                 "shmt_hashmap_create_planned: bad slot size %d", layout->slot_bytes);
+    return build_buckets(out, layout->slot_bytes, keys, vals, n, key_bytes, val_bytes, load_factor, table_mem,
+                         table_bytes, stream);
+  }
+  SHMT_REQUIRE(layout->kind == SHMT_MAP_DIRECT || layout->kind == SHMT_MAP_RANGE,
+               "shmt_hashmap_create_planned: unknown layout kind %d", layout->kind);
+  SHMT_REQUIRE(n > 0 && keys != nullptr && vals != nullptr && layout->lo >= 0 && layout->span > 0,
+               "shmt_hashmap_create_planned: a flat layout needs keys and a non-negative id range");
+  hipStream_t s = as_stream(stream);
+  if (layout->kind == SHMT_MAP_DIRECT) {
+    if (table_mem == nullptr || table_bytes < layout->table_bytes || layout->table_bytes < layout->span * 4) {
+      set_error("shmt_hashmap_create_planned: table_mem too small (%lld < %lld bytes)",
+                static_cast<long long>(table_bytes), static_cast<long long>(layout->table_bytes));
+      return SHMT_ENOMEM;
+    }
+    SHMT_REQUIRE((reinterpret_cast<uintptr_t>(table_mem) & 127) == 0,
+                 "shmt_hashmap_create_planned: table_mem must be 128-byte aligned");
+    int rc = launch_fill_ones(table_mem, layout->table_bytes / 16, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(direct_build_kernel, dim3(grid_for(n, 256 * 4)), dim3(256), 0, s,
+                       static_cast<int32_t *>(table_mem), layout->lo, layout->span, keys, vals, n, key_bytes,
+                       val_bytes);
+    SHMT_LAUNCH_CHECK();
+  }
+  shmt_hashmap *h = static_cast<shmt_hashmap *>(calloc(1, sizeof(shmt_hashmap)));
+  if (h == nullptr) {
+    set_error("shmt_hashmap_create_planned: out of host memory");
+    return SHMT_ENOMEM;
+  }
+  h->view = empty_map_view();
+  h->view.buckets = static_cast<const uint4 *>(table_mem);
+  h->view.key32 = (key_bytes == 4);
+  h->view.kind = layout->kind == SHMT_MAP_DIRECT ? kKindDirect : kKindRange;
+  h->view.lo = layout->lo;
+  h->view.span = layout->span;
+  h->view.delta = layout->delta;
+  h->kind = h->view.kind;
+  h->fmt = kSlot8;  // kernels that branch on the kind at run time are launched in this form
+  h->key_bytes = key_bytes;
+  h->val_bytes = val_bytes;
+  h->n = n;
+  h->table_bytes = layout->kind == SHMT_MAP_DIRECT ? layout->table_bytes : 0;
+  *out = h;
+  return SHMT_OK;
+}
+
 int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys, const void *vals, int64_t n,
                         int key_bytes, int val_bytes, double load_factor, void *table_mem,
                         int64_t table_bytes, void *stream) {
+  SHMT_REQUIRE(width_ok(key_bytes) && width_ok(val_bytes),
+               "shmt_hashmap_create: ID can only be int32 or int64 (key_bytes=%d, val_bytes=%d)",
+               key_bytes, val_bytes);
+  return build_buckets(out, format_for(key_bytes, val_bytes), keys, vals, n, key_bytes, val_bytes, load_factor,
+                       table_mem, table_bytes, stream);
+}
+
+// Bucket table in slot format `fmt` (kSlot8 requires that every key and value fits 32 bits).
+static int build_buckets(shmt_hashmap_t **out, const int fmt, const void *keys, const void *vals, int64_t n,
+                         int key_bytes, int val_bytes, double load_factor, void *table_mem,
+                         int64_t table_bytes, void *stream) {
   SHMT_REQUIRE(out != nullptr, "shmt_hashmap_create: out is null");
   *out = nullptr;
   SHMT_REQUIRE(n >= 0, "shmt_hashmap_create: n must be >= 0");
@@ -199,7 +446,6 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys, const void *vals
                "shmt_hashmap_create: load_factor must be in (0, 1], got %g", load_factor);
   SHMT_REQUIRE(n == 0 || (keys != nullptr && vals != nullptr),
                "shmt_hashmap_create: keys/vals are null");
-  const int fmt = format_for(key_bytes, val_bytes);
   const int64_t nb = buckets_for(n, load_factor, fmt);
   SHMT_REQUIRE(nb < (1ll << 31), "shmt_hashmap_create: table too large (%lld buckets)",
                static_cast<long long>(nb));
@@ -232,9 +478,12 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys, const void *vals
     set_error("shmt_hashmap_create: out of host memory");
     return SHMT_ENOMEM;
   }
+  h->view = empty_map_view();
   h->view.buckets = static_cast<const uint4 *>(table_mem);
   h->view.nbuckets = static_cast<uint32_t>(nb);
   h->view.key32 = (key_bytes == 4);
+  h->view.fits32 = (fmt == kSlot8 && key_bytes == 8);
+  h->kind = kKindBuckets;
   h->fmt = fmt;
   h->key_bytes = key_bytes;
   h->val_bytes = val_bytes;
@@ -263,6 +512,8 @@ int shmt_hashmap_query(const shmt_hashmap_t *map, const void *requests, int req_
   return SHMT_OK;
 }
 
+int shmt_hashmap_kind(const shmt_hashmap_t *map) { return map ? map->kind : -1; }
+int64_t shmt_hashmap_used_bytes(const shmt_hashmap_t *map) { return map ? map->table_bytes : 0; }
 int shmt_hashmap_key_bytes(const shmt_hashmap_t *map) { return map ? map->key_bytes : 0; }
 int shmt_hashmap_val_bytes(const shmt_hashmap_t *map) { return map ? map->val_bytes : 0; }
 int64_t shmt_hashmap_size(const shmt_hashmap_t *map) { return map ? map->n : 0; }

@@ -13,6 +13,17 @@
 // linearly from hash(key) and are always placed in the first bucket of their
 // probe sequence that still has a free slot, so a lookup stops at the first
 // bucket that contains either the key or an empty slot.
+//
+// Two flat forms exist beside the bucket table, chosen when the map is built
+// from what its keys look like (node ids are dense small integers, and caches
+// of re-numbered graphs hold an id range):
+//   direct (kKindDirect): keys lie in [lo, lo + span) with span a small
+//                     multiple of their number; the table is int32
+//                     value[key - lo], -1 where no key was given. One 4-byte
+//                     load per lookup, no probe sequence.
+//   range  (kKindRange) : the keys are exactly the ids lo .. lo + span - 1 and
+//                     every value is key + delta; lookups are arithmetic and
+//                     touch no memory at all.
 #pragma once
 #include "wave.h"
 
@@ -23,17 +34,38 @@ enum SlotFormat : int { kSlot16 = 16, kSlot8 = 8 };
 constexpr int kProbeGroup = 8;      // lanes that cooperate on one key
 constexpr int kBucketBytes = 128;
 
+enum MapKind : int { kKindBuckets = 0, kKindDirect = 1, kKindRange = 2 };
+
 struct MapView {
-  const uint4 *buckets;   // nbuckets * 8 uint4
+  const uint4 *buckets;   // bucket table: nbuckets * 8 uint4; direct form: int32 values[span]
   uint32_t nbuckets;
-  int key32;              // 1: keys are int32 -> narrow requests before hashing
+  int key32;              // 1: keys are int32 -> requests are narrowed before the lookup
+  int kind;               // MapKind
+  int fits32;             // 1: 64-bit keys stored in narrow slots (they all fit): a request that
+                          //    does not fit 32 bits is absent
+  int64_t lo;             // flat forms: smallest key
+  int64_t span;           // flat forms: keys lie in [lo, lo + span)
+  int64_t delta;          // range form: value = key + delta
 };
+
+inline MapView empty_map_view() { return MapView{nullptr, 1, 0, kKindBuckets, 0, 0, 0, 0}; }
 
 // Normalise a request to the key domain of the map (what requests.to(key
 // dtype) does in the reference): int32-keyed maps see the low 32 bits,
-// sign-extended.
+// sign-extended. A request that cannot be a key of a narrow-stored 64-bit
+// map becomes the empty sentinel, which every lookup resolves to -1.
 __device__ __forceinline__ int64_t map_key(const MapView &m, int64_t req) {
-  return m.key32 ? static_cast<int64_t>(static_cast<int32_t>(req)) : req;
+  if (m.key32) return static_cast<int64_t>(static_cast<int32_t>(req));
+  if (m.fits32 && req != static_cast<int64_t>(static_cast<int32_t>(req))) return -1;
+  return req;
+}
+
+// Lookup in a flat map (kind != kKindBuckets); every lane for itself.
+__device__ __forceinline__ int64_t flat_find(const MapView &m, int64_t key) {
+  const uint64_t off = static_cast<uint64_t>(key) - static_cast<uint64_t>(m.lo);  // key < lo wraps around
+  if (off >= static_cast<uint64_t>(m.span)) return -1;
+  if (m.kind == kKindRange) return key + m.delta;
+  return static_cast<int64_t>(reinterpret_cast<const int32_t *>(m.buckets)[off]);
 }
 
 __device__ __forceinline__ uint32_t map_bucket(const MapView &m, int64_t key) {
@@ -79,6 +111,7 @@ __device__ __forceinline__ bool probe_step(const uint4 frag, int64_t key, int64_
 // table still terminates.
 template <int FMT>
 __device__ __forceinline__ int64_t group_find(const MapView &m, int64_t key) {
+  if (m.kind != kKindBuckets) return flat_find(m, key);
   const int sub = lane_id() & (kProbeGroup - 1);
   uint32_t b = map_bucket(m, key);
   int64_t val = -1;
@@ -97,10 +130,12 @@ __device__ __forceinline__ int64_t group_find(const MapView &m, int64_t key) {
 // examined, so the number of dependent HBM round trips is the longest probe
 // chain among the 64 keys, not the sum. Every lane gets the value for its own
 // key (or -1). All 64 lanes must be active; lanes with nothing to look up
-// pass -1 (the empty sentinel, which resolves to -1 in one round).
+// pass -1 (the empty sentinel, which resolves to -1 in one round). Flat maps
+// (direct / range form) are answered by every lane for itself.
 template <int FMT, int BATCH = kProbeGroup>
 __device__ __forceinline__ int64_t wave_find(const MapView &m, int64_t mykey) {
   static_assert(kProbeGroup % BATCH == 0, "BATCH must divide the probe group size");
+  if (m.kind != kKindBuckets) return flat_find(m, mykey);  // uniform across the launch
   const int sub = lane_id() & (kProbeGroup - 1);
   const int gbase = lane_id() & ~(kProbeGroup - 1);
   int64_t res = -1;

@@ -150,12 +150,19 @@ class StaticHashmap {
     values = values.contiguous();
     const int64_t n = keys.numel();
     capacity_ = shmt_hashmap_capacity(n, load_factor);
-    const int64_t bytes = shmt_hashmap_table_bytes(n, load_factor, kb, vb);
-    TORCH_CHECK(bytes > 0, shmt_last_error());
-    table_ = device_bytes(bytes);
-    memory_usage_ = bytes;
-    check(shmt_hashmap_create(&handle_, keys.data_ptr(), values.data_ptr(), n, kb, vb, load_factor,
-                              table_.data_ptr(), bytes, current_stream()));
+    // the layout follows from the keys (dense id range, 32-bit ids ...): look first, then allocate what it needs
+    shmt_hashmap_layout layout;
+    {
+      const int64_t scratch_bytes = shmt_hashmap_plan_scratch_bytes(n);
+      torch::Tensor scratch = device_bytes(scratch_bytes);
+      check(shmt_hashmap_plan(keys.data_ptr(), values.data_ptr(), n, kb, vb, load_factor, scratch.data_ptr(),
+                              scratch_bytes, &layout, current_stream()));
+    }
+    table_ = device_bytes(layout.table_bytes);
+    memory_usage_ = layout.kind == SHMT_MAP_RANGE ? 0 : layout.table_bytes;
+    kind_ = layout.kind;
+    check(shmt_hashmap_create_planned(&handle_, &layout, keys.data_ptr(), values.data_ptr(), n, kb, vb,
+                                      load_factor, table_.data_ptr(), layout.table_bytes, current_stream()));
   }
   ~StaticHashmap() { shmt_hashmap_destroy(handle_); }
   StaticHashmap(const StaticHashmap &) = delete;
@@ -173,6 +180,8 @@ class StaticHashmap {
   }
   int64_t capacity() const { return capacity_; }
   int64_t memory_usage() const { return memory_usage_; }
+  // "buckets", "direct" or "range": the layout the constructor chose for these keys
+  std::string layout() const { return kind_ == SHMT_MAP_RANGE ? "range" : kind_ == SHMT_MAP_DIRECT ? "direct" : "buckets"; }
   const shmt_hashmap_t *handle() const { return handle_; }
 
  private:
@@ -180,6 +189,7 @@ class StaticHashmap {
   torch::Tensor table_;
   torch::ScalarType key_type_, value_type_;
   int64_t capacity_ = 0, memory_usage_ = 0;
+  int kind_ = SHMT_MAP_BUCKETS;
 };
 
 // ---- pin / unpin -----------------------------------------------------------
@@ -1652,5 +1662,6 @@ PYBIND11_MODULE(ShmTensorLib, m) {
       .def(py::init<torch::Tensor, torch::Tensor, double>())
       .def("query", &StaticHashmap::query)
       .def("capacity", &StaticHashmap::capacity)
-      .def("memory_usage", &StaticHashmap::memory_usage);
+      .def("memory_usage", &StaticHashmap::memory_usage)
+      .def("layout", &StaticHashmap::layout);
 }

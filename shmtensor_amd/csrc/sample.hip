@@ -581,7 +581,7 @@ static int plan_impl(const void *indptr, int ptr_bytes, const void *cache_indptr
   a.partials = S > 0 ? reinterpret_cast<uint64_t *>(static_cast<char *>(plan) + S * sizeof(SeedPlan))
                      : nullptr;
   a.nnz_out = nnz_out;
-  if (map) a.map = map->view; else a.map = MapView{nullptr, 1, 0};
+  if (map) a.map = map->view; else a.map = empty_map_view();
   a.S = S;
   a.k = k;
   a.ptr_bytes = ptr_bytes;

@@ -103,3 +103,189 @@ def test_full_size_membership_property(capi):
     out = h.query(req[perm])
     expect = torch.cat([pick, torch.full_like(non, -1)])[perm]
     assert torch.equal(out, expect)
+
+
+# ---- layouts chosen from the keys ------------------------------------------------------------------
+# Whatever layout the constructor picks (bucket table with 16- or 8-byte slots, direct table, id range),
+# query() must answer like a dict of the pairs (include/cuco_hashmap.cuh:81-87): the oracle is the judge.
+
+def _probe_requests(rng, keys, lo, hi):
+    """Members, near misses on both sides of the key range, far values, values beyond 32 bits, -1."""
+    return np.concatenate([keys, rng.integers(lo - 50, hi + 50, size=5000), [lo - 1, hi + 1, -1, -2, 0],
+                           rng.integers(-2**40, 2**40, size=1000), [2**31, 2**32, 2**32 + int(keys[0]), -2**31]])
+
+
+_LAYOUT_CASES = ["range_identity", "range_offset", "range_shuffled", "range_from_zero_one_key", "range_with_repeat",
+                 "range_negative_values", "direct_permuted", "direct_sparse", "direct_too_sparse", "negative_keys",
+                 "values_beyond_32_bits"]
+
+
+@pytest.mark.parametrize("kd,vd,case", [(kd, vd, case) for kd in (np.int32, np.int64) for vd in (np.int32, np.int64)
+                                        for case in _LAYOUT_CASES
+                                        if not (case == "values_beyond_32_bits" and vd is np.int32)])
+def test_layouts_answer_like_a_dict(capi, oracle, kd, vd, case):
+    rng = np.random.default_rng(len(case) * 7 + np.dtype(kd).itemsize + 3 * np.dtype(vd).itemsize)
+    n = 30_000
+    expect_layout = None
+    if case == "range_identity":                     # a cache holding ids 0 .. n-1 in slot order
+        keys = np.arange(n)
+        vals = keys.copy()
+        expect_layout = "range"
+    elif case == "range_offset":                     # ids 1000 .. 1000+n-1 -> slots 7 ..
+        keys = np.arange(1000, 1000 + n)
+        vals = keys - 993
+        expect_layout = "range"
+    elif case == "range_shuffled":                   # the same pairs in any order
+        keys = rng.permutation(np.arange(500, 500 + n))
+        vals = keys - 500
+        expect_layout = "range"
+    elif case == "range_from_zero_one_key":
+        keys, vals = np.array([0]), np.array([5])
+        expect_layout = "range"
+    elif case == "range_with_repeat":                # n pairs over n ids but one id twice, so one is missing
+        keys = np.arange(n)
+        keys[17] = 16
+        vals = keys.copy()
+        expect_layout = "direct"
+    elif case == "range_negative_values":            # value = key - 20: key 19 maps to -1, i.e. reads as absent
+        keys = np.arange(n)
+        vals = keys - 20
+        expect_layout = "range"
+    elif case == "direct_permuted":                  # dense ids, slots in insertion (hotness) order
+        keys = rng.permutation(n)
+        vals = np.arange(n)
+        expect_layout = "direct"
+    elif case == "direct_sparse":                    # a third of an id universe
+        keys = rng.choice(3 * n, size=n, replace=False) + 12345
+        vals = np.arange(n)
+        expect_layout = "direct"
+    elif case == "direct_too_sparse":                # 1 id in 20: the bucket table is smaller
+        keys = rng.choice(20 * n, size=n, replace=False)
+        vals = np.arange(n)
+        expect_layout = "buckets"
+    elif case == "negative_keys":                    # dense, but ids below zero: bucket table
+        keys = rng.permutation(n) - 100
+        keys = keys[keys != -1]                      # -1 is the empty key
+        vals = np.arange(keys.size)
+        expect_layout = "buckets"
+    else:                                            # dense keys whose values need 64 bits
+        keys = rng.permutation(n)
+        vals = np.arange(n) + 2**33
+        expect_layout = "buckets"
+    keys, vals = keys.astype(kd), vals.astype(vd)
+    h = capi.CUCOStaticHashmap(_cuda(keys), _cuda(vals), 0.8)
+    assert h.layout() == expect_layout
+    ref = oracle.Hashmap(keys, vals, 0.8)
+    lo, hi = int(keys.min()), int(keys.max())
+    req = _probe_requests(rng, keys.astype(np.int64), lo, hi)
+    for rd in (np.int32, np.int64):
+        r = req.astype(rd)                           # int32: two's-complement narrowing, like .to(int32)
+        out = h.query(_cuda(r))
+        assert out.dtype == TD[vd]
+        if case == "range_with_repeat":
+            # the repeated key has one winner among its two values; every other answer is determined
+            want = ref.query(r)
+            got = out.cpu().numpy()
+            dup = r.astype(kd) == 16
+            assert np.array_equal(got[~dup], want[~dup]) and set(got[dup].tolist()) <= {16}
+            assert got[r.astype(kd) == 17].tolist() == [-1] * int((r.astype(kd) == 17).sum())
+        else:
+            assert np.array_equal(out.cpu().numpy(), ref.query(r))
+    assert h.capacity() == int(np.ceil(keys.size / 0.8))
+    if expect_layout == "range":
+        assert h.memory_usage() == 0
+    elif expect_layout == "direct":
+        assert h.memory_usage() <= (hi - lo + 1) * 4 + 128
+
+
+def test_wide_dtypes_with_small_ids_use_narrow_slots(capi, oracle):
+    """int64 keys and values that all fit 32 bits are stored in 8-byte slots; requests that do not fit
+    32 bits are absent (not truncated: only int32-KEYED maps narrow their requests)."""
+    rng = np.random.default_rng(3)
+    keys = rng.choice(50_000_000, size=40_000, replace=False).astype(np.int64)
+    vals = rng.integers(0, 2**31 - 1, size=keys.size).astype(np.int64)
+    h = capi.CUCOStaticHashmap(_cuda(keys), _cuda(vals), 0.5)
+    assert h.layout() == "buckets" and h.memory_usage() == 40_000 * 8 * 2
+    req = np.concatenate([keys, keys + 2**32, keys - 2**32, rng.integers(0, 50_000_000, size=10_000)])
+    assert np.array_equal(h.query(_cuda(req)).cpu().numpy(), oracle.Hashmap(keys, vals, 0.5).query(req))
+    wide = capi.CUCOStaticHashmap(_cuda(keys + 2**32), _cuda(vals), 0.5)        # keys beyond 32 bits: 16-byte slots
+    assert wide.memory_usage() == 40_000 * 16 * 2
+    assert np.array_equal(wide.query(_cuda(req)).cpu().numpy(), oracle.Hashmap(keys + 2**32, vals, 0.5).query(req))
+
+
+@pytest.mark.parametrize("layout", ["range", "direct"])
+def test_flat_layouts_route_fetch_set_and_sampling(capi, oracle, layout):
+    """cache_fetch / cache_set / csr_cache_sampling through a map in a flat layout against the oracle, with
+    cache rows made different from the host rows so that routing shows."""
+    rng = np.random.default_rng(8)
+    n, c = 5000, 2000
+    ids = np.arange(100, 100 + c) if layout == "range" else rng.choice(n, size=c, replace=False)
+    slots = ids - 100 if layout == "range" else np.arange(c)
+    h = capi.CUCOStaticHashmap(_cuda(ids), _cuda(slots), 0.8)
+    assert h.layout() == layout
+    ref = oracle.Hashmap(ids, slots, 0.8)
+    table = rng.standard_normal((n, 24)).astype(np.float32)
+    host = torch.from_numpy(table.copy()).pin_memory()
+    cache_np = np.empty((c, 24), np.float32)
+    cache_np[slots] = table[ids] + 1000.0
+    cache = _cuda(cache_np)
+    q = rng.integers(0, n, size=7001)
+    out = capi.cache_fetch(host, cache, _cuda(q), h)
+    assert np.array_equal(out.cpu().numpy(), oracle.fetch(table, cache_np, q, hashmap=ref))
+    w = rng.choice(n, size=1500, replace=False)
+    upd = rng.standard_normal((1500, 24)).astype(np.float32)
+    capi.cache_set(host, cache, _cuda(w), _cuda(upd), h)
+    torch.cuda.synchronize()
+    want_host, want_cache = table.copy(), cache_np.copy()
+    oracle.set_rows(want_host, want_cache, w, upd, hashmap=ref)
+    assert np.array_equal(host.numpy(), want_host) and np.array_equal(cache.cpu().numpy(), want_cache)
+    # sampling: cached rows (a sub-CSR in map order) and cold rows give what the uncached sampler gives
+    deg = rng.integers(0, 30, size=n)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    indices = rng.integers(0, n, size=int(indptr[-1])).astype(np.int32)
+    ip, ix = torch.from_numpy(indptr).pin_memory(), torch.from_numpy(indices).pin_memory()
+    order = np.empty(c, np.int64)
+    order[slots] = ids
+    gp, gi = capi.create_subcsr(ip, ix, _cuda(order))
+    seeds = _cuda(rng.permutation(n)[:3000])
+    a = capi.csr_cache_sampling(ip, ix, gp, gi, h, seeds, 7, False, seed=3)
+    b = capi.csr_sampling(ip, ix, seeds, 7, False, seed=3)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    esp, esi = oracle.sample(indptr, indices, seeds.cpu().numpy(), 7, False, seed=3, algo="floyd")
+    assert np.array_equal(a[0].cpu().numpy(), esp) and np.array_equal(a[1].cpu().numpy(), esi)
+
+
+def test_planned_build_through_the_c_abi(cabi):
+    """shmt_hashmap_plan / shmt_hashmap_create_planned with raw pointers: the layout struct, the sizes it
+    asks for and the answers of the built map."""
+    import ctypes
+    lib = cabi.load()
+    stream = cabi.current_stream()
+    keys = torch.arange(10, 1034).cuda()
+    vals = (keys - 10).contiguous()
+    n = keys.numel()
+    sb = lib.shmt_hashmap_plan_scratch_bytes(n)
+    assert sb >= 256 + n // 8
+    scratch = torch.empty(sb, dtype=torch.uint8, device="cuda")
+    lay = cabi.HashmapLayout()
+    cabi.check(lib.shmt_hashmap_plan(keys.data_ptr(), vals.data_ptr(), n, 8, 8, 0.8, scratch.data_ptr(), sb,
+                                     ctypes.byref(lay), stream))
+    assert (lay.kind, lay.lo, lay.span, lay.delta) == (2, 10, 1024, -10)
+    table = torch.empty(max(lay.table_bytes, 128), dtype=torch.uint8, device="cuda")
+    handle = ctypes.c_void_p()
+    cabi.check(lib.shmt_hashmap_create_planned(ctypes.byref(handle), ctypes.byref(lay), keys.data_ptr(),
+                                               vals.data_ptr(), n, 8, 8, 0.8, table.data_ptr(), table.numel(), stream))
+    assert lib.shmt_hashmap_kind(handle) == 2 and lib.shmt_hashmap_used_bytes(handle) == 0
+    req = torch.tensor([9, 10, 500, 1033, 1034, -1]).cuda()
+    out = torch.empty_like(req)
+    cabi.check(lib.shmt_hashmap_query(handle, req.data_ptr(), 8, req.numel(), out.data_ptr(), stream))
+    assert out.tolist() == [-1, 0, 490, 1023, -1, -1]
+    lib.shmt_hashmap_destroy(handle)
+    # scattered 64-bit keys: bucket table with 16-byte slots, sized like shmt_hashmap_table_bytes
+    big = (torch.arange(n).cuda() * 1_000_003 + (1 << 35)).contiguous()
+    cabi.check(lib.shmt_hashmap_plan(big.data_ptr(), vals.data_ptr(), n, 8, 8, 0.5, scratch.data_ptr(), sb,
+                                     ctypes.byref(lay), stream))
+    assert (lay.kind, lay.slot_bytes) == (0, 16) and lay.table_bytes == lib.shmt_hashmap_table_bytes(n, 0.5, 8, 8)
+    small = torch.empty(16, dtype=torch.uint8, device="cuda")
+    assert lib.shmt_hashmap_plan(big.data_ptr(), vals.data_ptr(), n, 8, 8, 0.5, small.data_ptr(), 16,
+                                 ctypes.byref(lay), stream) == -4                     # scratch too small
