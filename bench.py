@@ -26,7 +26,7 @@ Benchmark configurations referred to by number in this file:
      f32 features in pinned host memory, top-degree 25 % cached; 4,096 seeds, fanouts [25,15,10],
      relabel, then fetch of all input nodes
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,sampling,e2e]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,scan,sampling,e2e]
 """
 import argparse
 import collections
@@ -40,9 +40,22 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the config-4 fetch kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/rows_kernel_fetch_config4_pmc.md): FETCH_SIZE x 2.0 (calibrated on a copy of known size) + WRITE_SIZE.
-CONFIG4_TRAFFIC_BYTES = 414_600_424
+# HBM bytes per launch of the config-4 fetch kernel come from two rocprofv3 --pmc runs (FETCH_SIZE,
+# WRITE_SIZE); the summary of those runs states the scaled sum on a line of its own, which is read here.
+CONFIG4_PMC_SUMMARY = os.path.join(ROOT, "profiles", "rows_kernel_fetch_config4_pmc.md")
+
+
+def config4_traffic_bytes():
+    """`roofline.traffic`: the figure the counter summary under profiles/ states ("traffic_bytes_per_launch: N"),
+    or None when the summary is absent."""
+    try:
+        with open(CONFIG4_PMC_SUMMARY) as f:
+            for line in f:
+                if line.strip().startswith("traffic_bytes_per_launch:"):
+                    return int(line.split(":")[1].split()[0].replace(",", ""))
+    except OSError:
+        pass
+    return None
 
 
 def log(*a):
@@ -146,13 +159,14 @@ def bench_fetch(capi, args, result):
         "value": round(value, 2), "ms_per_step": round(ms_per_step, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": CONFIG4_TRAFFIC_BYTES if N == 100_000_000 else None,
-                     "kernel": "rows_kernel<u32x4, map16, fetch>", "kernel_ms": round(kern_ms, 4),
+                     "traffic": config4_traffic_bytes() if N == 100_000_000 else None,
+                     "kernel": "rows_kernel<u32x4, %s, fetch>" % ("map_flat" if hmap.layout() != "buckets" else "map8"),
+                     "kernel_ms": round(kern_ms, 4),
                      "bytes_per_launch": algo_bytes},
     })
     result["config"].update({"workload": "config 4: cache_fetch, %d x %d fp16 table pinned, %d rows cached, "
                              "Q=%d Zipf(1.1)" % (N, D, C, Q), "hit_rate": round(hit_rate, 4),
-                             "row_bytes": R, "queries_per_step": Q})
+                             "row_bytes": R, "queries_per_step": Q, "map_layout": hmap.layout()})
     extra = result["extra"]
     if args.headline_only:
         del host, cache, hmap
@@ -198,11 +212,33 @@ def bench_fetch(capi, args, result):
     t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qh, hmap), 30)
     a = algo_bytes / (t["median"] * 1e-3) / 1e9
     extra["fetch_all_hit"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "algorithmic_GBs": round(a, 1),
-                              "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 1)}
+                              "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 1),
+                              "map_layout": hmap.layout(),
+                              "note": "the configuration's own map: ids 0..C-1 -> slot = id, recognised as an id range"}
     tm = gpu_time_ms(lambda: capi.cache_fetch_with_mask(host, cache, qh, qh), 30)
     a = algo_bytes / (tm["median"] * 1e-3) / 1e9
     extra["fetch_all_hit_with_mask"] = {"ms": round(tm["median"], 4), "algorithmic_GBs": round(a, 1),
                                         "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
+    # The same all-hit batch through maps that do need a table: slots in arbitrary order over the same ids
+    # (direct table, one 4-byte load per row) and scattered ids (bucket table, one 128-byte bucket per probe).
+    # A random table read costs a whole 128-byte line whatever its size, so these move Q x (2R + 8 + 128)
+    # bytes for Q x (2R + 8) algorithmic ones: line_traffic_GBs is that real figure.
+    gq = torch.Generator(device="cuda").manual_seed(17)
+    ids = torch.arange(C, device="cuda")
+    slots = torch.randperm(C, device="cuda", generator=gq)
+    by_table = {}
+    for name, keys_t, req in (("direct_table", ids, qh), ("bucket_table_8B_slots", ids * 11 + 1, qh * 11 + 1),
+                              ("bucket_table_16B_slots", ids * 37 + (1 << 33), qh * 37 + (1 << 33))):
+        m = capi.CUCOStaticHashmap(keys_t, slots, 0.8)
+        assert torch.equal(capi.cache_fetch(host, cache, req[:4096], m), cache[slots[qh[:4096]]])
+        tt = gpu_time_ms(lambda: capi.cache_fetch(host, cache, req, m), 30)
+        a = algo_bytes / (tt["median"] * 1e-3) / 1e9
+        by_table[name] = {"ms": round(tt["median"], 4), "map_layout": m.layout(), "map_bytes": m.memory_usage(),
+                          "algorithmic_GBs": round(a, 1), "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4),
+                          "line_traffic_GBs": round(Q * (2 * R + 8 + 128) / tt["median"] / 1e6, 1)}
+        del m, keys_t, req
+    extra["fetch_all_hit_by_map_layout"] = by_table
+    del ids, slots
     # all-miss: uniform queries over the uncached ids, host-link bound
     qm = torch.randint(C, N, (Q,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
     t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qm, hmap), 10)
@@ -221,8 +257,12 @@ def bench_fetch(capi, args, result):
     t = gpu_time_ms(lambda: capi.cache_set(host, cache, sidx, upd, hmap), 30)
     assert torch.equal(capi.cache_fetch(host, cache, sidx, hmap), upd)
     a = ns * (2 * R + 8) / (t["median"] * 1e-3) / 1e9
+    # floor: the same bytes at the rate the 1,048,576-row all-hit fetch sustains (a launch four times shorter
+    # spends a larger share of its time filling and draining the chip)
     extra["cache_set_262144"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "algorithmic_GBs": round(a, 1),
-                                 "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
+                                 "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4),
+                                 "floor_ms_at_all_hit_fetch_rate": round(tm["median"] * ns / Q, 4),
+                                 "floor_ms_at_hbm_peak": round(ns * (2 * R + 8) / HBM_PEAK_GBS / 1e6, 4)}
 
     # scatter to the host table over the link (all misses): 262,144 uncached rows
     sm = torch.randperm(N - C, device="cuda", generator=torch.Generator(device="cuda").manual_seed(10))[:ns] + C
@@ -330,7 +370,11 @@ def bench_hashmap(capi, args, result):
         "query_ms": round(tq["median"], 4), "query_Mkeys_s": round(nq / tq["median"] / 1e3, 1),
         "query_algorithmic_GBs": round(nq * 32 / tq["median"] / 1e6, 1),
         "query_frac_hbm_peak": round(nq * 32 / tq["median"] / 1e6 / HBM_PEAK_GBS, 4),
-        "table_bytes": h.memory_usage()}
+        # what the memory system moves: a probe reads one whole 128-byte bucket line (FETCH_SIZE per launch in
+        # profiles/hashmap_sampling_kernels_pmc.md: 2,291 MB = nq x (128 + 8)), next to 8 B request + 8 B result
+        "query_line_traffic_GBs": round(nq * 144 / tq["median"] / 1e6, 1),
+        "query_line_traffic_frac_hbm_peak": round(nq * 144 / tq["median"] / 1e6 / HBM_PEAK_GBS, 4),
+        "table_bytes": h.memory_usage(), "map_layout": h.layout()}
     if not args.no_cpu:
         from oracle import oracle as orc
         k_np, v_np, r_np = keys.cpu().numpy(), vals.cpu().numpy(), req[: nq // 4].cpu().numpy()
@@ -343,6 +387,67 @@ def bench_hashmap(capi, args, result):
         result["extra"]["hashmap_config2"]["cpu_oracle"] = {
             "build_Mkeys_s": round(n / tbuild / 1e6, 2), "query_Mkeys_s": round(r_np.size / tquery / 1e6, 2),
             "cores": orc.num_threads(), "sample": "build 4,194,304 keys (1 thread); query 4,194,304 requests (OpenMP)"}
+
+
+def bench_hashmap_sweep(capi, args, result):
+    """Bulk query rate against the size of the bucket table (int64 keys, 16-byte slots, load factor 0.5):
+    where the probes are served from (the 4 MB L2 of each of the 8 XCDs, the 256 MB memory-side cache, HBM)."""
+    import torch
+    nq = 1 << 24
+    g = torch.Generator(device="cuda").manual_seed(1)
+    rows = []
+    for lg in range(14, 27):
+        n = 1 << lg
+        keys = (torch.randperm(1 << 27, device="cuda", generator=g)[:n] * 8191 + (1 << 34)).contiguous()
+        h = capi.CUCOStaticHashmap(keys, torch.arange(n, device="cuda"), 0.5)
+        req = keys[torch.randint(0, n, (nq,), device="cuda", generator=g)]
+        t = gpu_time_ms(lambda: h.query(req), 10)
+        rows.append({"keys": n, "table_MiB": round(h.memory_usage() / 2**20, 1), "query_ms": round(t["median"], 4),
+                     "Gkeys_s": round(nq / t["median"] / 1e6, 1),
+                     "line_traffic_GBs": round(nq * 144 / t["median"] / 1e6, 1)})
+        del h, req, keys
+    result["extra"]["hashmap_query_by_table_size"] = rows
+
+
+# ---------------------------------------------------------------------------
+# scans (cub_exclusiveSum / thrust_scan of the reference): 2 * n * element bytes against the HBM peak
+
+def bench_scan(capi, args, result):
+    import torch
+    from shmtensor_amd import cabi
+    lib = cabi.load()
+    n = 1 << 24
+    res = {}
+    a64 = torch.randint(0, 1000, (n,), device="cuda", dtype=torch.int64)
+    work = a64.clone()
+    tmp_bytes = lib.shmt_scan_tmp_bytes(n)
+    tmp = torch.empty(max(tmp_bytes, 1), dtype=torch.uint8, device="cuda")
+    stream = cabi.current_stream()
+    cabi.check(lib.shmt_exclusive_scan(work.data_ptr(), n, 8, tmp.data_ptr(), tmp_bytes, stream))
+    expect = torch.cumsum(a64, 0) - a64
+    assert torch.equal(work, expect), "exclusive scan differs from cumsum"
+    del expect
+
+    def ex64():     # in place: rescanning the scanned values costs the same
+        cabi.check(lib.shmt_exclusive_scan(work.data_ptr(), n, 8, tmp.data_ptr(), tmp_bytes, stream))
+    t = gpu_time_ms(ex64, 30)
+    res["exclusive_int64_16777216"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(2 * n * 8 / t["median"] / 1e6, 1),
+                                       "frac_hbm_peak": round(2 * n * 8 / t["median"] / 1e6 / HBM_PEAK_GBS, 4)}
+    a32 = torch.randint(0, 100, (n,), device="cuda", dtype=torch.int32)
+    t = gpu_time_ms(lambda: capi.thrust_scan(a32), 30)
+    res["thrust_scan_int32_16777216"] = {"ms": round(t["median"], 4), "algorithmic_GBs": round(2 * n * 4 / t["median"] / 1e6, 1),
+                                         "frac_hbm_peak": round(2 * n * 4 / t["median"] / 1e6 / HBM_PEAK_GBS, 4)}
+    tt = gpu_time_ms(lambda: torch.cumsum(a64, 0), 10)
+    res["torch_cumsum_int64_ms"] = round(tt["median"], 4)
+    if not args.no_cpu:
+        import numpy as np
+        from oracle import oracle as orc
+        a_np = a64.cpu().numpy()
+        t0 = time.perf_counter()
+        orc.exclusive_scan(a_np)
+        res["cpu_baseline"] = {"ms": round((time.perf_counter() - t0) * 1e3, 2), "cores": 1, "kind": "port",
+                               "sample": "one exclusive scan of the same 16,777,216 int64 (oracle, sequential, incl. a copy)"}
+    result["extra"]["scan"] = res
 
 
 # ---------------------------------------------------------------------------
@@ -472,19 +577,35 @@ def bench_sampling(capi, args, result):
         from oracle import oracle as orc
         ip, ix = indptr.numpy(), indices.numpy().astype(np.int64)
         nb_cpu = min(nbatch, 20)
-        t0 = time.perf_counter()
-        cpu_edges = 0
-        for b in range(nb_cpu):
-            seeds = seed_batches[b].cpu().numpy()
-            for hop, k in enumerate(reversed(fanouts)):
-                sp, si = orc.sample(ip, ix, seeds, k, False, seed=7777 + b, stream=hop, algo="reservoir")
-                uniq, _ = orc.relabel([seeds, si])
-                cpu_edges += si.size
-                seeds = uniq
-        cpu_t = time.perf_counter() - t0
-        res["cpu_baseline"] = {"sampled_edges_per_s": round(cpu_edges / cpu_t, 1), "cores": orc.num_threads(),
-                               "kind": "port", "sample": "%d batches, Algorithm-R sampler + hash relabel (oracle, OpenMP)" % nb_cpu}
-        res["speedup_vs_cpu"] = round((edges / gpu_t) / (cpu_edges / cpu_t), 2)
+
+        def cpu_pipeline(sampler, relabeler):
+            t0 = time.perf_counter()
+            total = 0
+            for b in range(nb_cpu):
+                seeds = seed_batches[b].cpu().numpy()
+                for hop, k in enumerate(reversed(fanouts)):
+                    sp, si = orc.sample(ip, ix, seeds, k, False, seed=7777 + b, stream=hop, algo=sampler)
+                    uniq, _ = orc.relabel([seeds, si], algo=relabeler)
+                    total += si.size
+                    seeds = uniq
+            return total, time.perf_counter() - t0
+
+        # (a) the reference's algorithms on host cores: Algorithm R (O(degree) draws per seed) and the four-pass
+        #     relabel over its low-bit hash table; (b) what a CPU programmer would write for the same contract:
+        #     Floyd's O(k) subset selection and a one-sweep relabel with a mixed hash. The speed-up is quoted
+        #     against the faster of the two.
+        e_ref, t_ref = cpu_pipeline("reservoir", "passes")
+        e_fast, t_fast = cpu_pipeline("floyd", "sweep")
+        res["cpu_baseline_reference_algorithms"] = {
+            "sampled_edges_per_s": round(e_ref / t_ref, 1), "cores": orc.num_threads(), "kind": "port",
+            "sample": "%d batches, Algorithm-R sampler + four-pass low-bit-hash relabel (oracle, OpenMP)" % nb_cpu}
+        res["cpu_baseline"] = {
+            "sampled_edges_per_s": round(e_fast / t_fast, 1), "cores": orc.num_threads(), "kind": "port",
+            "sample": "%d batches, Floyd O(k) sampler (OpenMP over seeds) + one-sweep mixed-hash relabel "
+                      "(sequential) (oracle)" % nb_cpu}
+        best = max(e_ref / t_ref, e_fast / t_fast)
+        res["speedup_vs_cpu"] = round((edges / gpu_t) / best, 2)
+        res["speedup_vs_cpu_reference_algorithms"] = round((edges / gpu_t) / (e_ref / t_ref), 2)
     result["extra"]["sampling_config3"] = res
 
 
@@ -620,7 +741,44 @@ def bench_e2e(capi, args, result):
     w0 = time.perf_counter()
     epoch()
     wall_pipe = time.perf_counter() - w0
+    cpu = None
+    if not args.no_cpu:
+        import numpy as np
+        from oracle import oracle as orc
+        ip, ix = indptr.numpy(), indices.numpy().astype(np.int64)
+        feats_np = feats.numpy()
+        nb_cpu = min(nbatch, 2)
+        t_samp = t_fetch = 0.0
+        c_edges = c_nodes = 0
+        for b in range(nb_cpu):
+            seeds = batches[b].cpu().numpy()
+            t0 = time.perf_counter()
+            for hop, k in enumerate(reversed(fanouts)):
+                sp, si = orc.sample(ip, ix, seeds, k, False, seed=7777 + b, stream=hop, algo="floyd")
+                uniq, _ = orc.relabel([seeds, si], algo="sweep")
+                c_edges += si.size
+                seeds = uniq
+            t1 = time.perf_counter()
+            rows = orc.fetch(feats_np, None, seeds)
+            t2 = time.perf_counter()
+            t_samp += t1 - t0
+            t_fetch += t2 - t1
+            c_nodes += seeds.size
+            del rows
+        idx_t = torch.from_numpy(seeds)
+        t0 = time.perf_counter()
+        torch.index_select(feats, 0, idx_t)
+        t_torch = time.perf_counter() - t0
+        cpu = {"cores": orc.num_threads(), "kind": "port",
+               "sample": "%d batches: Floyd sampler (OpenMP) + one-sweep relabel, then an OpenMP gather of the input "
+                         "nodes' rows from the same host table (oracle)" % nb_cpu,
+               "sample_relabel_ms": round(t_samp * 1e3 / nb_cpu, 2), "fetch_ms": round(t_fetch * 1e3 / nb_cpu, 2),
+               "batch_ms": round((t_samp + t_fetch) * 1e3 / nb_cpu, 2),
+               "sampled_edges_per_s": round(c_edges / t_samp, 1),
+               "fetch_payload_GBs": round(c_nodes * D * 4 / t_fetch / 1e9, 2),
+               "torch_index_select_ms": round(t_torch * 1e3, 2), "torch_threads": torch.get_num_threads()}
     result["extra"]["e2e_config5"] = {
+        "cpu_baseline": cpu,
         "graph": "R-MAT scale %d ef 16 symmetrised: %d nodes, %d edges; top 20 %% adjacency cached; features %d x %d "
                  "f32 pinned, top-degree 25 %% cached" % (args.e2e_scale, n, indices.numel(), n, D),
         "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
@@ -657,7 +815,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workloads", default="fetch,hashmap,sampling,e2e")
+    ap.add_argument("--workloads", default="fetch,hashmap,scan,sampling,e2e")
     ap.add_argument("--fetch-rows", type=int, default=100_000_000)
     ap.add_argument("--sampling-scale", type=int, default=21)
     ap.add_argument("--sampling-batches", type=int, default=50)
@@ -696,6 +854,10 @@ def main():
     if "hashmap" in todo:
         bench_hashmap(capi, args, result)
         torch.cuda.empty_cache()
+    if "hashmap_sweep" in todo:
+        bench_hashmap_sweep(capi, args, result)
+    if "scan" in todo:
+        bench_scan(capi, args, result)
     if "granularity" in todo:
         probe_granularity(capi, args, result)
     if "sampling" in todo:

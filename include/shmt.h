@@ -85,8 +85,8 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys,
 /* Build with a layout chosen from the keys. Node ids are small dense
  * integers, so beside the general bucket table two flat forms exist:
  *   SHMT_MAP_DIRECT  keys lie in [lo, lo + span) and an int32 table
- *                    value[key - lo] is no larger than the bucket table would
- *                    be: one 4-byte load per lookup;
+ *                    value[key - lo] is at most twice as large as the bucket
+ *                    table would be: one 4-byte load per lookup;
  *   SHMT_MAP_RANGE   the keys are exactly lo .. lo + span - 1 and every value
  *                    is key + delta (the cache holds an id range, as in
  *                    re-numbered graphs): lookups are arithmetic, no table;

@@ -299,6 +299,36 @@ ORC_EXPORT int64_t orc_relabel(const int64_t *total, int64_t N, int64_t *unique,
   return tot;
 }
 
+/* The same contract as a CPU programmer would write it (not a restatement of
+ * the reference's kernel structure; used as the faster of the two CPU
+ * baselines): one sequential sweep, open addressing with a mixed hash, a new
+ * id is appended to `unique` the first time it is met. First-occurrence order
+ * falls out of the sweep order, so no index table, no counting pass and no
+ * scan are needed (src/tensor_relabel.cu:127-130, 206-208 for the contract). */
+ORC_EXPORT int64_t orc_relabel_sweep(const int64_t *total, int64_t N, int64_t *unique, int64_t *labels) {
+  if (N == 0) return 0;
+  uint64_t cap = 16;
+  while (cap < (uint64_t)N * 2) cap <<= 1;
+  int64_t *kt = (int64_t *)malloc(sizeof(int64_t) * cap);
+  int64_t *vt = (int64_t *)malloc(sizeof(int64_t) * cap);
+  memset(kt, 0xff, sizeof(int64_t) * cap); /* -1: empty */
+  int64_t count = 0;
+  for (int64_t i = 0; i < N; ++i) {
+    const int64_t key = total[i];
+    uint64_t pos = mix64((uint64_t)key) & (cap - 1);
+    while (kt[pos] != -1 && kt[pos] != key) pos = (pos + 1) & (cap - 1);
+    if (kt[pos] == -1) {
+      kt[pos] = key;
+      vt[pos] = count;
+      unique[count++] = key;
+    }
+    labels[i] = vt[pos];
+  }
+  free(kt);
+  free(vt);
+  return count;
+}
+
 /* ------------------------------------------------------------------ */
 /* Philox4x32-10 (Random123), the generator of the new sampler. The reference
  * uses cuRAND's Philox4_32_10 state (src/cache_graph_sampling.cu:105-107),

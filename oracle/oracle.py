@@ -46,6 +46,8 @@ def lib():
         L.orc_inclusive_scan_i32.argtypes = [_vp, _i64]
         L.orc_relabel.restype = _i64
         L.orc_relabel.argtypes = [_vp, _i64, _vp, _vp]
+        L.orc_relabel_sweep.restype = _i64
+        L.orc_relabel_sweep.argtypes = [_vp, _i64, _vp, _vp]
         L.orc_philox4x32_10.argtypes = [_vp, _vp, _vp]
         L.orc_sample_counts.restype = _i64
         L.orc_sample_counts.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _vp]
@@ -163,15 +165,18 @@ def inclusive_scan_i32(a):
     return a
 
 
-def relabel(tensors):
+def relabel(tensors, algo="passes"):
     """tensor_relabel: src/tensor_relabel.cu:125-209. Returns (unique, [labels...])
-    with the dtype torch.cat would give (int64 if any input is int64)."""
+    with the dtype torch.cat would give (int64 if any input is int64). algo: "passes"
+    (the reference's four parallel passes over its low-bit hash table, OpenMP) or
+    "sweep" (one sequential sweep with a mixed hash: the plain CPU way, same results)."""
     tensors = [_ids(t) for t in tensors]
     dt = np.result_type(*[t.dtype for t in tensors]) if tensors else np.int64
     total = _i64a(np.concatenate(tensors)) if tensors else np.zeros(0, np.int64)
     unique = np.empty(total.size, np.int64)
     labels = np.empty(total.size, np.int64)
-    u = lib().orc_relabel(_p(total), total.size, _p(unique), _p(labels))
+    fn = {"passes": lib().orc_relabel, "sweep": lib().orc_relabel_sweep}[algo]
+    u = fn(_p(total), total.size, _p(unique), _p(labels))
     out, off = [], 0
     for t in tensors:
         out.append(labels[off:off + t.size].astype(dt))

@@ -348,8 +348,9 @@ int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_byt
       return SHMT_OK;
     }
   }
-  // direct table when it is no larger than the bucket table would be
-  if (vals32 && span * 4 <= layout->table_bytes) {
+  // direct table while it stays within twice the bucket table's size (ids up to 8 times as many as
+  // keys when both fit 32 bits): one load per lookup instead of a cooperative probe sequence
+  if (vals32 && span * 4 <= 2 * layout->table_bytes) {
     layout->kind = SHMT_MAP_DIRECT;
     layout->slot_bytes = 4;
     layout->lo = st.kmin;

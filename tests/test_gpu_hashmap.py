@@ -159,7 +159,7 @@ def test_layouts_answer_like_a_dict(capi, oracle, kd, vd, case):
         keys = rng.choice(3 * n, size=n, replace=False) + 12345
         vals = np.arange(n)
         expect_layout = "direct"
-    elif case == "direct_too_sparse":                # 1 id in 20: the bucket table is smaller
+    elif case == "direct_too_sparse":                # 1 id in 20: the bucket table is much smaller
         keys = rng.choice(20 * n, size=n, replace=False)
         vals = np.arange(n)
         expect_layout = "buckets"

@@ -113,18 +113,20 @@ def _relabel_closed_form(arrays):
     return list(first.keys()), [first[x] for x in total]
 
 
-def test_relabel_reference_kat(oracle):
+@pytest.mark.parametrize("algo", ["passes", "sweep"])
+def test_relabel_reference_kat(oracle, algo):
     g = load_golden("relabel_kat.json")
-    u, labels = oracle.relabel([np.array(x) for x in g["inputs"]])
+    u, labels = oracle.relabel([np.array(x) for x in g["inputs"]], algo=algo)
     assert u.tolist() == g["unique"]
     assert [l.tolist() for l in labels] == g["labels"]
 
 
+@pytest.mark.parametrize("algo", ["passes", "sweep"])
 @pytest.mark.parametrize("n", [1, 2, 7, 8, 9, 255, 256, 257, 5000])
-def test_relabel_closed_form(oracle, n):
+def test_relabel_closed_form(oracle, n, algo):
     a = RNG.integers(0, max(2, n // 2), size=n)
     b = RNG.integers(2**31, 2**31 + max(2, n // 2), size=n // 2 + 1)   # ids >= 2^31
-    u, labels = oracle.relabel([a, b])
+    u, labels = oracle.relabel([a, b], algo=algo)
     eu, el = _relabel_closed_form([a, b])
     assert u.tolist() == eu
     assert np.concatenate(labels).tolist() == el
