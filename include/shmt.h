@@ -209,15 +209,16 @@ int shmt_inclusive_scan_i32(void *data, int64_t len, void *tmp,
  * cub_exclusiveSum allocates its temporary storage on every call,
  * src/tensor_relabel.cu:15-25); it is for callers that cannot allocate:
  * code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc. The tile partials live in a 1 MiB array that is part of the
- * library's code object (one copy per GPU, held until the process ends), so
+ * hipMalloc. The tile counter and tile words live in a 256 KiB array that is
+ * part of the library's code object (one copy per GPU, held until the process
+ * ends), so
  * len is limited to SHMT_SCAN_NOALLOC_MAX_LEN elements; longer inputs are
  * rejected with SHMT_EINVAL. Same results as shmt_exclusive_scan. The first
  * call on a device looks up the array's device address (a call with len = 0
  * does only that and can serve as set-up before a capture). All calls on one
  * GPU share the array: calls that overlap on one GPU (different streams
  * without ordering between them) race; calls on one stream, or ordered by
- * events, are safe, and nothing needs clearing between calls.              */
+ * events, are safe (every call clears what it uses before it scans).       */
 #define SHMT_SCAN_NOALLOC_MAX_LEN (268435456ll)
 int shmt_exclusive_scan_noalloc(void *data, int64_t len, int elem_bytes,
                                 void *stream);

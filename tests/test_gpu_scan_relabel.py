@@ -43,6 +43,32 @@ def test_exclusive_scan_c_abi(cabi, oracle, bytes_, n):
     assert np.array_equal(t.cpu().numpy(), oracle.exclusive_scan(a))
 
 
+@pytest.mark.parametrize("bytes_", [4, 8])
+def test_single_pass_scan_tile_edges_and_unaligned_data(cabi, oracle, bytes_):
+    """Inputs beyond one workgroup are scanned in one pass over 128 KiB tiles (16,384 int64 / 32,768 int32
+    elements) that look back at each other: lengths on and around tile boundaries, several hundred tiles,
+    and a data pointer that is not 16-byte aligned (element-wise loads instead of vector loads)."""
+    lib = cabi.load()
+    dt = np.int32 if bytes_ == 4 else np.int64
+    tile = 131072 // bytes_
+    rng = np.random.default_rng(bytes_)
+    for n in (65_537, tile * 3 - 1, tile * 3, tile * 3 + 1, tile * 64, tile * 65 + 5, tile * 700 + 12345):
+        for shift in (0, 1):                                        # shift 1: data starts bytes_ past a 16-byte boundary
+            a = rng.integers(0, 2**29 if bytes_ == 4 else 2**60, size=n).astype(dt)      # sums wrap around
+            buf = torch.zeros(n + 4, dtype=torch.int32 if bytes_ == 4 else torch.int64).cuda()
+            t = buf[shift:shift + n]
+            t.copy_(torch.from_numpy(a))
+            tmp_bytes = lib.shmt_scan_tmp_bytes(n)
+            tmp = torch.empty(tmp_bytes, dtype=torch.uint8).cuda()
+            cabi.check(lib.shmt_exclusive_scan(t.data_ptr(), n, bytes_, tmp.data_ptr(), tmp_bytes,
+                                               cabi.current_stream()))
+            assert np.array_equal(t.cpu().numpy(), oracle.exclusive_scan(a)), (n, shift)
+            assert int(buf[shift + n]) == 0 and (shift == 0 or int(buf[0]) == 0)        # nothing written outside
+    small = torch.empty(8, dtype=torch.uint8).cuda()
+    big = torch.zeros(100_000, dtype=torch.int64).cuda()
+    assert lib.shmt_exclusive_scan(big.data_ptr(), 100_000, 8, small.data_ptr(), 8, cabi.current_stream()) == -4
+
+
 def test_relabel_reference_kat(capi):
     g = load_golden("relabel_kat.json")
     u, labels = capi.tensor_relabel([torch.tensor(x).cuda() for x in g["inputs"]])

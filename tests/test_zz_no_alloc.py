@@ -1,5 +1,5 @@
 """The entry point that allocates nothing: shmt_exclusive_scan_noalloc keeps its
-tile partials in an array inside the library's code object. Called through the
+tile counter and tile words in an array inside the library's code object. Called through the
 C ABI and checked bit for bit against shmt_exclusive_scan (caller-provided
 workspace) and the CPU oracle, on two calls in a row, the second on a smaller
 input."""
@@ -41,8 +41,8 @@ def test_no_alloc_scan_equals_workspace_scan_twice_in_a_row(cabi, oracle):
     # set-up call: looks up the workspace's device address, moves nothing
     cabi.check(lib.shmt_exclusive_scan_noalloc(None, 0, 8, cabi.current_stream()))
     rng = np.random.default_rng(11)
-    # first call: 5,000,001 int64 (2,442 tile partials); second, smaller: 300,001 int32 (147 partials),
-    # which finds the first call's partials in the workspace; third: one workgroup, no partials at all
+    # first call: 5,000,001 int64 (306 tiles of 16,384 elements); second, smaller: 300,001 int32 (10 tiles of
+    # 32,768), which finds the first call's tile words in the workspace; third: one workgroup, no workspace use
     for n, dt in ((5_000_001, np.int64), (300_001, np.int32), (4_097, np.int64)):
         hi = 2**61 if dt is np.int64 else 2**30                  # sums wrap around
         a = rng.integers(0, hi, size=n).astype(dt)
