@@ -23,6 +23,8 @@ ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
 HIP_SOURCES = ["hashmap.hip", "fetch.hip", "scan.hip", "relabel.hip", "sample.hip", "misc.hip",
                "host_mem.hip", "errors.cc"]
 
+MODULE_SOURCES = ["module.cc", "batch_driver.cc", "batch_sampler.cc", "host_tensors.cc"]
+
 # Packed-FP32 instruction selection is switched off for every HIP translation
 # unit (the kernels here do no floating-point arithmetic at all, rows are
 # moved as raw bytes).
@@ -82,8 +84,8 @@ def build_module():
         cmd += ["-isystem", inc]
     cmd += ["-isystem", "/opt/rocm/include", "-I" + sysconfig.get_paths()["include"],
             "-I" + INCLUDE]
-    cmd += [os.path.join(CSRC, "pybind", "module.cc"), os.path.join(CSRC, "pybind", "host_tensors.cc"),
-            "-o", module_path(),
+    cmd += [os.path.join(CSRC, "pybind", f) for f in MODULE_SOURCES]
+    cmd += ["-o", module_path(),
             "-L" + tlib, "-L" + LIB_DIR, "-lshmt", "-ltorch", "-ltorch_cpu", "-ltorch_python",
             "-lc10", "-lc10_hip", "-ltorch_hip",
             "-Wl,-rpath,$ORIGIN/lib", "-Wl,-rpath," + tlib]
