@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void hashmap_insert_kernel(
 struct KeyStats {
   long long kmin, kmax, vmin, vmax;
   unsigned long long not_affine;  // != 0: value - key differs between pairs
-  unsigned long long repeats;     // range candidates only: keys seen more than once
+  unsigned long long distinct;    // range candidates only: number of different keys
 };
 
 __global__ void stats_init_kernel(KeyStats *st) {
@@ -159,7 +159,7 @@ __global__ void stats_init_kernel(KeyStats *st) {
   st->vmin = INT64_MAX;
   st->vmax = INT64_MIN;
   st->not_affine = 0;
-  st->repeats = 0;
+  st->distinct = 0;
 }
 
 __device__ __forceinline__ int64_t wave_min64(int64_t v) {
@@ -207,20 +207,27 @@ __global__ __launch_bounds__(256) void key_stats_kernel(const void *keys, const 
   }
 }
 
-// Range candidates (as many pairs as ids between the extrema): every key sets
-// its bit; a bit found set already is a repeated key, and then some id of the
-// range is missing.
-__global__ __launch_bounds__(256) void key_repeats_kernel(const void *keys, int64_t n, int key_bytes,
-                                                          int64_t lo, uint32_t *bits, KeyStats *st) {
+// Range candidates (as many pairs as ids between the extrema): every key marks
+// its byte (plain stores: racing writers all write the same value), then the
+// marked bytes are counted; fewer marks than pairs means a key repeats, and
+// then some id of the range is missing.
+__global__ __launch_bounds__(256) void key_mark_kernel(const void *keys, int64_t n, int key_bytes,
+                                                       int64_t lo, uint8_t *seen) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  bool repeat = false;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
     const uint64_t off = static_cast<uint64_t>(load_int(keys, i, key_bytes) - lo);
-    if (off >= static_cast<uint64_t>(n)) continue;  // cannot happen for a true candidate
-    const uint32_t bit = 1u << (off & 31);
-    repeat |= (atomicOr(&bits[off >> 5], bit) & bit) != 0;
+    if (off < static_cast<uint64_t>(n)) seen[off] = 1;  // always true for a genuine candidate
   }
-  if (__builtin_amdgcn_ballot_w64(repeat) != 0 && lane_id() == 0) atomicOr(&st->repeats, 1ull);
+}
+
+__global__ __launch_bounds__(256) void key_count_marks_kernel(const uint32_t *seen_words, int64_t nwords,
+                                                              KeyStats *st) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  uint32_t mine = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nwords; i += stride)
+    mine += __builtin_popcount(seen_words[i]);  // a marked byte is 0x01
+  const uint32_t wave = wave_last(wave_inclusive_scan(mine));
+  if (lane_id() == 0 && wave) atomicAdd(&st->distinct, static_cast<unsigned long long>(wave));
 }
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *p, int64_t n) {
@@ -283,7 +290,7 @@ int64_t shmt_hashmap_table_bytes(int64_t n, double load_factor, int key_bytes, i
 
 int64_t shmt_hashmap_plan_scratch_bytes(int64_t n) {
   if (n < 0) return -1;
-  return 256 + ((n + 31) / 32) * 4;
+  return 256 + ((n + 3) / 4) * 4;
 }
 
 int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_bytes, int val_bytes,
@@ -311,7 +318,7 @@ int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_byt
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "shmt_hashmap_plan: scratch must be 16-byte aligned");
   hipStream_t s = as_stream(stream);
   KeyStats *dev_stats = static_cast<KeyStats *>(scratch);
-  uint32_t *bits = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + 256);
+  uint32_t *marks = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + 256);  // one byte per id
   hipLaunchKernelGGL(stats_init_kernel, dim3(1), dim3(1), 0, s, dev_stats);
   hipLaunchKernelGGL(key_stats_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, vals, n,
                      key_bytes, val_bytes, dev_stats);
@@ -331,14 +338,16 @@ int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_byt
   const int64_t span = st.kmax - st.kmin + 1;
   if (span == n && !st.not_affine) {
     // as many pairs as ids in the range and one offset for all: a range map unless a key repeats
-    const int64_t words = (n + 31) / 32;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(words, 256 * 4)), dim3(256), 0, s, bits, words);
-    hipLaunchKernelGGL(key_repeats_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, n,
-                       key_bytes, static_cast<int64_t>(st.kmin), bits, dev_stats);
+    const int64_t words = (n + 3) / 4;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(words, 256 * 4)), dim3(256), 0, s, marks, words);
+    hipLaunchKernelGGL(key_mark_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, n, key_bytes,
+                       static_cast<int64_t>(st.kmin), reinterpret_cast<uint8_t *>(marks));
+    hipLaunchKernelGGL(key_count_marks_kernel, dim3(grid_for(words, 256 * 8, 256 * 8)), dim3(256), 0, s, marks,
+                       words, dev_stats);
     SHMT_LAUNCH_CHECK();
     SHMT_HIP(hipMemcpyAsync(&st, dev_stats, sizeof(st), hipMemcpyDeviceToHost, s));
     SHMT_HIP(hipStreamSynchronize(s));
-    if (!st.repeats) {
+    if (st.distinct == static_cast<unsigned long long>(n)) {
       layout->kind = SHMT_MAP_RANGE;
       layout->slot_bytes = 0;
       layout->lo = st.kmin;

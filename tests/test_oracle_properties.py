@@ -81,3 +81,26 @@ def test_sampling_contract(oracle, degs, k, replace, seed, algo, data):
         cache = (gp, gi, oracle.Hashmap(rows, np.arange(rows.size), 0.8))
         sp2, si2 = oracle.sample(indptr, indices, seeds, k, replace, cache=cache, seed=seed, algo=algo)
         assert np.array_equal(sp, sp2) and np.array_equal(si, si2)
+
+
+def test_zipf_generator_follows_the_exact_law():
+    """The benchmark's query stream: ranks must follow P(r) ~ (r + 1)^-s exactly at the head (where almost
+    all of the mass and all of the repetition is) and within sampling noise in the tail. Chi-square over the
+    first 30 ranks one by one plus geometric buckets up to the last rank, against pmf values summed directly."""
+    import torch
+    from shmtensor_amd.synthetic import zipf_ranks
+    for num_items, s, head in ((200_000, 1.1, 1 << 20), (200_000, 1.1, 1000), (50_000, 0.8, 64)):
+        n = 2_000_000
+        r = zipf_ranks(n, num_items, s, seed=3, device="cpu", head=head).numpy()
+        assert r.min() >= 0 and r.max() < num_items
+        pmf = np.arange(1, num_items + 1, dtype=np.float64) ** -s
+        pmf /= pmf.sum()
+        edges = list(range(0, 31)) + [int(x) for x in np.unique(np.geomspace(31, num_items, 40).astype(np.int64))]
+        edges[-1] = num_items
+        observed = np.histogram(r, bins=edges)[0]
+        expected = np.add.reduceat(pmf, edges[:-1]) * n
+        chi2 = ((observed - expected) ** 2 / expected).sum()
+        dof = len(edges) - 2
+        assert chi2 < dof + 6 * np.sqrt(2 * dof), (num_items, s, head, chi2, dof)
+        # rank 0 alone: the continuous approximation that the exact head replaces is off by +11 % here
+        assert abs(observed[0] / n - pmf[0]) < 4 * np.sqrt(pmf[0] / n)
