@@ -5,6 +5,9 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "common.h"
 #include "hashmap.h"
 #include "hashmap_dev.h"
@@ -153,14 +156,9 @@ struct KeyStats {
   unsigned long long distinct;    // range candidates only: number of different keys
 };
 
-__global__ void stats_init_kernel(KeyStats *st) {
-  st->kmin = INT64_MAX;
-  st->kmax = INT64_MIN;
-  st->vmin = INT64_MAX;
-  st->vmax = INT64_MIN;
-  st->not_affine = 0;
-  st->distinct = 0;
-}
+constexpr int kStatBlocks = 1024;          // workgroups of a sweep, each leaving one partial result
+constexpr int64_t kStatPartialsOff = 256;  // scratch layout: header, partials, then one mark byte per id
+constexpr int64_t kStatMarksOff = kStatPartialsOff + ((kStatBlocks * 48 + 255) & ~255);
 
 __device__ __forceinline__ int64_t wave_min64(int64_t v) {
 #pragma unroll
@@ -179,32 +177,106 @@ __device__ __forceinline__ int64_t wave_max64(int64_t v) {
   return v;
 }
 
+// Combines the calling workgroup's per-thread values into one KeyStats, valid
+// in thread 0 (no atomics: thousands of them on a handful of addresses would
+// cost more than the sweep).
+__device__ __forceinline__ KeyStats block_combine(KeyStats mine) {
+  __shared__ KeyStats per_wave[256 / kWave];
+  mine.kmin = wave_min64(mine.kmin);
+  mine.kmax = wave_max64(mine.kmax);
+  mine.vmin = wave_min64(mine.vmin);
+  mine.vmax = wave_max64(mine.vmax);
+  mine.not_affine = __builtin_amdgcn_ballot_w64(mine.not_affine != 0) != 0;
+  mine.distinct = wave_last(wave_inclusive_scan(static_cast<uint64_t>(mine.distinct)));
+  if (lane_id() == 0) per_wave[threadIdx.x / kWave] = mine;
+  __syncthreads();
+  KeyStats all = per_wave[0];
+  if (threadIdx.x == 0) {
+    for (unsigned w = 1; w < blockDim.x / kWave; ++w) {
+      const KeyStats o = per_wave[w];
+      all.kmin = o.kmin < all.kmin ? o.kmin : all.kmin;
+      all.kmax = o.kmax > all.kmax ? o.kmax : all.kmax;
+      all.vmin = o.vmin < all.vmin ? o.vmin : all.vmin;
+      all.vmax = o.vmax > all.vmax ? o.vmax : all.vmax;
+      all.not_affine |= o.not_affine;
+      all.distinct += o.distinct;
+    }
+  }
+  return all;
+}
+
+__device__ __forceinline__ KeyStats neutral_stats() {
+  return KeyStats{INT64_MAX, INT64_MIN, INT64_MAX, INT64_MIN, 0, 0};
+}
+
 __global__ __launch_bounds__(256) void key_stats_kernel(const void *keys, const void *vals, int64_t n,
-                                                        int key_bytes, int val_bytes, KeyStats *st) {
+                                                        int key_bytes, int val_bytes, KeyStats *partials) {
   const int64_t delta0 = load_int(vals, 0, val_bytes) - load_int(keys, 0, key_bytes);
-  int64_t kmin = INT64_MAX, kmax = INT64_MIN, vmin = INT64_MAX, vmax = INT64_MIN;
-  bool off = false;
+  KeyStats mine = neutral_stats();
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
     const int64_t k = load_int(keys, i, key_bytes), v = load_int(vals, i, val_bytes);
-    kmin = k < kmin ? k : kmin;
-    kmax = k > kmax ? k : kmax;
-    vmin = v < vmin ? v : vmin;
-    vmax = v > vmax ? v : vmax;
-    off |= (v - k != delta0);
+    mine.kmin = k < mine.kmin ? k : mine.kmin;
+    mine.kmax = k > mine.kmax ? k : mine.kmax;
+    mine.vmin = v < mine.vmin ? v : mine.vmin;
+    mine.vmax = v > mine.vmax ? v : mine.vmax;
+    mine.not_affine |= (v - k != delta0);
   }
-  kmin = wave_min64(kmin);
-  kmax = wave_max64(kmax);
-  vmin = wave_min64(vmin);
-  vmax = wave_max64(vmax);
-  const bool any_off = __builtin_amdgcn_ballot_w64(off) != 0;
-  if (lane_id() == 0) {
-    atomicMin(&st->kmin, static_cast<long long>(kmin));
-    atomicMax(&st->kmax, static_cast<long long>(kmax));
-    atomicMin(&st->vmin, static_cast<long long>(vmin));
-    atomicMax(&st->vmax, static_cast<long long>(vmax));
-    if (any_off) atomicOr(&st->not_affine, 1ull);
+  const KeyStats all = block_combine(mine);
+  if (threadIdx.x == 0) partials[blockIdx.x] = all;
+}
+
+// One workgroup merges the partial results of a sweep and hands the outcome to
+// the host through a slot of pinned host memory (a device-to-host copy into
+// pageable memory would go through the runtime's staging path).
+__global__ __launch_bounds__(256) void stats_merge_kernel(const KeyStats *partials, int nb, KeyStats *host_slot) {
+  KeyStats mine = neutral_stats();
+  for (int b = threadIdx.x; b < nb; b += blockDim.x) {
+    const KeyStats o = partials[b];
+    mine.kmin = o.kmin < mine.kmin ? o.kmin : mine.kmin;
+    mine.kmax = o.kmax > mine.kmax ? o.kmax : mine.kmax;
+    mine.vmin = o.vmin < mine.vmin ? o.vmin : mine.vmin;
+    mine.vmax = o.vmax > mine.vmax ? o.vmax : mine.vmax;
+    mine.not_affine |= o.not_affine;
+    mine.distinct += o.distinct;
   }
+  const KeyStats all = block_combine(mine);
+  if (threadIdx.x == 0) *host_slot = all;
+}
+
+constexpr int kStatSlots = 16;  // concurrent map builds each take their own
+static std::mutex g_stat_mutex;
+static KeyStats *g_stat_slots = nullptr;      // pinned host memory
+static KeyStats *g_stat_slots_dev = nullptr;  // its device alias
+static std::atomic<unsigned> g_stat_next{0};
+
+static int stat_slot(KeyStats **host, KeyStats **dev) {
+  {
+    std::lock_guard<std::mutex> lock(g_stat_mutex);
+    if (g_stat_slots == nullptr) {
+      void *p = nullptr, *d = nullptr;
+      SHMT_HIP(hipHostMalloc(&p, kStatSlots * sizeof(KeyStats), hipHostMallocMapped));
+      SHMT_HIP(hipHostGetDevicePointer(&d, p, 0));
+      g_stat_slots = static_cast<KeyStats *>(p);
+      g_stat_slots_dev = static_cast<KeyStats *>(d);
+    }
+  }
+  const unsigned i = g_stat_next.fetch_add(1) % kStatSlots;
+  *host = g_stat_slots + i;
+  *dev = g_stat_slots_dev + i;
+  return SHMT_OK;
+}
+
+// Merge the partial results of a sweep, hand them to the host and wait for them.
+static int read_stats(const KeyStats *partials, int nb, KeyStats *out, hipStream_t s) {
+  KeyStats *host = nullptr, *host_dev = nullptr;
+  int rc = stat_slot(&host, &host_dev);
+  if (rc) return rc;
+  hipLaunchKernelGGL(stats_merge_kernel, dim3(1), dim3(256), 0, s, partials, nb, host_dev);
+  SHMT_LAUNCH_CHECK();
+  SHMT_HIP(hipStreamSynchronize(s));
+  *out = *host;
+  return SHMT_OK;
 }
 
 // Range candidates (as many pairs as ids between the extrema): every key marks
@@ -221,13 +293,13 @@ __global__ __launch_bounds__(256) void key_mark_kernel(const void *keys, int64_t
 }
 
 __global__ __launch_bounds__(256) void key_count_marks_kernel(const uint32_t *seen_words, int64_t nwords,
-                                                              KeyStats *st) {
+                                                              KeyStats *partials) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  uint32_t mine = 0;
+  KeyStats mine = neutral_stats();
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nwords; i += stride)
-    mine += __builtin_popcount(seen_words[i]);  // a marked byte is 0x01
-  const uint32_t wave = wave_last(wave_inclusive_scan(mine));
-  if (lane_id() == 0 && wave) atomicAdd(&st->distinct, static_cast<unsigned long long>(wave));
+    mine.distinct += __builtin_popcount(seen_words[i]);  // a marked byte is 0x01
+  const KeyStats all = block_combine(mine);
+  if (threadIdx.x == 0) partials[blockIdx.x] = all;
 }
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *p, int64_t n) {
@@ -290,7 +362,7 @@ int64_t shmt_hashmap_table_bytes(int64_t n, double load_factor, int key_bytes, i
 
 int64_t shmt_hashmap_plan_scratch_bytes(int64_t n) {
   if (n < 0) return -1;
-  return 256 + ((n + 3) / 4) * 4;
+  return kStatMarksOff + ((n + 3) / 4) * 4;
 }
 
 int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_bytes, int val_bytes,
@@ -317,15 +389,14 @@ int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_byt
   }
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "shmt_hashmap_plan: scratch must be 16-byte aligned");
   hipStream_t s = as_stream(stream);
-  KeyStats *dev_stats = static_cast<KeyStats *>(scratch);
-  uint32_t *marks = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + 256);  // one byte per id
-  hipLaunchKernelGGL(stats_init_kernel, dim3(1), dim3(1), 0, s, dev_stats);
-  hipLaunchKernelGGL(key_stats_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, vals, n,
-                     key_bytes, val_bytes, dev_stats);
+  KeyStats *partials = reinterpret_cast<KeyStats *>(static_cast<char *>(scratch) + kStatPartialsOff);
+  uint32_t *marks = reinterpret_cast<uint32_t *>(static_cast<char *>(scratch) + kStatMarksOff);  // one byte per id
+  const unsigned nb = grid_for(n, 256 * 8, kStatBlocks);
+  hipLaunchKernelGGL(key_stats_kernel, dim3(nb), dim3(256), 0, s, keys, vals, n, key_bytes, val_bytes, partials);
   SHMT_LAUNCH_CHECK();
   KeyStats st;
-  SHMT_HIP(hipMemcpyAsync(&st, dev_stats, sizeof(st), hipMemcpyDeviceToHost, s));
-  SHMT_HIP(hipStreamSynchronize(s));
+  int rc = read_stats(partials, static_cast<int>(nb), &st, s);
+  if (rc) return rc;
 
   const bool keys32 = st.kmin >= INT32_MIN && st.kmax <= INT32_MAX;
   const bool vals32 = st.vmin >= INT32_MIN && st.vmax <= INT32_MAX;
@@ -342,12 +413,13 @@ int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_byt
     hipLaunchKernelGGL(fill_zero_kernel, dim3(grid_for(words, 256 * 4)), dim3(256), 0, s, marks, words);
     hipLaunchKernelGGL(key_mark_kernel, dim3(grid_for(n, 256 * 8, 256 * 8)), dim3(256), 0, s, keys, n, key_bytes,
                        static_cast<int64_t>(st.kmin), reinterpret_cast<uint8_t *>(marks));
-    hipLaunchKernelGGL(key_count_marks_kernel, dim3(grid_for(words, 256 * 8, 256 * 8)), dim3(256), 0, s, marks,
-                       words, dev_stats);
+    const unsigned nbc = grid_for(words, 256 * 8, kStatBlocks);
+    hipLaunchKernelGGL(key_count_marks_kernel, dim3(nbc), dim3(256), 0, s, marks, words, partials);
     SHMT_LAUNCH_CHECK();
-    SHMT_HIP(hipMemcpyAsync(&st, dev_stats, sizeof(st), hipMemcpyDeviceToHost, s));
-    SHMT_HIP(hipStreamSynchronize(s));
-    if (st.distinct == static_cast<unsigned long long>(n)) {
+    KeyStats counted;
+    rc = read_stats(partials, static_cast<int>(nbc), &counted, s);
+    if (rc) return rc;
+    if (counted.distinct == static_cast<unsigned long long>(n)) {
       layout->kind = SHMT_MAP_RANGE;
       layout->slot_bytes = 0;
       layout->lo = st.kmin;

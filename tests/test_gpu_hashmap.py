@@ -286,6 +286,6 @@ def test_planned_build_through_the_c_abi(cabi):
     cabi.check(lib.shmt_hashmap_plan(big.data_ptr(), vals.data_ptr(), n, 8, 8, 0.5, scratch.data_ptr(), sb,
                                      ctypes.byref(lay), stream))
     assert (lay.kind, lay.slot_bytes) == (0, 16) and lay.table_bytes == lib.shmt_hashmap_table_bytes(n, 0.5, 8, 8)
-    small = torch.empty(16, dtype=torch.uint8, device="cuda")
-    assert lib.shmt_hashmap_plan(big.data_ptr(), vals.data_ptr(), n, 8, 8, 0.5, small.data_ptr(), 16,
+    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    assert lib.shmt_hashmap_plan(big.data_ptr(), vals.data_ptr(), n, 8, 8, 0.5, small.data_ptr(), 1024,
                                  ctypes.byref(lay), stream) == -4                     # scratch too small
