@@ -684,7 +684,11 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   const RlUniqueArgs unq{total, elem_bytes, n, labels_out, partials, unique_out, rank_of, count_out, count_copy,
                          scanned};
   const RlLabelsArgs lab{labels_out, elem_bytes, n, rank_of};
-  const unsigned ins_blocks = grid_for(N, kRlInsertTile, 256 * 32), lab_blocks = grid_for(N, 256);
+  // At most 1,024 workgroups insert, each walking its tiles in turn: random global atomics run at 20-26 G/s on
+  // this part whatever the grid (a third of the rate of plain stores), and a workgroup's later tiles then find
+  // the ids of hub nodes already in the table with a smaller index and skip their atomics, where 8,192
+  // workgroups starting together all miss them (8 batches per launch: 64.5 -> 62.3 us per batch).
+  const unsigned ins_blocks = grid_for(N, kRlInsertTile, 1024), lab_blocks = grid_for(N, 256);
   if (defer) {
     if (!prepared || scanned) {
       defer->mergeable = false;

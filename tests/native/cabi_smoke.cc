@@ -1,7 +1,8 @@
 // Stand-alone check of the C ABI: no Python, no torch. Links libshmt.so and the
 // HIP runtime only, allocates with hipMalloc / hipHostMalloc, and compares the
-// hashmap, fetch, set, scan, relabel and sampling entry points with plain C++
-// loops on the host. Exit status 0 = every check passed.
+// hashmap (dtype-chosen and key-chosen layouts), fetch, set, scan (with and
+// without a workspace), relabel, sampling, the fused hop and the coordinate
+// form of a block with plain C++ loops on the host. Exit status 0 = every check passed.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -255,6 +256,116 @@ int main() {
     EXPECT(to_host(d_total, all.size()) == all);
     std::vector<int64_t> lab2 = to_host(d_lab2, all.size());
     for (size_t i = 0; i < all.size(); ++i) EXPECT(lab2[i] == first2[all[i]]);
+  }
+
+  // ---- map layouts chosen from the keys: id range, direct table, bucket table ----
+  {
+    const int64_t m = 50000;
+    std::vector<int64_t> rk(m), rv(m), dk(m), dv(m);
+    for (int64_t i = 0; i < m; ++i) {
+      rk[i] = 700 + i;       // ids 700 .. 50,699 -> slot id - 700: a range
+      rv[i] = i;
+      dk[i] = 3 * i + 5;     // every third id: a direct table over the id universe
+      dv[i] = m - 1 - i;
+    }
+    struct Case { std::vector<int64_t> *k, *v; int kind; } cases[2] = {{&rk, &rv, SHMT_MAP_RANGE}, {&dk, &dv, SHMT_MAP_DIRECT}};
+    const int64_t sbytes = shmt_hashmap_plan_scratch_bytes(m);
+    void *d_ps = nullptr;
+    HIP_OK(hipMalloc(&d_ps, sbytes));
+    for (const Case &c : cases) {
+      int64_t *dk_ = to_device(*c.k), *dv_ = to_device(*c.v);
+      shmt_hashmap_layout lay;
+      SHMT_OK_(shmt_hashmap_plan(dk_, dv_, m, 8, 8, 0.8, d_ps, sbytes, &lay, stream));
+      EXPECT(lay.kind == c.kind);
+      void *d_t = nullptr;
+      HIP_OK(hipMalloc(&d_t, lay.table_bytes));
+      shmt_hashmap_t *pm = nullptr;
+      SHMT_OK_(shmt_hashmap_create_planned(&pm, &lay, dk_, dv_, m, 8, 8, 0.8, d_t, lay.table_bytes, stream));
+      EXPECT(shmt_hashmap_kind(pm) == c.kind);
+      std::vector<int64_t> rq(100001);
+      for (auto &x : rq) x = static_cast<int64_t>(rnd() % 200000) - 100;
+      int64_t *d_rq = to_device(rq), *d_rr = nullptr;
+      HIP_OK(hipMalloc(&d_rr, rq.size() * 8));
+      SHMT_OK_(shmt_hashmap_query(pm, d_rq, 8, static_cast<int64_t>(rq.size()), d_rr, stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      std::unordered_map<int64_t, int64_t> t;
+      for (int64_t i = 0; i < m; ++i) t[(*c.k)[i]] = (*c.v)[i];
+      std::vector<int64_t> rr = to_host(d_rr, rq.size());
+      for (size_t i = 0; i < rq.size(); ++i) {
+        auto it = t.find(rq[i]);
+        EXPECT(rr[i] == (it == t.end() ? -1 : it->second));
+      }
+      shmt_hashmap_destroy(pm);
+      HIP_OK(hipFree(d_t));
+      HIP_OK(hipFree(d_rq));
+      HIP_OK(hipFree(d_rr));
+      HIP_OK(hipFree(dk_));
+      HIP_OK(hipFree(dv_));
+    }
+    HIP_OK(hipFree(d_ps));
+  }
+
+  // ---- scan without a workspace argument: 3,000,001 int64, then a shorter int32 array ----
+  {
+    const int64_t l1 = 3000001, l2 = 70001;
+    std::vector<int64_t> b1(l1);
+    for (auto &x : b1) x = static_cast<int64_t>(rnd() >> 8);
+    std::vector<int32_t> b2(l2);
+    for (auto &x : b2) x = static_cast<int32_t>(rnd() % 77);
+    int64_t *d_b1 = to_device(b1);
+    int32_t *d_b2 = to_device(b2);
+    SHMT_OK_(shmt_exclusive_scan_noalloc(nullptr, 0, 8, stream));     // set-up call
+    SHMT_OK_(shmt_exclusive_scan_noalloc(d_b1, l1, 8, stream));
+    SHMT_OK_(shmt_exclusive_scan_noalloc(d_b2, l2, 4, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<int64_t> s1 = to_host(d_b1, l1);
+    uint64_t r1 = 0;
+    for (int64_t i = 0; i < l1; ++i) {
+      EXPECT(static_cast<uint64_t>(s1[i]) == r1);
+      r1 += static_cast<uint64_t>(b1[i]);
+    }
+    std::vector<int32_t> s2 = to_host(d_b2, l2);
+    uint32_t r2 = 0;
+    for (int64_t i = 0; i < l2; ++i) {
+      EXPECT(static_cast<uint32_t>(s2[i]) == r2);
+      r2 += static_cast<uint32_t>(b2[i]);
+    }
+    EXPECT(shmt_exclusive_scan_noalloc(d_b1, SHMT_SCAN_NOALLOC_MAX_LEN + 1, 8, stream) == SHMT_EINVAL);
+  }
+
+  // ---- coordinate form: destination position of every sampled id, from a hop job and from sub_indptr ----
+  {
+    const int64_t S = 7, k = 5, n_max = S + S * k;
+    int64_t *d_sp = nullptr, *d_sub3 = nullptr, *d_total = nullptr, *d_uniq = nullptr, *d_lab = nullptr;
+    int64_t *d_coo = nullptr, *d_rows = nullptr, *h_sizes = nullptr;
+    void *d_plan3 = nullptr, *d_scr = nullptr;
+    HIP_OK(hipMalloc(&d_sp, (S + 1) * 8));
+    HIP_OK(hipMalloc(&d_sub3, S * k * 8));
+    HIP_OK(hipMalloc(&d_total, n_max * 8));
+    HIP_OK(hipMalloc(&d_uniq, n_max * 8));
+    HIP_OK(hipMalloc(&d_lab, n_max * 8));
+    HIP_OK(hipMalloc(&d_coo, S * k * 8));
+    HIP_OK(hipMalloc(&d_rows, S * k * 8));
+    HIP_OK(hipMalloc(&d_plan3, pbytes));
+    const int64_t sb3 = shmt_relabel_scratch_bytes(n_max);
+    HIP_OK(hipMalloc(&d_scr, sb3));
+    HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&h_sizes), 16, hipHostMallocDefault));
+    shmt_hop_job job = {};
+    job.indptr = d_indptr; job.ptr_bytes = 8; job.indices = d_indices; job.idx_bytes = 8;
+    job.seeds = d_seeds; job.seed_bytes = 8; job.max_seeds = S; job.k = k; job.replace = 0;
+    job.rng_seed = 7777; job.rng_stream = 0;
+    job.sub_indptr = d_sp; job.sub_indices = d_sub3; job.plan = d_plan3; job.plan_bytes = pbytes;
+    job.elem_bytes = 8; job.total_out = d_total; job.scratch = d_scr; job.scratch_bytes = sb3;
+    job.unique_out = d_uniq; job.labels_out = d_lab; job.nnz_out = h_sizes; job.count_out = h_sizes + 1;
+    job.coo_dst = d_coo; job.coo_bytes = 8;
+    SHMT_OK_(shmt_sample_hops_chained(&job, 1, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    EXPECT(h_sizes[0] == 25);
+    SHMT_OK_(shmt_csr_rows(d_sp, 8, S, h_sizes[0], d_rows, 8, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    const std::vector<int64_t> want = {0, 2, 2, 2, 2, 3, 3, 3, 3, 3, 4, 4, 4, 4, 4, 5, 5, 5, 5, 5, 6, 6, 6, 6, 6};
+    EXPECT(to_host(d_coo, 25) == want);
+    EXPECT(to_host(d_rows, 25) == want);
   }
 
   shmt_hashmap_destroy(map);
