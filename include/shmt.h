@@ -234,11 +234,22 @@ int shmt_exclusive_scan_noalloc(void *data, int64_t len, int elem_bytes,
  * device-accessible; when it points into pinned host memory the caller reads
  * it after synchronising the stream. unique_out must hold N elements. The
  * value -1 is not representable (empty key, src/tensor_relabel.cu:119).
- * N < 2^31.                                                                */
+ * Inputs of 2^31 ids or more (elem_bytes must then be 8) are relabelled with
+ * 64-bit positions throughout, by the passes of shmt_relabel_wide; the
+ * reference stops at 2^31 (int numel, uint32_t table positions,
+ * src/tensor_relabel.cu:75-76,122,136).                                    */
 int64_t shmt_relabel_scratch_bytes(int64_t N);
 int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  int64_t scratch_bytes, void *unique_out, void *labels_out,
                  int64_t *count_out, void *stream);
+/* The 64-bit-position form on its own, for 8-byte ids and any N < 2^40
+ * (shmt_relabel switches to it at N >= 2^31; below that it is the slower
+ * choice: 16-byte slots, no per-workgroup de-duplication, 8-byte ranks).
+ * scratch >= shmt_relabel_wide_scratch_bytes(N), 16-byte aligned.           */
+int64_t shmt_relabel_wide_scratch_bytes(int64_t N);
+int shmt_relabel_wide(const void *total, int64_t N, void *scratch,
+                      int64_t scratch_bytes, void *unique_out,
+                      void *labels_out, int64_t *count_out, void *stream);
 /* Same, with the concatenation of the caller's tensors (torch::cat,
  * src/tensor_relabel.cu:131) done on the way in: nseg <= SHMT_RELABEL_MAX_SEGMENTS
  * segments seg_ptrs[s] of seg_lens[s] ids, seg_bytes[s] in {4,8} wide, are

@@ -316,6 +316,26 @@ std::tuple<torch::Tensor, torch::Tensor> create_subcsr(torch::Tensor uva_indptr,
 // ---- relabel ---------------------------------------------------------------------
 
 // TensorRelabel, src/tensor_relabel.cu:125-209.
+// 2^31 ids or more: concatenated as int64 and relabelled with 64-bit positions (shmt_relabel switches to
+// its wide form); the reference cannot represent such inputs (int numel, src/tensor_relabel.cu:136).
+static std::tuple<torch::Tensor, std::vector<torch::Tensor>> relabel_huge(const std::vector<torch::Tensor> &tensors,
+                                                                          const std::vector<int64_t> &split_sizes,
+                                                                          int64_t N) {
+  std::vector<torch::Tensor> wide;
+  for (const auto &t : tensors) wide.push_back(t.to(torch::kInt64));
+  torch::Tensor total = torch::cat(wide, 0).contiguous();
+  wide.clear();
+  torch::Tensor unique = torch::empty({N}, total.options());
+  torch::Tensor labels = torch::empty({N}, total.options());
+  const int64_t scratch_bytes = shmt_relabel_scratch_bytes(N);
+  torch::Tensor scratch = device_bytes(scratch_bytes);
+  const Readback::Slot count = readback().acquire();
+  check(shmt_relabel(total.data_ptr(), N, 8, scratch.data_ptr(), scratch_bytes, unique.data_ptr(),
+                     labels.data_ptr(), count.dev, current_stream()));
+  const int64_t U = Readback::wait(count);
+  return std::make_tuple(unique.narrow(0, 0, U), labels.split_with_sizes(split_sizes, 0));
+}
+
 std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
     std::vector<torch::Tensor> tensors) {
   TORCH_CHECK(!tensors.empty(), "tensor_relabel needs at least one tensor");
@@ -330,6 +350,8 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> tensor_relabel(
   const auto options = tensors[0].options().dtype(eb == 8 ? torch::kInt64 : torch::kInt32);
   int64_t N = 0;
   for (int64_t n : split_sizes) N += n;
+  // 2^31 ids and more: positions need 64 bits, so the results are int64 whatever the inputs are
+  if (N >= (int64_t{1} << 31)) return relabel_huge(tensors, split_sizes, N);
   torch::Tensor unique = torch::empty({N}, options);
   torch::Tensor labels = torch::empty({N}, options);
   if (N == 0) return std::make_tuple(unique, labels.split_with_sizes(split_sizes, 0));

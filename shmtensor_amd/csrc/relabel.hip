@@ -606,6 +606,172 @@ uint64_t relabel_nonce() {
   return z ^ (z >> 31);
 }
 
+
+// ---- 2^31 ids and more: 64-bit positions ------------------------------------------
+// The passes above keep first-occurrence indices, ranks and table positions in
+// 32 bits (the reference does the same: int numel / uint32_t positions,
+// src/tensor_relabel.cu:75-76,122,136). Inputs of 2^31 ids or more take this
+// path instead: the same four passes with 64-bit indices and ranks throughout
+// ({int64 key, uint64 first index} slots, a 64-bit hash position, a rank array
+// of 8 bytes per id), without the small-input, packed-slot and merged-launch
+// forms, which such inputs have no use for. Ids are 8 bytes wide.
+struct RlSlot64 {
+  int64_t key;
+  unsigned long long first;
+};
+static_assert(sizeof(RlSlot64) == 16, "slot must be 16 bytes");
+
+constexpr int kRl64Tile = 512;  // ids per workgroup in the first-occurrence and unique passes
+
+__device__ __forceinline__ uint64_t rl64_home(int64_t key, uint64_t cap) {
+  uint64_t x = static_cast<uint64_t>(key);
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdull;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ull;
+  x ^= x >> 33;
+  return __umul64hi(x, cap);  // floor(x * cap / 2^64) < cap
+}
+
+__global__ __launch_bounds__(256) void rl64_insert_kernel(RlSlot64 *tbl, uint64_t cap, const int64_t *total,
+                                                          int64_t N) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < N; i += stride) {
+    const int64_t key = total[i];
+    uint64_t pos = rl64_home(key, cap);
+    for (uint64_t probes = 0; probes < cap; ++probes) {
+      // look before the atomics (see rl_global_insert)
+      const int64_t seen = __hip_atomic_load(&tbl[pos].key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (seen == key) {
+        if (__hip_atomic_load(&tbl[pos].first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >
+            static_cast<unsigned long long>(i))
+          atomicMin(&tbl[pos].first, static_cast<unsigned long long>(i));
+        break;
+      }
+      if (seen == -1) {
+        const unsigned long long prev = atomicCAS(reinterpret_cast<unsigned long long *>(&tbl[pos].key), ~0ull,
+                                                  static_cast<unsigned long long>(key));
+        if (prev == ~0ull || static_cast<int64_t>(prev) == key) {
+          atomicMin(&tbl[pos].first, static_cast<unsigned long long>(i));
+          break;
+        }
+      }
+      pos = (pos + 1 == cap) ? 0 : pos + 1;
+    }
+  }
+}
+
+// labels[i] = first index of total[i]; partials[tile] = number of first occurrences in the tile.
+__global__ __launch_bounds__(kRl64Tile) void rl64_first_kernel(const RlSlot64 *tbl, uint64_t cap,
+                                                               const int64_t *total, int64_t N, int64_t *labels,
+                                                               uint64_t *partials) {
+  __shared__ uint64_t lds[kRl64Tile / kWave];
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kRl64Tile + threadIdx.x;
+  uint64_t cnt = 0;
+  if (i < N) {
+    const int64_t key = total[i];
+    uint64_t pos = rl64_home(key, cap);
+    unsigned long long f = ~0ull;
+    for (uint64_t probes = 0; probes < cap; ++probes) {
+      const RlSlot64 s = tbl[pos];
+      if (s.key == key) {
+        f = s.first;
+        break;
+      }
+      if (s.key == -1) break;  // cannot happen: every key was inserted
+      pos = (pos + 1 == cap) ? 0 : pos + 1;
+    }
+    labels[i] = static_cast<int64_t>(f);
+    cnt = (f == static_cast<unsigned long long>(i));
+  }
+  uint64_t tile_total;
+  block_exclusive_scan<uint64_t, kRl64Tile>(cnt, lds, &tile_total);
+  if (threadIdx.x == 0) partials[blockIdx.x] = tile_total;
+}
+
+// partials: exclusive scan of the tile counts, partials[nb] = number of distinct ids.
+__global__ __launch_bounds__(kRl64Tile) void rl64_unique_kernel(const int64_t *total, int64_t N,
+                                                                const int64_t *labels, const uint64_t *partials,
+                                                                int64_t nb, int64_t *unique_out,
+                                                                unsigned long long *rank_of, int64_t *count_out) {
+  __shared__ uint64_t lds[kRl64Tile / kWave];
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kRl64Tile + threadIdx.x;
+  const bool win = i < N && labels[i] == i;
+  uint64_t tile_total;
+  const uint64_t ex = block_exclusive_scan<uint64_t, kRl64Tile>(win ? 1 : 0, lds, &tile_total);
+  if (win) {
+    const uint64_t rank = partials[blockIdx.x] + ex;
+    unique_out[rank] = total[i];
+    rank_of[i] = rank;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) publish_size(count_out, static_cast<int64_t>(partials[nb]));
+}
+
+__global__ __launch_bounds__(256) void rl64_labels_kernel(int64_t *labels, int64_t N,
+                                                          const unsigned long long *rank_of) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < N; i += stride)
+    labels[i] = static_cast<int64_t>(rank_of[labels[i]]);
+}
+
+struct Rl64Layout {
+  int64_t cap, table_off, rank_off, partial_off, scan_off, scan_bytes, total;
+};
+
+static Rl64Layout rl64_layout(int64_t N) {
+  Rl64Layout l;
+  l.cap = (2 * N + 7) & ~7ll;
+  if (l.cap < 64) l.cap = 64;
+  l.table_off = 0;
+  l.rank_off = l.cap * 16;
+  l.partial_off = l.rank_off + ((N * 8 + 255) & ~255ll);
+  const int64_t nb = (N + kRl64Tile - 1) / kRl64Tile;
+  l.scan_off = l.partial_off + (((nb + 1) * 8 + 255) & ~255ll);
+  l.scan_bytes = shmt_scan_tmp_bytes(nb + 1);
+  l.total = l.scan_off + ((l.scan_bytes + 255) & ~255ll) + 256;
+  return l;
+}
+
+static int relabel_wide_impl(const void *total, int64_t N, void *scratch, int64_t scratch_bytes, void *unique_out,
+                             void *labels_out, int64_t *count_out, hipStream_t s) {
+  SHMT_REQUIRE(N >= 1, "shmt_relabel_wide: N must be >= 1");
+  SHMT_REQUIRE(N < (1ll << 40), "shmt_relabel_wide: N must be < 2^40");
+  SHMT_REQUIRE(total && unique_out && labels_out && count_out, "shmt_relabel_wide: null buffer");
+  const Rl64Layout l = rl64_layout(N);
+  if (scratch == nullptr || scratch_bytes < l.total) {
+    set_error("shmt_relabel_wide: scratch too small (%lld < %lld bytes)", static_cast<long long>(scratch_bytes),
+              static_cast<long long>(l.total));
+    return SHMT_ENOMEM;
+  }
+  SHMT_REQUIRE((reinterpret_cast<uintptr_t>(scratch) & 15) == 0, "shmt_relabel_wide: scratch must be 16-byte aligned");
+  char *base = static_cast<char *>(scratch);
+  RlSlot64 *tbl = reinterpret_cast<RlSlot64 *>(base + l.table_off);
+  unsigned long long *rank_of = reinterpret_cast<unsigned long long *>(base + l.rank_off);
+  uint64_t *partials = reinterpret_cast<uint64_t *>(base + l.partial_off);
+  const int64_t nb = (N + kRl64Tile - 1) / kRl64Tile;
+  SHMT_REQUIRE(nb < (1ll << 31), "shmt_relabel_wide: input too large");
+  int rc = launch_fill_ones(tbl, l.cap, s);
+  if (rc) return rc;
+  const int64_t *ids = static_cast<const int64_t *>(total);
+  hipLaunchKernelGGL(rl64_insert_kernel, dim3(grid_for(N, 256, 4096)), dim3(256), 0, s, tbl,
+                     static_cast<uint64_t>(l.cap), ids, N);
+  SHMT_LAUNCH_CHECK();
+  hipLaunchKernelGGL(rl64_first_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRl64Tile), 0, s, tbl,
+                     static_cast<uint64_t>(l.cap), ids, N, static_cast<int64_t *>(labels_out), partials);
+  SHMT_LAUNCH_CHECK();
+  // nb + 1 entries (the last one arbitrary: an exclusive scan ignores it) -> partials[nb] = number of distinct ids
+  rc = shmt_exclusive_scan(partials, nb + 1, 8, base + l.scan_off, l.scan_bytes, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(rl64_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRl64Tile), 0, s, ids, N,
+                     static_cast<const int64_t *>(labels_out), partials, nb, static_cast<int64_t *>(unique_out),
+                     rank_of, count_out);
+  SHMT_LAUNCH_CHECK();
+  hipLaunchKernelGGL(rl64_labels_kernel, dim3(grid_for(N, 256, 8192)), dim3(256), 0, s,
+                     static_cast<int64_t *>(labels_out), N, rank_of);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
+
 }  // namespace shmt
 
 using namespace shmt;
@@ -614,7 +780,12 @@ extern "C" {
 
 int64_t shmt_relabel_scratch_bytes(int64_t N) {
   if (N < 0) return -1;
-  return rl_layout(N).total;
+  return N < (1ll << 31) ? rl_layout(N).total : rl64_layout(N).total;
+}
+
+int64_t shmt_relabel_wide_scratch_bytes(int64_t N) {
+  if (N < 0) return -1;
+  return rl64_layout(N > 0 ? N : 1).total;
 }
 
 // N is the host-known number of ids, or an upper bound of it when `n.extra`
@@ -626,7 +797,13 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
                         uint64_t prepared_nonce = 0, int64_t *count_copy = nullptr,
                         int64_t prepared_slots = 0) {
   SHMT_REQUIRE(N >= 0, "shmt_relabel: N must be >= 0");
-  SHMT_REQUIRE(N < (1ll << 31), "shmt_relabel: N must be < 2^31");
+  if (N >= (1ll << 31)) {
+    // 64-bit positions: a plain call only (segments are concatenated by the caller, hops stay below 2^31)
+    SHMT_REQUIRE(!segs && !prepared && !launcher.defer && !n.fixed_dev && !n.extra,
+                 "shmt_relabel: inputs of 2^31 ids or more are relabelled by shmt_relabel / shmt_relabel_wide only");
+    SHMT_REQUIRE(elem_bytes == 8, "shmt_relabel: inputs of 2^31 ids or more must be 8 bytes wide");
+    return relabel_wide_impl(total, N, scratch, scratch_bytes, unique_out, labels_out, count_out, launcher.stream);
+  }
   SHMT_REQUIRE(width_ok(elem_bytes), "shmt_relabel: ID can only be int32 or int64");
   SHMT_REQUIRE(count_out != nullptr, "shmt_relabel: count_out is null");
   hipStream_t s = launcher.stream;
@@ -811,6 +988,19 @@ int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  void *stream) {
   return relabel_impl(total, nullptr, N, RlCount{N, nullptr, nullptr, 8, N}, elem_bytes, scratch, scratch_bytes,
                       unique_out, labels_out, count_out, Launcher{as_stream(stream), nullptr});
+}
+
+int shmt_relabel_wide(const void *total, int64_t N, void *scratch, int64_t scratch_bytes, void *unique_out,
+                      void *labels_out, int64_t *count_out, void *stream) {
+  SHMT_REQUIRE(N >= 0, "shmt_relabel_wide: N must be >= 0");
+  SHMT_REQUIRE(count_out != nullptr, "shmt_relabel_wide: count_out is null");
+  if (N == 0) {
+    hipLaunchKernelGGL(rl_zero_count_kernel, dim3(1), dim3(1), 0, as_stream(stream), count_out,
+                       static_cast<int64_t *>(nullptr));
+    SHMT_LAUNCH_CHECK();
+    return SHMT_OK;
+  }
+  return relabel_wide_impl(total, N, scratch, scratch_bytes, unique_out, labels_out, count_out, as_stream(stream));
 }
 
 int shmt_relabel_segments(const void *const *seg_ptrs, const int64_t *seg_lens, const int *seg_bytes,

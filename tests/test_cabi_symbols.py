@@ -37,6 +37,13 @@ def test_size_queries_and_validation(cabi):
     assert lib.shmt_scan_tmp_bytes(1000) == 0 and lib.shmt_scan_tmp_bytes(1 << 20) == 64 + 64 * 16
     assert lib.shmt_relabel_scratch_bytes(1000) >= 2000 * 16 + 4000
     assert lib.shmt_sample_plan_bytes(1024) >= 1024 * 16
+    # relabel with 64-bit positions: 16-byte slots at load <= 0.5, 8-byte ranks; shmt_relabel uses it from 2^31 ids
+    assert lib.shmt_relabel_wide_scratch_bytes(1000) >= 2000 * 16 + 1000 * 8
+    big = 1 << 31
+    assert lib.shmt_relabel_scratch_bytes(big) == lib.shmt_relabel_wide_scratch_bytes(big) >= big * (32 + 8)
+    assert lib.shmt_relabel_scratch_bytes(big - 1) < big * 40
+    assert lib.shmt_relabel(None, big, 4, None, 0, None, None, None, None) == -1
+    assert b"8 bytes wide" in lib.shmt_last_error()
     # empty inputs are no-ops that need no device
     assert lib.shmt_fetch(None, None, None, 8, None, None, 0, None, 0, 512, None) == 0
     assert lib.shmt_set(None, None, None, 8, None, None, 0, None, 0, 512, None) == 0
