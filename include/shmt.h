@@ -8,7 +8,7 @@
  *    or host memory that is pinned and device-mapped (see shmt_host_devptr).
  *    No torch types cross this boundary; callers allocate every buffer,
  *    including scratch (the library itself allocates no device memory; it
- *    keeps 1 KiB of pinned host memory for reading small results back), and
+ *    keeps 256 bytes of pinned host memory for reading small results back), and
  *    pass element SIZES in bytes (4 or 8 for integer
  *    ids; any size for feature rows, which are copied bit for bit).
  *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).

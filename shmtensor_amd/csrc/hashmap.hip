@@ -5,7 +5,6 @@
 #include <math.h>
 #include <stdlib.h>
 
-#include <atomic>
 #include <mutex>
 
 #include "common.h"
@@ -244,38 +243,26 @@ __global__ __launch_bounds__(256) void stats_merge_kernel(const KeyStats *partia
   if (threadIdx.x == 0) *host_slot = all;
 }
 
-constexpr int kStatSlots = 16;  // concurrent map builds each take their own
+// One slot of pinned host memory per process, allocated on first use; map
+// builds that run at the same time take turns at it.
 static std::mutex g_stat_mutex;
-static KeyStats *g_stat_slots = nullptr;      // pinned host memory
-static KeyStats *g_stat_slots_dev = nullptr;  // its device alias
-static std::atomic<unsigned> g_stat_next{0};
-
-static int stat_slot(KeyStats **host, KeyStats **dev) {
-  {
-    std::lock_guard<std::mutex> lock(g_stat_mutex);
-    if (g_stat_slots == nullptr) {
-      void *p = nullptr, *d = nullptr;
-      SHMT_HIP(hipHostMalloc(&p, kStatSlots * sizeof(KeyStats), hipHostMallocMapped));
-      SHMT_HIP(hipHostGetDevicePointer(&d, p, 0));
-      g_stat_slots = static_cast<KeyStats *>(p);
-      g_stat_slots_dev = static_cast<KeyStats *>(d);
-    }
-  }
-  const unsigned i = g_stat_next.fetch_add(1) % kStatSlots;
-  *host = g_stat_slots + i;
-  *dev = g_stat_slots_dev + i;
-  return SHMT_OK;
-}
+static KeyStats *g_stat_slot = nullptr;      // pinned host memory
+static KeyStats *g_stat_slot_dev = nullptr;  // its device alias
 
 // Merge the partial results of a sweep, hand them to the host and wait for them.
 static int read_stats(const KeyStats *partials, int nb, KeyStats *out, hipStream_t s) {
-  KeyStats *host = nullptr, *host_dev = nullptr;
-  int rc = stat_slot(&host, &host_dev);
-  if (rc) return rc;
-  hipLaunchKernelGGL(stats_merge_kernel, dim3(1), dim3(256), 0, s, partials, nb, host_dev);
+  std::lock_guard<std::mutex> lock(g_stat_mutex);
+  if (g_stat_slot == nullptr) {
+    void *p = nullptr, *d = nullptr;
+    SHMT_HIP(hipHostMalloc(&p, 256, hipHostMallocMapped));
+    SHMT_HIP(hipHostGetDevicePointer(&d, p, 0));
+    g_stat_slot = static_cast<KeyStats *>(p);
+    g_stat_slot_dev = static_cast<KeyStats *>(d);
+  }
+  hipLaunchKernelGGL(stats_merge_kernel, dim3(1), dim3(256), 0, s, partials, nb, g_stat_slot_dev);
   SHMT_LAUNCH_CHECK();
   SHMT_HIP(hipStreamSynchronize(s));
-  *out = *host;
+  *out = *g_stat_slot;
   return SHMT_OK;
 }
 

@@ -197,24 +197,35 @@ __device__ __forceinline__ void rl_insert_body(unsigned bx, unsigned gx, const R
   const bool packed = rl_packed(a.path);
   __shared__ unsigned long long lkey[kRlLdsSlots];
   __shared__ uint32_t lfirst[kRlLdsSlots];
+  // ids that fit 32 bits (the packed table's case) are staged as 32-bit keys: a slot then lies in one LDS
+  // bank and the compare-and-swap is a 32-bit one, which halves the staging table's bank conflicts
+  uint32_t *const lkey32 = reinterpret_cast<uint32_t *>(lkey);
   const int64_t ntiles = (N + kRlInsertTile - 1) / kRlInsertTile;
   for (int64_t tile = bx; tile < ntiles; tile += gx) {
     for (int t = threadIdx.x; t < kRlLdsSlots; t += kRlBlock) {
-      lkey[t] = ~0ull;
+      if (packed) lkey32[t] = 0xFFFFFFFFu; else lkey[t] = ~0ull;
       lfirst[t] = 0xFFFFFFFFu;
     }
     __syncthreads();
     const int64_t i = tile * kRlInsertTile + threadIdx.x;
     int64_t key = 0;
     uint32_t pos = 0;
+    bool staged = false;  // the id went through the staging table (always, except the one id that looks empty there)
     if (i < N) {
       key = load_int(total, i, eb);
       pos = hash_id(key) & (kRlLdsSlots - 1);
+      staged = !(packed && static_cast<uint32_t>(key) == 0xFFFFFFFFu);
       // the staging table has twice as many slots as the tile has ids: a free slot always turns up
-      for (int probes = 0; probes < kRlLdsSlots; ++probes) {
-        const unsigned long long prev =
-            atomicCAS(&lkey[pos], ~0ull, static_cast<unsigned long long>(key));
-        if (prev == ~0ull || static_cast<int64_t>(prev) == key) {
+      for (int probes = 0; staged && probes < kRlLdsSlots; ++probes) {
+        bool mine;
+        if (packed) {
+          const uint32_t prev = atomicCAS(&lkey32[pos], 0xFFFFFFFFu, static_cast<uint32_t>(key));
+          mine = prev == 0xFFFFFFFFu || prev == static_cast<uint32_t>(key);
+        } else {
+          const unsigned long long prev = atomicCAS(&lkey[pos], ~0ull, static_cast<unsigned long long>(key));
+          mine = prev == ~0ull || static_cast<int64_t>(prev) == key;
+        }
+        if (mine) {
           atomicMin(&lfirst[pos], static_cast<uint32_t>(i));
           break;
         }
@@ -224,7 +235,7 @@ __device__ __forceinline__ void rl_insert_body(unsigned bx, unsigned gx, const R
     __syncthreads();
     // the thread holding the smallest index of an id inserts it for the whole tile:
     // one global probe chain per thread at most
-    if (i < N && lfirst[pos] == static_cast<uint32_t>(i)) {
+    if (i < N && (!staged || lfirst[pos] == static_cast<uint32_t>(i))) {
       if (packed)
         rl_packed_insert(reinterpret_cast<unsigned long long *>(tbl), rl_cap8(cap),
                          static_cast<uint32_t>(key), static_cast<uint32_t>(i));

@@ -201,6 +201,20 @@ def test_c_abi_relabel_of_one_array(cabi, oracle, n, bytes_):
     assert np.array_equal(unique[:eu.size].cpu().numpy(), eu) and np.array_equal(labels.cpu().numpy(), el)
 
 
+def test_relabel_ids_at_the_top_of_32_bits(capi, oracle):
+    """int64 ids that all fit 32 bits take the packed table and a 32-bit staging table per workgroup; the id
+    2^32 - 1 looks like an empty staging slot and must still be relabelled (it bypasses the staging)."""
+    rng = np.random.default_rng(9)
+    top = 2**32 - 1
+    a = rng.integers(top - 50, top + 1, size=60_000).astype(np.int64)          # includes 2^32 - 1 many times
+    b = rng.integers(0, 1000, size=40_000).astype(np.int64)
+    u, (la, lb) = capi.tensor_relabel([torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()])
+    eu, (ea, eb_) = oracle.relabel([a, b])
+    assert top in eu
+    assert np.array_equal(u.cpu().numpy(), eu)
+    assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb_)
+
+
 # ---- 2^31 ids and more: 64-bit positions -------------------------------------------------------------
 
 @pytest.mark.parametrize("n", [1, 2, 511, 512, 513, 70_000, 3_000_000])
