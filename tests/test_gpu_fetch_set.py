@@ -351,3 +351,38 @@ def test_c_abi_fetch_with_the_row_count_in_device_memory(cabi, route, count):
     if hnd is not None:
         torch.cuda.synchronize()
         lib.shmt_hashmap_destroy(hnd)
+
+
+@pytest.mark.parametrize("D,dtype", [(32, torch.float32), (64, torch.float16), (7, torch.int8), (300, torch.float32)])
+@pytest.mark.parametrize("slots", ["8-byte", "16-byte"])
+def test_fetch_and_set_through_bucket_tables(capi, oracle, D, dtype, slots):
+    """Key sets that are too sparse for a flat map keep the bucket table: with ids that fit 32 bits its
+    8-byte slots (a small share of a large id universe is cached), with ids beyond 32 bits its 16-byte slots
+    (there the queries are all hits: no host table has 2^33 rows). Routing stays observable because cache
+    rows differ from host rows."""
+    rng = np.random.default_rng(D + len(slots))
+    n = 40_000
+    raw = torch.from_numpy(rng.integers(-120, 120, size=(n, D)).astype(np.int8 if dtype == torch.int8 else np.float32))
+    data = raw.to(dtype).pin_memory()
+    view = torch.int16 if dtype == torch.float16 else dtype
+    ids_np = rng.choice(n, size=n // 50, replace=False)                      # 1 id in 50 cached
+    gpu_data = (data[torch.from_numpy(ids_np)].float() + 1).to(dtype).cuda()
+    shift = 0 if slots == "8-byte" else 1 << 33
+    h = capi.CUCOStaticHashmap(torch.from_numpy(ids_np + shift).cuda(), torch.arange(ids_np.size).cuda(), 0.8)
+    assert h.layout() == "buckets" and h.memory_usage() == ids_np.size * 2 * (8 if shift == 0 else 16)
+    if shift == 0:
+        q_np = np.concatenate([rng.integers(0, n, size=3000), ids_np[rng.integers(0, ids_np.size, size=2001)]])
+    else:
+        q_np = ids_np[rng.integers(0, ids_np.size, size=5001)]
+    ref_h = oracle.Hashmap(ids_np, np.arange(ids_np.size), 0.8)
+    expect = oracle.fetch(data.view(view).numpy(), gpu_data.cpu().view(view).numpy(), q_np, hashmap=ref_h)
+    got = capi.cache_fetch(data, gpu_data, torch.from_numpy(q_np + shift).cuda(), h)
+    assert np.array_equal(got.cpu().view(view).numpy(), expect)
+    # set through the same map: final state of both tables
+    w_np = np.unique(q_np)
+    upd = torch.from_numpy(rng.integers(-100, 100, size=(w_np.size, D)).astype(np.float32)).to(dtype)
+    host_ref, gpu_ref = data.view(view).numpy().copy(), gpu_data.cpu().view(view).numpy().copy()
+    oracle.set_rows(host_ref, gpu_ref, w_np, upd.view(view).numpy(), hashmap=ref_h)
+    capi.cache_set(data, gpu_data, torch.from_numpy(w_np + shift).cuda(), upd.cuda(), h)
+    torch.cuda.synchronize()
+    assert np.array_equal(data.view(view).numpy(), host_ref) and np.array_equal(gpu_data.cpu().view(view).numpy(), gpu_ref)

@@ -239,6 +239,14 @@ def test_flat_layouts_route_fetch_set_and_sampling(capi, oracle, layout):
     want_host, want_cache = table.copy(), cache_np.copy()
     oracle.set_rows(want_host, want_cache, w, upd, hashmap=ref)
     assert np.array_equal(host.numpy(), want_host) and np.array_equal(cache.cpu().numpy(), want_cache)
+    # write-through: a hit also updates the host row
+    upd2 = rng.standard_normal((1500, 24)).astype(np.float32)
+    capi.cache_set(host, cache, _cuda(w), _cuda(upd2), h, write_through=True)
+    torch.cuda.synchronize()
+    want_host[w] = upd2
+    hit = ref.query(w) >= 0
+    want_cache[ref.query(w)[hit]] = upd2[hit]
+    assert np.array_equal(host.numpy(), want_host) and np.array_equal(cache.cpu().numpy(), want_cache)
     # sampling: cached rows (a sub-CSR in map order) and cold rows give what the uncached sampler gives
     deg = rng.integers(0, 30, size=n)
     indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
