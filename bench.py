@@ -219,14 +219,27 @@ def bench_fetch(capi, args, result):
     a = algo_bytes / (tm["median"] * 1e-3) / 1e9
     extra["fetch_all_hit_with_mask"] = {"ms": round(tm["median"], 4), "algorithmic_GBs": round(a, 1),
                                         "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
-    # The same all-hit batch through maps that do need a table: slots in arbitrary order over the same ids
-    # (direct table, one 4-byte load per row) and scattered ids (bucket table, one 128-byte bucket per probe).
-    # A random table read costs a whole 128-byte line whatever its size, so these move Q x (2R + 8 + 128)
-    # bytes for Q x (2R + 8) algorithmic ones: line_traffic_GBs is that real figure.
+    # The same all-hit batch through maps that do need a table. A cache whose rows are kept in id order (39 % of
+    # the ids 0 .. N-1, scattered; slot = rank of the id): bitmap with running counts, 16.7 MB, served from the
+    # caches. Slots in arbitrary order over the ids 0 .. C-1: direct table, one 4-byte load per row. Scattered
+    # ids with slots in arbitrary order: bucket table, one 128-byte bucket per probe. A random read from a table
+    # that does not fit the caches costs a whole 128-byte line whatever its size, so the last two move
+    # Q x (2R + 8 + 128) bytes for Q x (2R + 8) algorithmic ones: line_traffic_GBs is that real figure.
     gq = torch.Generator(device="cuda").manual_seed(17)
+    by_table = {}
+    kept = torch.nonzero(torch.rand(N, device="cuda", generator=gq) < 0.39).flatten()[:C].contiguous()
+    m = capi.CUCOStaticHashmap(kept, torch.arange(kept.numel(), device="cuda"), 0.8)
+    pos = torch.randint(0, kept.numel(), (Q,), device="cuda", generator=gq)
+    req = kept[pos]
+    assert torch.equal(capi.cache_fetch(host, cache, req[:4096], m), cache[pos[:4096]])
+    tt = gpu_time_ms(lambda: capi.cache_fetch(host, cache, req, m), 30)
+    a = algo_bytes / (tt["median"] * 1e-3) / 1e9
+    by_table["rank_bitmap"] = {"ms": round(tt["median"], 4), "map_layout": m.layout(), "map_bytes": m.memory_usage(),
+                               "keys": kept.numel(), "algorithmic_GBs": round(a, 1),
+                               "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4)}
+    del m, kept, pos, req
     ids = torch.arange(C, device="cuda")
     slots = torch.randperm(C, device="cuda", generator=gq)
-    by_table = {}
     for name, keys_t, req in (("direct_table", ids, qh), ("bucket_table_8B_slots", ids * 11 + 1, qh * 11 + 1),
                               ("bucket_table_16B_slots", ids * 37 + (1 << 33), qh * 37 + (1 << 33))):
         m = capi.CUCOStaticHashmap(keys_t, slots, 0.8)
@@ -463,7 +476,8 @@ def bench_sampling(capi, args, result):
     indptr = indptr_d.cpu().pin_memory()
     indices = indices_d.cpu().pin_memory()
     deg = indptr_d[1:] - indptr_d[:-1]
-    hot = torch.sort(deg, descending=True, stable=True).indices[: n * 3 // 10].contiguous()
+    # the cached rows are kept in id order (slot = rank of the id): the map is then a bitmap with running counts
+    hot = torch.sort(torch.sort(deg, descending=True, stable=True).indices[: n * 3 // 10]).values.contiguous()
     del indptr_d, indices_d
     gp, gi = capi.create_subcsr(indptr, indices, hot)
     hmap = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel(), device="cuda"), 0.8)
@@ -563,6 +577,7 @@ def bench_sampling(capi, args, result):
     del sampler
     res = {"graph": "R-MAT scale %d ef 30 symmetrised: %d nodes, %d edges; top 30 %% by degree cached"
                     % (args.sampling_scale, n, indices.numel()),
+           "map_layout": hmap.layout(),
            "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
            "edges_per_batch": edges // nbatch, "ms_per_batch": round(gpu_t * 1e3 / nbatch, 4),
            "sampled_edges_per_s": round(edges / gpu_t, 1),
@@ -622,7 +637,7 @@ def bench_e2e(capi, args, result):
     deg = indptr_d[1:] - indptr_d[:-1]
     by_degree = torch.sort(deg, descending=True, stable=True).indices
     del indptr_d, indices_d, deg
-    hot_adj = by_degree[: n // 5].contiguous()
+    hot_adj = torch.sort(by_degree[: n // 5]).values.contiguous()       # cache rows in id order, as above
     gp, gi = capi.create_subcsr(indptr, indices, hot_adj)
     adj_map = capi.CUCOStaticHashmap(hot_adj, torch.arange(hot_adj.numel(), device="cuda"), 0.8)
     D = 256
@@ -632,7 +647,7 @@ def bench_e2e(capi, args, result):
         hi = min(n, lo + 2_000_000)
         feats[lo:hi].copy_(torch.randn((hi - lo, D), device="cuda", generator=g))
     torch.cuda.synchronize()
-    hot_feat = by_degree[: n // 4].contiguous()
+    hot_feat = torch.sort(by_degree[: n // 4]).values.contiguous()
     feat_cache = capi.uva_fetch(feats, hot_feat)
     feat_map = capi.CUCOStaticHashmap(hot_feat, torch.arange(hot_feat.numel(), device="cuda"), 0.8)
     log("[e2e] R-MAT scale %d ef 16: %d nodes, %d edges; adjacency cache %d rows / %d edges; features %.1f GB "
@@ -741,6 +756,7 @@ def bench_e2e(capi, args, result):
     w0 = time.perf_counter()
     epoch()
     wall_pipe = time.perf_counter() - w0
+    dl.close()          # the producer thread has ended with its epoch; this only makes that explicit
     cpu = None
     if not args.no_cpu:
         import numpy as np
@@ -781,6 +797,7 @@ def bench_e2e(capi, args, result):
         "cpu_baseline": cpu,
         "graph": "R-MAT scale %d ef 16 symmetrised: %d nodes, %d edges; top 20 %% adjacency cached; features %d x %d "
                  "f32 pinned, top-degree 25 %% cached" % (args.e2e_scale, n, indices.numel(), n, D),
+        "map_layouts": {"adjacency": adj_map.layout(), "features": feat_map.layout()},
         "seeds_per_batch": S, "fanouts_in_call_order": list(reversed(fanouts)), "batches": nbatch,
         "edges_per_batch": tot_edges // nbatch, "input_nodes_per_batch": tot_nodes // nbatch,
         "feature_hit_rate": round(hit, 4),

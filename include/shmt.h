@@ -85,13 +85,19 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys,
                         int val_bytes, double load_factor, void *table_mem,
                         int64_t table_bytes, void *stream);
 /* Build with a layout chosen from the keys. Node ids are small dense
- * integers, so beside the general bucket table two flat forms exist:
+ * integers, so beside the general bucket table three flat forms exist:
  *   SHMT_MAP_DIRECT  keys lie in [lo, lo + span) and an int32 table
  *                    value[key - lo] is at most twice as large as the bucket
  *                    table would be: one 4-byte load per lookup;
  *   SHMT_MAP_RANGE   the keys are exactly lo .. lo + span - 1 and every value
  *                    is key + delta (the cache holds an id range, as in
  *                    re-numbered graphs): lookups are arithmetic, no table;
+ *   SHMT_MAP_RANK    the pairs are given in ascending key order with values
+ *                    v0, v0 + 1, ... (a cache whose rows are kept in id
+ *                    order): a bitmap with running counts, 16 bytes per 96
+ *                    ids of [lo, lo + span), value = rank of the key + delta;
+ *                    one 16-byte load per lookup from a table that stays in
+ *                    the caches (span / 6 bytes);
  * and the bucket table uses 8-byte slots whenever all keys and values fit 32
  * bits, whatever their dtype. Every form answers exactly like the general
  * table (same contract as the constructor above: include/cuco_hashmap.cuh:
@@ -104,11 +110,12 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys,
 #define SHMT_MAP_BUCKETS 0
 #define SHMT_MAP_DIRECT 1
 #define SHMT_MAP_RANGE 2
+#define SHMT_MAP_RANK 3
 typedef struct shmt_hashmap_layout {
   int kind;            /* SHMT_MAP_*                                        */
-  int slot_bytes;      /* buckets: 16 or 8; direct: 4; range: 0             */
+  int slot_bytes;      /* buckets: 16 or 8; direct: 4; range: 0; rank: 16   */
   int64_t lo, span;    /* flat forms: id range [lo, lo + span)              */
-  int64_t delta;       /* range: value = key + delta                        */
+  int64_t delta;       /* range: value = key + delta; rank: rank + delta    */
   int64_t table_bytes; /* device memory the build needs (128-byte aligned)  */
 } shmt_hashmap_layout;
 int64_t shmt_hashmap_plan_scratch_bytes(int64_t n);

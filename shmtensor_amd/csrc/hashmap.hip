@@ -153,11 +153,12 @@ struct KeyStats {
   long long kmin, kmax, vmin, vmax;
   unsigned long long not_affine;  // != 0: value - key differs between pairs
   unsigned long long distinct;    // range candidates only: number of different keys
+  unsigned long long not_ranked;  // != 0: keys do not ascend strictly, or value i is not value 0 + i
 };
 
 constexpr int kStatBlocks = 1024;          // workgroups of a sweep, each leaving one partial result
 constexpr int64_t kStatPartialsOff = 256;  // scratch layout: header, partials, then one mark byte per id
-constexpr int64_t kStatMarksOff = kStatPartialsOff + ((kStatBlocks * 48 + 255) & ~255);
+constexpr int64_t kStatMarksOff = kStatPartialsOff + ((kStatBlocks * sizeof(KeyStats) + 255) & ~255ll);
 
 __device__ __forceinline__ int64_t wave_min64(int64_t v) {
 #pragma unroll
@@ -186,6 +187,7 @@ __device__ __forceinline__ KeyStats block_combine(KeyStats mine) {
   mine.vmin = wave_min64(mine.vmin);
   mine.vmax = wave_max64(mine.vmax);
   mine.not_affine = __builtin_amdgcn_ballot_w64(mine.not_affine != 0) != 0;
+  mine.not_ranked = __builtin_amdgcn_ballot_w64(mine.not_ranked != 0) != 0;
   mine.distinct = wave_last(wave_inclusive_scan(static_cast<uint64_t>(mine.distinct)));
   if (lane_id() == 0) per_wave[threadIdx.x / kWave] = mine;
   __syncthreads();
@@ -198,6 +200,7 @@ __device__ __forceinline__ KeyStats block_combine(KeyStats mine) {
       all.vmin = o.vmin < all.vmin ? o.vmin : all.vmin;
       all.vmax = o.vmax > all.vmax ? o.vmax : all.vmax;
       all.not_affine |= o.not_affine;
+      all.not_ranked |= o.not_ranked;
       all.distinct += o.distinct;
     }
   }
@@ -205,12 +208,13 @@ __device__ __forceinline__ KeyStats block_combine(KeyStats mine) {
 }
 
 __device__ __forceinline__ KeyStats neutral_stats() {
-  return KeyStats{INT64_MAX, INT64_MIN, INT64_MAX, INT64_MIN, 0, 0};
+  return KeyStats{INT64_MAX, INT64_MIN, INT64_MAX, INT64_MIN, 0, 0, 0};
 }
 
 __global__ __launch_bounds__(256) void key_stats_kernel(const void *keys, const void *vals, int64_t n,
                                                         int key_bytes, int val_bytes, KeyStats *partials) {
-  const int64_t delta0 = load_int(vals, 0, val_bytes) - load_int(keys, 0, key_bytes);
+  const int64_t v0 = load_int(vals, 0, val_bytes);
+  const int64_t delta0 = v0 - load_int(keys, 0, key_bytes);
   KeyStats mine = neutral_stats();
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
@@ -220,6 +224,8 @@ __global__ __launch_bounds__(256) void key_stats_kernel(const void *keys, const 
     mine.vmin = v < mine.vmin ? v : mine.vmin;
     mine.vmax = v > mine.vmax ? v : mine.vmax;
     mine.not_affine |= (v - k != delta0);
+    // the neighbour's key is the load of the thread next door: served by the caches
+    mine.not_ranked |= (v != v0 + i) || (i > 0 && load_int(keys, i - 1, key_bytes) >= k);
   }
   const KeyStats all = block_combine(mine);
   if (threadIdx.x == 0) partials[blockIdx.x] = all;
@@ -237,6 +243,7 @@ __global__ __launch_bounds__(256) void stats_merge_kernel(const KeyStats *partia
     mine.vmin = o.vmin < mine.vmin ? o.vmin : mine.vmin;
     mine.vmax = o.vmax > mine.vmax ? o.vmax : mine.vmax;
     mine.not_affine |= o.not_affine;
+    mine.not_ranked |= o.not_ranked;
     mine.distinct += o.distinct;
   }
   const KeyStats all = block_combine(mine);
@@ -303,6 +310,36 @@ __global__ __launch_bounds__(256) void direct_build_kernel(int32_t *table, int64
     const uint64_t off = static_cast<uint64_t>(load_int(keys, i, key_bytes) - lo);
     if (off < static_cast<uint64_t>(span)) table[off] = static_cast<int32_t>(load_int(vals, i, val_bytes));
   }
+}
+
+// Rank form: one thread per 16-byte block = 96 consecutive ids. The keys
+// ascend, so the thread finds the first key of its block by bisection (that
+// index is the number of keys below the block) and walks the keys from there
+// while they stay inside the block. Every block is written whole, the empty
+// ones too: no clearing pass and no atomics.
+__global__ __launch_bounds__(256) void rank_build_kernel(uint4 *table, int64_t nblocks, int64_t lo,
+                                                         const void *keys, int64_t n, int key_bytes) {
+  const int64_t b = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (b >= nblocks) return;
+  const int64_t first_id = lo + b * kRankIdsPerBlock;
+  int64_t below = 0, above = n;  // keys[below - 1] < first_id <= keys[above]
+  while (below < above) {
+    const int64_t mid = below + (above - below) / 2;
+    if (load_int(keys, mid, key_bytes) < first_id)
+      below = mid + 1;
+    else
+      above = mid;
+  }
+  uint32_t bits[3] = {0, 0, 0};
+  for (int64_t j = below; j < n; ++j) {
+    const uint64_t r = static_cast<uint64_t>(load_int(keys, j, key_bytes) - first_id);
+    if (r >= static_cast<uint64_t>(kRankIdsPerBlock)) break;
+    const uint32_t bit = 1u << (r & 31);
+    bits[0] |= r < 32 ? bit : 0u;
+    bits[1] |= (r >= 32 && r < 64) ? bit : 0u;
+    bits[2] |= r >= 64 ? bit : 0u;
+  }
+  table[b] = make_uint4(static_cast<uint32_t>(below), bits[0], bits[1], bits[2]);
 }
 
 // Bulk query: a wave owns 64 consecutive requests. The eight bucket loads of
@@ -416,6 +453,19 @@ int shmt_hashmap_plan(const void *keys, const void *vals, int64_t n, int key_byt
       return SHMT_OK;
     }
   }
+  // pairs in ascending key order with consecutive values: bitmap with running counts, 16 bytes per 96 ids,
+  // while that stays within twice the bucket table's size (ids up to 190 times as many as keys)
+  const int64_t rank_bytes = ((span + kRankIdsPerBlock - 1) / kRankIdsPerBlock * 16 + kBucketBytes - 1) /
+                             kBucketBytes * kBucketBytes;
+  if (!st.not_ranked && n < (1ll << 32) && rank_bytes <= 2 * layout->table_bytes) {
+    layout->kind = SHMT_MAP_RANK;
+    layout->slot_bytes = 16;
+    layout->lo = st.kmin;
+    layout->span = span;
+    layout->delta = st.vmin;  // the first pair holds the smallest key and the smallest value
+    layout->table_bytes = rank_bytes;
+    return SHMT_OK;
+  }
   // direct table while it stays within twice the bucket table's size (ids up to 8 times as many as
   // keys when both fit 32 bits): one load per lookup instead of a cooperative probe sequence
   if (vals32 && span * 4 <= 2 * layout->table_bytes) {
@@ -449,7 +499,7 @@ int shmt_hashmap_create_planned(shmt_hashmap_t **out, const shmt_hashmap_layout 
     return build_buckets(out, layout->slot_bytes, keys, vals, n, key_bytes, val_bytes, load_factor, table_mem,
                          table_bytes, stream);
   }
-  SHMT_REQUIRE(layout->kind == SHMT_MAP_DIRECT || layout->kind == SHMT_MAP_RANGE,
+  SHMT_REQUIRE(layout->kind == SHMT_MAP_DIRECT || layout->kind == SHMT_MAP_RANGE || layout->kind == SHMT_MAP_RANK,
                "shmt_hashmap_create_planned: unknown layout kind %d", layout->kind);
   SHMT_REQUIRE(n > 0 && keys != nullptr && vals != nullptr && layout->lo >= 0 && layout->span > 0,
                "shmt_hashmap_create_planned: a flat layout needs keys and a non-negative id range");
@@ -469,6 +519,19 @@ int shmt_hashmap_create_planned(shmt_hashmap_t **out, const shmt_hashmap_layout 
                        val_bytes);
     SHMT_LAUNCH_CHECK();
   }
+  if (layout->kind == SHMT_MAP_RANK) {
+    const int64_t nblocks = (layout->span + kRankIdsPerBlock - 1) / kRankIdsPerBlock;
+    if (table_mem == nullptr || table_bytes < layout->table_bytes || layout->table_bytes < nblocks * 16) {
+      set_error("shmt_hashmap_create_planned: table_mem too small (%lld < %lld bytes)",
+                static_cast<long long>(table_bytes), static_cast<long long>(layout->table_bytes));
+      return SHMT_ENOMEM;
+    }
+    SHMT_REQUIRE((reinterpret_cast<uintptr_t>(table_mem) & 127) == 0,
+                 "shmt_hashmap_create_planned: table_mem must be 128-byte aligned");
+    hipLaunchKernelGGL(rank_build_kernel, dim3(grid_for(nblocks, 256)), dim3(256), 0, s,
+                       static_cast<uint4 *>(table_mem), nblocks, layout->lo, keys, n, key_bytes);
+    SHMT_LAUNCH_CHECK();
+  }
   shmt_hashmap *h = static_cast<shmt_hashmap *>(calloc(1, sizeof(shmt_hashmap)));
   if (h == nullptr) {
     set_error("shmt_hashmap_create_planned: out of host memory");
@@ -477,7 +540,8 @@ int shmt_hashmap_create_planned(shmt_hashmap_t **out, const shmt_hashmap_layout 
   h->view = empty_map_view();
   h->view.buckets = static_cast<const uint4 *>(table_mem);
   h->view.key32 = (key_bytes == 4);
-  h->view.kind = layout->kind == SHMT_MAP_DIRECT ? kKindDirect : kKindRange;
+  h->view.kind = layout->kind == SHMT_MAP_DIRECT ? kKindDirect
+                 : layout->kind == SHMT_MAP_RANK ? kKindRank : kKindRange;
   h->view.lo = layout->lo;
   h->view.span = layout->span;
   h->view.delta = layout->delta;
@@ -486,7 +550,7 @@ int shmt_hashmap_create_planned(shmt_hashmap_t **out, const shmt_hashmap_layout 
   h->key_bytes = key_bytes;
   h->val_bytes = val_bytes;
   h->n = n;
-  h->table_bytes = layout->kind == SHMT_MAP_DIRECT ? layout->table_bytes : 0;
+  h->table_bytes = layout->kind == SHMT_MAP_RANGE ? 0 : layout->table_bytes;
   *out = h;
   return SHMT_OK;
 }

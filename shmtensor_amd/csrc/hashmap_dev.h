@@ -14,9 +14,10 @@
 // probe sequence that still has a free slot, so a lookup stops at the first
 // bucket that contains either the key or an empty slot.
 //
-// Two flat forms exist beside the bucket table, chosen when the map is built
-// from what its keys look like (node ids are dense small integers, and caches
-// of re-numbered graphs hold an id range):
+// Three flat forms exist beside the bucket table, chosen when the map is built
+// from what its keys look like (node ids are dense small integers, caches of
+// re-numbered graphs hold an id range, and a cache built in id order numbers
+// its rows by rank):
 //   direct (kKindDirect): keys lie in [lo, lo + span) with span a small
 //                     multiple of their number; the table is int32
 //                     value[key - lo], -1 where no key was given. One 4-byte
@@ -24,6 +25,13 @@
 //   range  (kKindRange) : the keys are exactly the ids lo .. lo + span - 1 and
 //                     every value is key + delta; lookups are arithmetic and
 //                     touch no memory at all.
+//   rank   (kKindRank)  : the pairs came in ascending key order with values
+//                     v0, v0 + 1, v0 + 2, ...: the value is the key's rank
+//                     among the keys (+ delta = v0). The table is a bitmap
+//                     with running counts, 16-byte blocks {uint32 keys below
+//                     this block, 96 presence bits}: one 16-byte load per
+//                     lookup from a table of span / 6 bytes, which stays in
+//                     the caches where a 4-byte-per-id table does not.
 #pragma once
 #include "wave.h"
 
@@ -34,10 +42,13 @@ enum SlotFormat : int { kSlot16 = 16, kSlot8 = 8 };
 constexpr int kProbeGroup = 8;      // lanes that cooperate on one key
 constexpr int kBucketBytes = 128;
 
-enum MapKind : int { kKindBuckets = 0, kKindDirect = 1, kKindRange = 2 };
+enum MapKind : int { kKindBuckets = 0, kKindDirect = 1, kKindRange = 2, kKindRank = 3 };
+
+constexpr int kRankIdsPerBlock = 96;  // presence bits of one 16-byte rank block
 
 struct MapView {
-  const uint4 *buckets;   // bucket table: nbuckets * 8 uint4; direct form: int32 values[span]
+  const uint4 *buckets;   // bucket table: nbuckets * 8 uint4; direct form: int32 values[span];
+                          // rank form: one uint4 block per 96 ids
   uint32_t nbuckets;
   int key32;              // 1: keys are int32 -> requests are narrowed before the lookup
   int kind;               // MapKind
@@ -45,7 +56,7 @@ struct MapView {
                           //    does not fit 32 bits is absent
   int64_t lo;             // flat forms: smallest key
   int64_t span;           // flat forms: keys lie in [lo, lo + span)
-  int64_t delta;          // range form: value = key + delta
+  int64_t delta;          // range form: value = key + delta; rank form: value = rank + delta
 };
 
 inline MapView empty_map_view() { return MapView{nullptr, 1, 0, kKindBuckets, 0, 0, 0, 0}; }
@@ -65,6 +76,18 @@ __device__ __forceinline__ int64_t flat_find(const MapView &m, int64_t key) {
   const uint64_t off = static_cast<uint64_t>(key) - static_cast<uint64_t>(m.lo);  // key < lo wraps around
   if (off >= static_cast<uint64_t>(m.span)) return -1;
   if (m.kind == kKindRange) return key + m.delta;
+  if (m.kind == kKindRank) {
+    const uint64_t blk = off / kRankIdsPerBlock;
+    const uint32_t r = static_cast<uint32_t>(off - blk * kRankIdsPerBlock);
+    const uint4 b = m.buckets[blk];  // x: keys below this block; y, z, w: presence of ids 0-31, 32-63, 64-95
+    const uint32_t word = r < 32 ? b.y : (r < 64 ? b.z : b.w);
+    const uint32_t bit = r & 31;
+    if (((word >> bit) & 1u) == 0) return -1;
+    uint32_t below = __builtin_popcount(word & ((1u << bit) - 1u));
+    if (r >= 32) below += __builtin_popcount(b.y);
+    if (r >= 64) below += __builtin_popcount(b.z);
+    return static_cast<int64_t>(b.x + below) + m.delta;
+  }
   return static_cast<int64_t>(reinterpret_cast<const int32_t *>(m.buckets)[off]);
 }
 

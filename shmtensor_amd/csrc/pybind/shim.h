@@ -182,8 +182,10 @@ class StaticHashmap {
   }
   int64_t capacity() const { return capacity_; }
   int64_t memory_usage() const { return memory_usage_; }
-  // "buckets", "direct" or "range": the layout the constructor chose for these keys
-  std::string layout() const { return kind_ == SHMT_MAP_RANGE ? "range" : kind_ == SHMT_MAP_DIRECT ? "direct" : "buckets"; }
+  // "buckets", "direct", "range" or "rank": the layout the constructor chose for these keys
+  std::string layout() const {
+    return kind_ == SHMT_MAP_RANGE ? "range" : kind_ == SHMT_MAP_DIRECT ? "direct" : kind_ == SHMT_MAP_RANK ? "rank" : "buckets";
+  }
   const shmt_hashmap_t *handle() const { return handle_; }
 
  private:

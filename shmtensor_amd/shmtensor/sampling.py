@@ -313,7 +313,9 @@ class GPUSamplingDataloader:
         size = degrees[candidates] * self.indices.element_size() + self.indptr.element_size() + 1.25 * 2 * 4
         prefix = torch.cumsum(size, dim=0)
         cache_size = torch.searchsorted(prefix, cache_capacity).item()
-        candidates = candidates[:cache_size].cuda()
+        # the cached rows are kept in id order: a node's slot is then its rank among the cached ids, which the
+        # map stores as a bitmap with running counts instead of a table (samples do not depend on the slot)
+        candidates = torch.sort(candidates[:cache_size]).values.cuda()
         if candidates.numel() > 0:
             self.gpu_indptr, self.gpu_indices = capi.create_subcsr(self.indptr, self.indices, candidates)
             self.hashmap = capi.CUCOStaticHashmap(

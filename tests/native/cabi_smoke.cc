@@ -258,17 +258,19 @@ int main() {
     for (size_t i = 0; i < all.size(); ++i) EXPECT(lab2[i] == first2[all[i]]);
   }
 
-  // ---- map layouts chosen from the keys: id range, direct table, bucket table ----
+  // ---- map layouts chosen from the keys: id range, direct table, rank bitmap ----
   {
     const int64_t m = 50000;
-    std::vector<int64_t> rk(m), rv(m), dk(m), dv(m);
+    std::vector<int64_t> rk(m), rv(m), dk(m), dv(m), bk(m), bv(m);
     for (int64_t i = 0; i < m; ++i) {
       rk[i] = 700 + i;       // ids 700 .. 50,699 -> slot id - 700: a range
       rv[i] = i;
       dk[i] = 3 * i + 5;     // every third id: a direct table over the id universe
       dv[i] = m - 1 - i;
+      bk[i] = 7 * i + 3 + (i % 5);  // ascending ids with consecutive slots from 11 on: ranks
+      bv[i] = 11 + i;
     }
-    struct Case { std::vector<int64_t> *k, *v; int kind; } cases[2] = {{&rk, &rv, SHMT_MAP_RANGE}, {&dk, &dv, SHMT_MAP_DIRECT}};
+    struct Case { std::vector<int64_t> *k, *v; int kind; } cases[3] = {{&rk, &rv, SHMT_MAP_RANGE}, {&dk, &dv, SHMT_MAP_DIRECT}, {&bk, &bv, SHMT_MAP_RANK}};
     const int64_t sbytes = shmt_hashmap_plan_scratch_bytes(m);
     void *d_ps = nullptr;
     HIP_OK(hipMalloc(&d_ps, sbytes));
@@ -283,7 +285,7 @@ int main() {
       SHMT_OK_(shmt_hashmap_create_planned(&pm, &lay, dk_, dv_, m, 8, 8, 0.8, d_t, lay.table_bytes, stream));
       EXPECT(shmt_hashmap_kind(pm) == c.kind);
       std::vector<int64_t> rq(100001);
-      for (auto &x : rq) x = static_cast<int64_t>(rnd() % 200000) - 100;
+      for (auto &x : rq) x = static_cast<int64_t>(rnd() % 400000) - 100;
       int64_t *d_rq = to_device(rq), *d_rr = nullptr;
       HIP_OK(hipMalloc(&d_rr, rq.size() * 8));
       SHMT_OK_(shmt_hashmap_query(pm, d_rq, 8, static_cast<int64_t>(rq.size()), d_rr, stream));

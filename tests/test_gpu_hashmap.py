@@ -117,12 +117,14 @@ def _probe_requests(rng, keys, lo, hi):
 
 _LAYOUT_CASES = ["range_identity", "range_offset", "range_shuffled", "range_from_zero_one_key", "range_with_repeat",
                  "range_negative_values", "direct_permuted", "direct_sparse", "direct_too_sparse", "negative_keys",
-                 "values_beyond_32_bits"]
+                 "values_beyond_32_bits", "rank_sorted_sparse", "rank_offset_values", "rank_values_beyond_32_bits",
+                 "rank_one_id_in_100", "rank_too_sparse", "rank_block_edges", "rank_broken_by_one_value",
+                 "rank_broken_by_order"]
 
 
 @pytest.mark.parametrize("kd,vd,case", [(kd, vd, case) for kd in (np.int32, np.int64) for vd in (np.int32, np.int64)
                                         for case in _LAYOUT_CASES
-                                        if not (case == "values_beyond_32_bits" and vd is np.int32)])
+                                        if not (case.endswith("values_beyond_32_bits") and vd is np.int32)])
 def test_layouts_answer_like_a_dict(capi, oracle, kd, vd, case):
     rng = np.random.default_rng(len(case) * 7 + np.dtype(kd).itemsize + 3 * np.dtype(vd).itemsize)
     n = 30_000
@@ -168,10 +170,45 @@ def test_layouts_answer_like_a_dict(capi, oracle, kd, vd, case):
         keys = keys[keys != -1]                      # -1 is the empty key
         vals = np.arange(keys.size)
         expect_layout = "buckets"
-    else:                                            # dense keys whose values need 64 bits
+    elif case == "values_beyond_32_bits":            # dense keys whose values need 64 bits
         keys = rng.permutation(n)
         vals = np.arange(n) + 2**33
         expect_layout = "buckets"
+    elif case == "rank_sorted_sparse":               # a cache kept in id order: slot = rank of the id
+        keys = np.sort(rng.choice(3 * n, size=n, replace=False)) + 12345
+        vals = np.arange(n)
+        expect_layout = "rank"
+    elif case == "rank_offset_values":
+        keys = np.sort(rng.choice(10 * n, size=n, replace=False))
+        vals = np.arange(n) + 77
+        expect_layout = "rank"
+    elif case == "rank_values_beyond_32_bits":       # ranks are computed, so wide values cost nothing
+        keys = np.sort(rng.choice(5 * n, size=n, replace=False))
+        vals = np.arange(n) + 2**33
+        expect_layout = "rank"
+    elif case == "rank_one_id_in_100":               # most 96-id blocks hold no key or one
+        keys = np.sort(rng.choice(100 * n, size=n, replace=False))
+        vals = np.arange(n)
+        expect_layout = "rank"
+    elif case == "rank_too_sparse":                  # 1 id in 400: the bitmap would outgrow the bucket table
+        keys = np.sort(rng.choice(400 * n, size=n, replace=False))
+        vals = np.arange(n)
+        expect_layout = "buckets"
+    elif case == "rank_block_edges":                 # first / last id of the 96-id blocks and of their 32-bit words
+        a = np.sort(rng.choice(4000, size=1500, replace=False))[:, None] * 96
+        keys = np.unique((a + np.array([0, 31, 32, 63, 64, 95])[None, :]).ravel()) + 5
+        vals = np.arange(keys.size)
+        expect_layout = "rank"
+    elif case == "rank_broken_by_one_value":         # ascending ids, but two slots swapped: a plain table again
+        keys = np.sort(rng.choice(3 * n, size=n, replace=False))
+        vals = np.arange(n)
+        vals[[100, 20_000]] = vals[[20_000, 100]]
+        expect_layout = "direct"
+    else:                                            # consecutive values, but two ids out of order
+        keys = np.sort(rng.choice(3 * n, size=n, replace=False))
+        keys[[7, 8]] = keys[[8, 7]]
+        vals = np.arange(n)
+        expect_layout = "direct"
     keys, vals = keys.astype(kd), vals.astype(vd)
     h = capi.CUCOStaticHashmap(_cuda(keys), _cuda(vals), 0.8)
     assert h.layout() == expect_layout
@@ -196,6 +233,8 @@ def test_layouts_answer_like_a_dict(capi, oracle, kd, vd, case):
         assert h.memory_usage() == 0
     elif expect_layout == "direct":
         assert h.memory_usage() <= (hi - lo + 1) * 4 + 128
+    elif expect_layout == "rank":
+        assert h.memory_usage() <= (hi - lo + 1 + 95) // 96 * 16 + 128
 
 
 def test_wide_dtypes_with_small_ids_use_narrow_slots(capi, oracle):
@@ -213,13 +252,15 @@ def test_wide_dtypes_with_small_ids_use_narrow_slots(capi, oracle):
     assert np.array_equal(wide.query(_cuda(req)).cpu().numpy(), oracle.Hashmap(keys + 2**32, vals, 0.5).query(req))
 
 
-@pytest.mark.parametrize("layout", ["range", "direct"])
+@pytest.mark.parametrize("layout", ["range", "direct", "rank"])
 def test_flat_layouts_route_fetch_set_and_sampling(capi, oracle, layout):
     """cache_fetch / cache_set / csr_cache_sampling through a map in a flat layout against the oracle, with
     cache rows made different from the host rows so that routing shows."""
     rng = np.random.default_rng(8)
     n, c = 5000, 2000
     ids = np.arange(100, 100 + c) if layout == "range" else rng.choice(n, size=c, replace=False)
+    if layout == "rank":
+        ids = np.sort(ids)
     slots = ids - 100 if layout == "range" else np.arange(c)
     h = capi.CUCOStaticHashmap(_cuda(ids), _cuda(slots), 0.8)
     assert h.layout() == layout
