@@ -218,7 +218,7 @@ int shmt_inclusive_scan_i32(void *data, int64_t len, void *tmp,
  * cub_exclusiveSum allocates its temporary storage on every call,
  * src/tensor_relabel.cu:15-25); it is for callers that cannot allocate:
  * code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc. The tile counter and tile words live in a 256 KiB array that is
+ * hipMalloc. The sums its tiles publish live in a 260 KiB array that is
  * part of the library's code object (one copy per GPU, held until the process
  * ends), so
  * len is limited to SHMT_SCAN_NOALLOC_MAX_LEN elements; longer inputs are

@@ -7,12 +7,14 @@
 // LDS word per wave. Device level: inputs up to kSingleBlockMax elements are
 // scanned by one 1024-thread workgroup that walks the array with a running
 // carry (one launch). Larger inputs are scanned in ONE pass over the data
-// (read once, written once): every workgroup takes the next tile from a
-// counter, scans it locally, publishes the tile's sum, and obtains the sum of
-// everything before its tile by looking back over the sums (or, where
-// available, the finished prefixes) that the tiles before it have published.
-// A tile only ever waits for tiles with smaller numbers, which were handed
-// out earlier to workgroups that are already running, so the waiting ends.
+// (read once, written once) by a grid no larger than the device holds at
+// once: workgroup b takes tiles b, b + grid, b + 2 grid, ..., scans each
+// locally, publishes the tile's sum, and obtains the sum of everything before
+// the tile from the sums that the tiles before it have published (per tile,
+// per group of 64 tiles, per run of 64 groups). A tile only ever waits for
+// tiles with smaller numbers; the smallest unfinished tile belongs to a
+// workgroup whose earlier tiles are all done, so it is being worked on and
+// waits for nothing unfinished: the waiting ends.
 #include <mutex>
 
 #include "common.h"
@@ -47,76 +49,112 @@ int launch_scan_partials(uint64_t *partials, int64_t nb, hipStream_t s) {
 }
 
 // ---- single-pass device scan ---------------------------------------------------
-// What a tile has published so far lives in two 64-bit words per tile, each
-// {state : 32 | half of a 64-bit sum : 32}: state 0 = nothing yet, 1 = the
-// tile's own sum, 2 = the sum of everything up to and including the tile.
-// A reader takes a value only when both words carry the same non-zero state,
-// so the two halves always belong together and no fence is needed: the payload
-// travels inside the (relaxed, device-scope) atomic accesses themselves.
+// What the tiles publish lives in 64-bit word pairs, each word {state : 32 |
+// half of a 64-bit sum : 32}: state 0 = nothing yet, 1 = published. A reader
+// takes a value only when both words carry the state, so the two halves
+// always belong together and no fence is needed: the payload travels inside
+// the (relaxed, device-scope) atomic accesses themselves.
 //
-// Tiles are large (128 KiB): finished prefixes spread along the tiles at one
-// look-back step (64 tiles) per memory round trip, and with small tiles that
-// spreading, not the memory bandwidth, bounds the scan. Measured for
-// 16,777,216 int64 (reduce / scan / apply in three launches, which this
-// replaces: 125 us): 16 KiB tiles 204 us, 64 KiB 78 us, 128 KiB 64 us, 256 KiB
-// 114 us (registers); inspecting 128 or 256 tiles per step gained nothing.
-constexpr uint32_t kTileSum = 1, kTilePrefix = 2;
-constexpr int64_t kScanHeaderBytes = 64;       // tile counter (+ padding) in front of the tile words
+// Three levels of sums keep the look-back at two or three dependent steps
+// wherever a tile lies: every tile publishes its own sum; the last tile of
+// each aligned group of 64 tiles also publishes the group's sum (its own plus
+// the 63 before it, which it reads anyway); the last tile of each aligned run
+// of 64 groups publishes that run's sum. A tile's prefix is then: tiles before
+// it in its group + groups before its group in the run + runs before its run,
+// three reads of at most 64 entries that are issued together.
+//
+// Measured on MI355X, 16,777,216 int64 in place (268 MB of traffic): a
+// publish -> read step between workgroups takes tens of microseconds while the
+// memory queues are full of tile traffic, so the scan wants few, large tiles
+// and few levels: tiles of 16 / 32 / 64 / 128 KiB 216 / 90 / 57 / 52 us
+// (256 KiB: 111 us, the tile no longer fits the registers); groups of 16 or 8
+// instead of 64 (one level more for the same tiles) 67 / 112 us. Without
+// effect: requesting the workgroup's next tile before the look-back, one
+// 128-byte line per published entry, 256 instead of 512 workgroups. Walking
+// back over single tiles with a tile counter (the earlier form) took 64 us.
+constexpr uint32_t kPublished = 1;
 constexpr uint32_t kLookbackSpinLimit = 1u << 24;  // a wait that long means a tile before this one died
-constexpr int kLbBlock = 512;                  // threads per tile
+constexpr int kLbBlock = 1024;                 // threads per tile
 constexpr int kLbWaves = kLbBlock / kWave;
-constexpr int kLbChunks = 16;                  // 16-byte vectors per lane
-constexpr int kLbLook = 1;                     // tiles a lane inspects per look-back step
+constexpr int kLbChunks = 8;                   // 16-byte vectors per lane
 constexpr int64_t kLbTileBytes = static_cast<int64_t>(kLbWaves) * kLbChunks * kWave * 16;
+constexpr int kLbFan = kWave;                  // tiles per group, groups per run
 
 struct ScanState {
-  unsigned long long *counter;  // next tile to hand out
-  uint64_t *words;              // 2 per tile
+  uint64_t *tiles;              // 2 words per tile
+  uint64_t *groups;             // 2 words per group of 64 tiles
+  uint64_t *runs;               // 2 words per run of 64 groups
 };
 
-__device__ __forceinline__ void tile_publish(const ScanState &st, int64_t tile, uint32_t state, uint64_t sum) {
-  const uint64_t tag = static_cast<uint64_t>(state) << 32;
-  __hip_atomic_store(&st.words[2 * tile], tag | (sum & 0xFFFFFFFFull), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(&st.words[2 * tile + 1], tag | (sum >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+struct ScanTmpLayout {
+  int64_t nb, ng, nr, tiles_off, groups_off, runs_off, total;
+};
+
+static ScanTmpLayout scan_tmp_layout(int64_t nb) {
+  ScanTmpLayout l;
+  l.nb = nb;
+  l.ng = (nb + kLbFan - 1) / kLbFan;
+  l.nr = (l.ng + kLbFan - 1) / kLbFan;
+  l.tiles_off = 0;
+  l.groups_off = l.tiles_off + nb * 16;
+  l.runs_off = l.groups_off + l.ng * 16;
+  l.total = l.runs_off + l.nr * 16;
+  return l;
 }
 
-// Sum of all tiles before `tile` (tile >= 1), by one whole wave: in every step
-// lane l looks at the tiles (look - l - 64 j), j < kLbLook; the nearest tile
-// that already knows its prefix ends the walk, the own sums of the tiles in
-// between are added up.
-__device__ __forceinline__ uint64_t tile_lookback(const ScanState &st, int64_t tile) {
+__device__ __forceinline__ void sum_publish(uint64_t *words, int64_t i, uint64_t sum) {
+  const uint64_t tag = static_cast<uint64_t>(kPublished) << 32;
+  __hip_atomic_store(&words[2 * i], tag | (sum & 0xFFFFFFFFull), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(&words[2 * i + 1], tag | (sum >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Reads entry i when `want`; false while it is not published yet.
+__device__ __forceinline__ bool sum_read(const uint64_t *words, int64_t i, bool want, uint64_t *sum) {
+  *sum = 0;
+  if (!want) return true;
+  const uint64_t w0 = __hip_atomic_load(&words[2 * i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t w1 = __hip_atomic_load(&words[2 * i + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  *sum = (w1 << 32) | (w0 & 0xFFFFFFFFull);
+  return static_cast<uint32_t>(w0 >> 32) == kPublished && static_cast<uint32_t>(w1 >> 32) == kPublished;
+}
+
+__device__ __forceinline__ uint64_t wave_sum_all(uint64_t v) { return wave_last(wave_inclusive_scan(v)); }
+
+// Sum of all tiles before `tile`, by one whole wave; `own` is the tile's own
+// sum (already published). Publishes the sums of the group and of the run
+// that end with this tile. A tile only waits for entries that tiles with
+// smaller numbers publish, which were handed out earlier to workgroups that
+// are already running, so the waiting ends.
+__device__ __forceinline__ uint64_t tile_lookback(const ScanState &st, int64_t tile, uint64_t own) {
   const int lane = lane_id();
-  uint64_t prefix = 0;
+  const int64_t group = tile / kLbFan, run = group / kLbFan;
+  const int in_group = static_cast<int>(tile % kLbFan), in_run = static_cast<int>(group % kLbFan);
+  // runs before this tile's run: at most 64 up to 262,144 tiles, in further steps of 64 beyond
+  uint64_t far = 0;
   uint32_t spins = 0;
-  for (int64_t look = tile - 1;; look -= kWave * kLbLook) {
-    uint32_t state[kLbLook];
-    uint64_t sum[kLbLook];
-    for (;;) {
-      bool ready = true;
-#pragma unroll
-      for (int j = 0; j < kLbLook; ++j) {
-        const int64_t t = look - lane - kWave * j;
-        state[j] = kTilePrefix;  // in front of tile 0: an empty prefix
-        sum[j] = 0;
-        if (t >= 0) {
-          const uint64_t w0 = __hip_atomic_load(&st.words[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint64_t w1 = __hip_atomic_load(&st.words[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          state[j] = static_cast<uint32_t>(w0 >> 32);
-          ready = ready && state[j] != 0 && state[j] == static_cast<uint32_t>(w1 >> 32);
-          sum[j] = (w1 << 32) | (w0 & 0xFFFFFFFFull);
-        }
-      }
-      if (__builtin_amdgcn_ballot_w64(!ready) == 0 || ++spins >= kLookbackSpinLimit) break;
-      __builtin_amdgcn_s_sleep(1);
-    }
-#pragma unroll
-    for (int j = 0; j < kLbLook; ++j) {
-      const uint64_t done = __builtin_amdgcn_ballot_w64(state[j] == kTilePrefix);
-      const int last = done ? __builtin_ctzll(done) : kWave - 1;  // nearest tile with a finished prefix
-      prefix += wave_last(wave_inclusive_scan(lane <= last ? sum[j] : static_cast<uint64_t>(0)));
-      if (done) return prefix;
-    }
+  for (int64_t first = kWave; first < run; first += kWave) {
+    uint64_t part = 0;
+    while (!sum_read(st.runs, first + lane, first + lane < run, &part) && ++spins < kLookbackSpinLimit)
+      __builtin_amdgcn_s_sleep(8);
+    far += part;
   }
+  // a lane asks again only for what it has not seen published yet
+  uint64_t a = 0, b = 0, c = 0;
+  bool ok_a = false, ok_b = false, ok_c = false;
+  for (;;) {
+    if (!ok_a) ok_a = sum_read(st.tiles, group * kLbFan + lane, lane < in_group, &a);
+    if (!ok_b) ok_b = sum_read(st.groups, run * kLbFan + lane, lane < in_run, &b);
+    if (!ok_c) ok_c = sum_read(st.runs, lane, lane < run, &c);
+    if (__builtin_amdgcn_ballot_w64(!(ok_a && ok_b && ok_c)) == 0 || ++spins >= kLookbackSpinLimit) break;
+    __builtin_amdgcn_s_sleep(8);
+  }
+  c += far;
+  const uint64_t tiles_before = wave_sum_all(a), groups_before = wave_sum_all(b), runs_before = wave_sum_all(c);
+  if (lane == 0 && in_group == kLbFan - 1) {
+    sum_publish(st.groups, group, tiles_before + own);
+    if (in_run == kLbFan - 1) sum_publish(st.runs, run, groups_before + tiles_before + own);
+  }
+  return tiles_before + groups_before + runs_before;
 }
 
 __global__ __launch_bounds__(256) void scan_state_clear_kernel(uint64_t *p, int64_t n) {
@@ -136,24 +174,12 @@ struct alignas(16) ScanVec {
 // front of the first 16-byte boundary of the caller's array (`head`, n_head of
 // them) are scanned by the first thread of tile 0, and their sum starts the
 // prefix that the tiles hand on.
-template <typename T, bool INCLUSIVE>
-__global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_head, T *data, int64_t len,
-                                                                 ScanState st) {
+template <typename T, int C>
+__device__ __forceinline__ void scan_tile_load(const T *data, int64_t len, int64_t lane_base, bool whole,
+                                               T (&v)[C][16 / sizeof(T)]) {
   constexpr int V = 16 / sizeof(T);
-  constexpr int64_t kTileElems = kLbTileBytes / sizeof(T);
-  __shared__ uint64_t wave_total[kLbWaves];
-  __shared__ uint64_t shared[2];  // tile number, then the sum of everything before the tile
-  if (threadIdx.x == 0) shared[0] = atomicAdd(st.counter, 1ull);
-  __syncthreads();
-  const int64_t tile = static_cast<int64_t>(shared[0]);
-  const int wave = threadIdx.x / kWave, lane = lane_id();
-  const int64_t lane_base = tile * kTileElems + static_cast<int64_t>(wave) * kLbChunks * kWave * V + lane * V;
-  const bool whole = (tile + 1) * kTileElems <= len;
-  T v[kLbChunks][V];
-  T excl[kLbChunks];  // sum (mod 2^width) of the tile's elements in front of this lane's vector of chunk c
-  T carry = 0;  // all in-tile sums are taken in the element type: results are defined modulo its width
 #pragma unroll
-  for (int c = 0; c < kLbChunks; ++c) {
+  for (int c = 0; c < C; ++c) {
     const int64_t i = lane_base + static_cast<int64_t>(c) * kWave * V;
     if (whole) {
       const ScanVec<T> x = *reinterpret_cast<const ScanVec<T> *>(data + i);
@@ -164,64 +190,86 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
       for (int e = 0; e < V; ++e) v[c][e] = (i + e < len) ? data[i + e] : static_cast<T>(0);
     }
   }
+}
+
+template <typename T, bool INCLUSIVE>
+__global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_head, T *data, int64_t len,
+                                                                 int64_t nb, ScanState st) {
+  constexpr int V = 16 / sizeof(T);
+  constexpr int64_t kTileElems = kLbTileBytes / sizeof(T);
+  __shared__ uint64_t wave_total[kLbWaves];
+  __shared__ uint64_t shared_before;  // the sum of everything before the tile
+  const int wave = threadIdx.x / kWave, lane = lane_id();
+  const int64_t lane_off = static_cast<int64_t>(wave) * kLbChunks * kWave * V + lane * V;
+  T v[kLbChunks][V];
+  int64_t tile = blockIdx.x;
+  if (tile < nb) scan_tile_load<T, kLbChunks>(data, len, tile * kTileElems + lane_off, (tile + 1) * kTileElems <= len, v);
+  for (; tile < nb; tile += gridDim.x) {
+    const int64_t lane_base = tile * kTileElems + lane_off;
+    const bool whole = (tile + 1) * kTileElems <= len;
+    T excl[kLbChunks];  // sum (mod 2^width) of the tile's elements in front of this lane's vector of chunk c
+    T carry = 0;  // all in-tile sums are taken in the element type: results are defined modulo its width
 #pragma unroll
-  for (int c = 0; c < kLbChunks; ++c) {
-    T mine = 0;
+    for (int c = 0; c < kLbChunks; ++c) {
+      T mine = 0;
 #pragma unroll
-    for (int e = 0; e < V; ++e) mine += v[c][e];
-    const T inc = wave_inclusive_scan(mine);
-    excl[c] = carry + inc - mine;
-    carry += wave_last(inc);
-  }
-  if (lane == 0) wave_total[wave] = carry;
-  __syncthreads();
-  uint64_t in_tile = 0, total = 0;
+      for (int e = 0; e < V; ++e) mine += v[c][e];
+      const T inc = wave_inclusive_scan(mine);
+      excl[c] = carry + inc - mine;
+      carry += wave_last(inc);
+    }
+    const int64_t next = tile + gridDim.x;
+    if (lane == 0) wave_total[wave] = carry;
+    __syncthreads();
+    uint64_t in_tile = 0, total = 0;
 #pragma unroll
-  for (int w = 0; w < kLbWaves; ++w) {
-    const uint64_t t = wave_total[w];
-    if (w < wave) in_tile += t;
-    total += t;
-  }
-  if (threadIdx.x < kWave) {  // the first wave talks to the other tiles
-    uint64_t before = 0;
-    if (tile > 0) {
-      if (threadIdx.x == 0) tile_publish(st, tile, kTileSum, total);
-      before = tile_lookback(st, tile);
-    } else if (threadIdx.x == 0) {
-      T run = 0;
-      for (int k = 0; k < n_head; ++k) {
-        const T x = head[k];
-        head[k] = INCLUSIVE ? run + x : run;
-        run += x;
+    for (int w = 0; w < kLbWaves; ++w) {
+      const uint64_t t = wave_total[w];
+      if (w < wave) in_tile += t;
+      total += t;
+    }
+    if (threadIdx.x < kWave) {  // the first wave talks to the other tiles
+      uint64_t before = 0;
+      if (tile == 0) {
+        T run = 0;
+        if (threadIdx.x == 0) {
+          for (int k = 0; k < n_head; ++k) {
+            const T x = head[k];
+            head[k] = INCLUSIVE ? run + x : run;
+            run += x;
+          }
+        }
+        before = static_cast<uint64_t>(run);  // used by thread 0 only
+        if (threadIdx.x == 0) sum_publish(st.tiles, 0, before + total);
+      } else {
+        if (threadIdx.x == 0) sum_publish(st.tiles, tile, total);
+        before = tile_lookback(st, tile, total);
       }
-      before = static_cast<uint64_t>(run);
+      if (threadIdx.x == 0) shared_before = before;
     }
-    if (threadIdx.x == 0) {
-      tile_publish(st, tile, kTilePrefix, before + total);
-      shared[1] = before;
-    }
-  }
-  __syncthreads();
-  const uint64_t base = shared[1] + in_tile;
+    __syncthreads();
+    const uint64_t base = shared_before + in_tile;
 #pragma unroll
-  for (int c = 0; c < kLbChunks; ++c) {
-    const int64_t i = lane_base + static_cast<int64_t>(c) * kWave * V;
-    T run = static_cast<T>(base) + excl[c];
-    ScanVec<T> out;
+    for (int c = 0; c < kLbChunks; ++c) {
+      const int64_t i = lane_base + static_cast<int64_t>(c) * kWave * V;
+      T run = static_cast<T>(base) + excl[c];
+      ScanVec<T> out;
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      if (INCLUSIVE) run += v[c][e];
-      out.e[e] = run;
-      if (!INCLUSIVE) run += v[c][e];
-    }
-    if (whole) {
-      *reinterpret_cast<ScanVec<T> *>(data + i) = out;
-    } else {
+      for (int e = 0; e < V; ++e) {
+        if (INCLUSIVE) run += v[c][e];
+        out.e[e] = run;
+        if (!INCLUSIVE) run += v[c][e];
+      }
+      if (whole) {
+        *reinterpret_cast<ScanVec<T> *>(data + i) = out;
+      } else {
 #pragma unroll
-      for (int e = 0; e < V; ++e)
-        if (i + e < len) data[i + e] = out.e[e];
+        for (int e = 0; e < V; ++e)
+          if (i + e < len) data[i + e] = out.e[e];
+      }
     }
-  }
+    if (next < nb) scan_tile_load<T, kLbChunks>(data, len, next * kTileElems + lane_off, (next + 1) * kTileElems <= len, v);
+  }  // the barriers above also order the reuse of the LDS words by the next tile
 }
 
 template <typename T, bool INCLUSIVE>
@@ -230,6 +278,27 @@ __global__ __launch_bounds__(1024) void scan_single_kernel(T *data, int64_t len)
   T carry = 0;
   for (int64_t base = 0; base < len; base += 1024 * kScanItems)
     tile_scan_inplace<T, 1024, kScanItems, INCLUSIVE>(data, base, len, lds, &carry);
+}
+
+// Workgroups of `kernel` that the current device holds at once (cached per kernel and device).
+static int resident_workgroups(const void *kernel, int *out) {
+  static std::mutex mu;
+  struct Entry { const void *kernel; int dev, n; };
+  static Entry cache[32];
+  static int used = 0;
+  int dev = -1;
+  SHMT_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  for (int i = 0; i < used; ++i)
+    if (cache[i].kernel == kernel && cache[i].dev == dev) { *out = cache[i].n; return SHMT_OK; }
+  int per_cu = 0, cus = 0;
+  SHMT_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kLbBlock, 0));
+  SHMT_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  SHMT_REQUIRE(per_cu >= 1 && cus >= 1, "scan: the device reports no room for the scan kernel");
+  const int n = per_cu * cus;
+  if (used < 32) cache[used++] = Entry{kernel, dev, n};
+  *out = n;
+  return SHMT_OK;
 }
 
 template <typename T, bool INCLUSIVE>
@@ -247,7 +316,8 @@ static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, hipS
   const int64_t main_len = len - n_head;
   const int64_t tile_elems = kLbTileBytes / static_cast<int64_t>(sizeof(T));
   const int64_t nb = (main_len + tile_elems - 1) / tile_elems;
-  const int64_t need = kScanHeaderBytes + nb * 16;
+  const ScanTmpLayout l = scan_tmp_layout(nb);
+  const int64_t need = l.total;
   if (tmp == nullptr || tmp_bytes < need) {
     set_error("scan: tmp buffer too small (%lld < %lld bytes)", static_cast<long long>(tmp_bytes),
               static_cast<long long>(need));
@@ -256,27 +326,35 @@ static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, hipS
   SHMT_REQUIRE(nb < (1ll << 31), "scan: input too large");
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(tmp) & 7) == 0, "scan: tmp must be 8-byte aligned");
   ScanState st;
-  st.counter = static_cast<unsigned long long *>(tmp);
-  st.words = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + kScanHeaderBytes);
-  // counter and tile words start at zero (a kernel, not a memset, so that the scan can be captured in a graph)
+  st.tiles = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.tiles_off);
+  st.groups = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.groups_off);
+  st.runs = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.runs_off);
+  // the words start at zero (a kernel, not a memset, so that the scan can be captured in a graph)
   hipLaunchKernelGGL(scan_state_clear_kernel, dim3(grid_for(need / 8, 256 * 4)), dim3(256), 0, s,
                      static_cast<uint64_t *>(tmp), need / 8);
   SHMT_LAUNCH_CHECK();
-  hipLaunchKernelGGL((scan_lookback_kernel<T, INCLUSIVE>), dim3(static_cast<unsigned>(nb)), dim3(kLbBlock), 0, s,
-                     data, n_head, main_data, main_len, st);
+  int resident = 0;
+  int rc = resident_workgroups(reinterpret_cast<const void *>(&scan_lookback_kernel<T, INCLUSIVE>), &resident);
+  if (rc) return rc;
+  const unsigned grid = static_cast<unsigned>(nb < resident ? nb : resident);
+  hipLaunchKernelGGL((scan_lookback_kernel<T, INCLUSIVE>), dim3(grid), dim3(kLbBlock), 0, s,
+                     data, n_head, main_data, main_len, nb, st);
   SHMT_LAUNCH_CHECK();
   return SHMT_OK;
 }
 
 // ---- scan without a caller-provided workspace -------------------------------
-// The tile counter and tile words of shmt_exclusive_scan_noalloc live in this array, which
+// The published sums of shmt_exclusive_scan_noalloc live in this array, which
 // is part of the loaded code object: every GPU the library runs on holds its
 // own copy, at its own address, until the process ends. The name below is a
 // host-side handle only; kernels are given the device address that
 // hipGetSymbolAddress returns for the current device.
 constexpr int64_t kStaticScanMaxLen = 1ll << 28;  // 268,435,456 elements
 constexpr int64_t kStaticScanTiles = kStaticScanMaxLen / (kLbTileBytes / 8);
-constexpr int64_t kStaticScanWords = kScanHeaderBytes / 8 + 2 * kStaticScanTiles;  // 256 KiB + 64 B
+constexpr int64_t kStaticScanGroups = kStaticScanTiles / kLbFan;
+constexpr int64_t kStaticScanRuns = (kStaticScanGroups + kLbFan - 1) / kLbFan;
+constexpr int64_t kStaticScanWords =  // 256 KiB of tile words + 4 KiB of group words + 64 B of run words
+    2 * (kStaticScanTiles + kStaticScanGroups + kStaticScanRuns);
 static __device__ __align__(256) uint64_t scratch[kStaticScanWords];
 
 constexpr int kMaxDevices = 64;
@@ -308,7 +386,7 @@ extern "C" {
 int64_t shmt_scan_tmp_bytes(int64_t len) {
   if (len <= kSingleBlockMax) return 0;
   const int64_t tile_elems = kLbTileBytes / 8;  // tiles of the wider element type: an upper bound for both
-  return kScanHeaderBytes + ((len + tile_elems - 1) / tile_elems) * 16;
+  return scan_tmp_layout((len + tile_elems - 1) / tile_elems).total;
 }
 
 int shmt_exclusive_scan(void *data, int64_t len, int elem_bytes, void *tmp, int64_t tmp_bytes,
@@ -338,7 +416,7 @@ int shmt_exclusive_scan_noalloc(void *data, int64_t len, int elem_bytes, void *s
   if (rc) return rc;
   if (len == 0) return SHMT_OK;
   // The workspace keeps what the last call left in it; every call clears the
-  // tile counter and the tile words it is going to use before it scans.
+  // words it is going to use before it scans.
   const int64_t tmp_bytes = kStaticScanWords * static_cast<int64_t>(sizeof(uint64_t));
   if (elem_bytes == 8)
     return scan_inplace<uint64_t, false>(static_cast<uint64_t *>(data), len, partials, tmp_bytes,
