@@ -69,6 +69,31 @@ def test_single_pass_scan_tile_edges_and_unaligned_data(cabi, oracle, bytes_):
     assert lib.shmt_exclusive_scan(big.data_ptr(), 100_000, 8, small.data_ptr(), 8, cabi.current_stream()) == -4
 
 
+def test_single_pass_scan_all_three_levels_of_published_sums(cabi):
+    """A tile adds up the tiles before it in its group of 64, the groups before its group in its run of 64
+    groups, and the runs before its run. 3 x 2^26 int64 (12,289 tiles, 4 runs) against torch.cumsum; then
+    ones over 268,145 int32 tiles (35 GB, more than 64 runs: the runs are read in several steps), where the
+    exclusive scan is the position itself modulo 2^32."""
+    lib = cabi.load()
+    g = torch.Generator(device="cuda").manual_seed(9)
+    n = 3 * (1 << 26) + 5
+    a = torch.randint(0, 2**40, (n,), device="cuda", generator=g)
+    ref = torch.cumsum(a, 0) - a
+    tmp_bytes = lib.shmt_scan_tmp_bytes(n)
+    tmp = torch.empty(tmp_bytes, dtype=torch.uint8, device="cuda")
+    cabi.check(lib.shmt_exclusive_scan(a.data_ptr(), n, 8, tmp.data_ptr(), tmp_bytes, cabi.current_stream()))
+    assert torch.equal(a, ref)
+    del a, ref
+    n = (262_144 + 6_000) * 32_768 + 17
+    ones = torch.ones(n, dtype=torch.int32, device="cuda")
+    tmp_bytes = lib.shmt_scan_tmp_bytes(n)
+    tmp = torch.empty(tmp_bytes, dtype=torch.uint8, device="cuda")
+    cabi.check(lib.shmt_exclusive_scan(ones.data_ptr(), n, 4, tmp.data_ptr(), tmp_bytes, cabi.current_stream()))
+    probe = torch.cat([torch.randint(0, n, (1_000_000,), device="cuda", generator=g),
+                       torch.tensor([0, n - 1, 262_144 * 32_768 - 1, 262_144 * 32_768], device="cuda")])
+    assert torch.equal(ones[probe].long() & 0xFFFFFFFF, probe & 0xFFFFFFFF)
+
+
 def test_relabel_reference_kat(capi):
     g = load_golden("relabel_kat.json")
     u, labels = capi.tensor_relabel([torch.tensor(x).cuda() for x in g["inputs"]])
