@@ -8,13 +8,16 @@
 // scanned by one 1024-thread workgroup that walks the array with a running
 // carry (one launch). Larger inputs are scanned in ONE pass over the data
 // (read once, written once) by a grid no larger than the device holds at
-// once: workgroup b takes tiles b, b + grid, b + 2 grid, ..., scans each
-// locally, publishes the tile's sum, and obtains the sum of everything before
-// the tile from the sums that the tiles before it have published (per tile,
-// per group of 64 tiles, per run of 64 groups). A tile only ever waits for
-// tiles with smaller numbers; the smallest unfinished tile belongs to a
-// workgroup whose earlier tiles are all done, so it is being worked on and
-// waits for nothing unfinished: the waiting ends.
+// once: a workgroup takes tile numbers from a counter, one after the other,
+// scans each tile locally, publishes the tile's sum, and obtains the sum of
+// everything before the tile from the sums that the tiles before it have
+// published (per tile, per group of 64 tiles, per run of 64 groups). A tile
+// only ever waits for tiles with smaller numbers, and a number is only ever
+// held by a workgroup that is running (and that never waits for a larger
+// one), so the waiting ends whatever else shares the GPU. (Fixed tile
+// numbers b, b + grid, ... would not give that: two such kernels on two
+// streams could each hold compute units while waiting for workgroups of
+// their own that have not been started.)
 #include <mutex>
 
 #include "common.h"
@@ -66,12 +69,15 @@ int launch_scan_partials(uint64_t *partials, int64_t nb, hipStream_t s) {
 // Measured on MI355X, 16,777,216 int64 in place (268 MB of traffic): a
 // publish -> read step between workgroups takes tens of microseconds while the
 // memory queues are full of tile traffic, so the scan wants few, large tiles
-// and few levels: tiles of 16 / 32 / 64 / 128 KiB 216 / 90 / 57 / 52 us
+// and few levels (figures for fixed tile numbers): tiles of 16 / 32 / 64 / 128 KiB 216 / 90 / 57 / 52 us
 // (256 KiB: 111 us, the tile no longer fits the registers); groups of 16 or 8
 // instead of 64 (one level more for the same tiles) 67 / 112 us. Without
 // effect: requesting the workgroup's next tile before the look-back, one
-// 128-byte line per published entry, 256 instead of 512 workgroups. Walking
-// back over single tiles with a tile counter (the earlier form) took 64 us.
+// 128-byte line per published entry, 256 instead of 512 workgroups. Fixed
+// tile numbers (b, b + grid, ...) instead of the counter: 52 us, but not safe
+// beside other kernels (see the top of this file); with the counter 57 us.
+// Walking back over single tiles, one tile per workgroup (the earlier form),
+// took 64 us.
 constexpr uint32_t kPublished = 1;
 constexpr uint32_t kLookbackSpinLimit = 1u << 24;  // a wait that long means a tile before this one died
 constexpr int kLbBlock = 1024;                 // threads per tile
@@ -80,7 +86,10 @@ constexpr int kLbChunks = 8;                   // 16-byte vectors per lane
 constexpr int64_t kLbTileBytes = static_cast<int64_t>(kLbWaves) * kLbChunks * kWave * 16;
 constexpr int kLbFan = kWave;                  // tiles per group, groups per run
 
+constexpr int64_t kScanHeaderBytes = 64;  // tile counter (+ padding) in front of the published sums
+
 struct ScanState {
+  unsigned long long *counter;  // next tile number to hand out
   uint64_t *tiles;              // 2 words per tile
   uint64_t *groups;             // 2 words per group of 64 tiles
   uint64_t *runs;               // 2 words per run of 64 groups
@@ -95,7 +104,7 @@ static ScanTmpLayout scan_tmp_layout(int64_t nb) {
   l.nb = nb;
   l.ng = (nb + kLbFan - 1) / kLbFan;
   l.nr = (l.ng + kLbFan - 1) / kLbFan;
-  l.tiles_off = 0;
+  l.tiles_off = kScanHeaderBytes;
   l.groups_off = l.tiles_off + nb * 16;
   l.runs_off = l.groups_off + l.ng * 16;
   l.total = l.runs_off + l.nr * 16;
@@ -199,12 +208,20 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
   constexpr int64_t kTileElems = kLbTileBytes / sizeof(T);
   __shared__ uint64_t wave_total[kLbWaves];
   __shared__ uint64_t shared_before;  // the sum of everything before the tile
+  __shared__ uint64_t shared_tile;    // the workgroup's next tile number
   const int wave = threadIdx.x / kWave, lane = lane_id();
   const int64_t lane_off = static_cast<int64_t>(wave) * kLbChunks * kWave * V + lane * V;
   T v[kLbChunks][V];
-  int64_t tile = blockIdx.x;
+  if (threadIdx.x == 0) shared_tile = atomicAdd(st.counter, 1ull);
+  __syncthreads();
+  int64_t tile = static_cast<int64_t>(shared_tile);
   if (tile < nb) scan_tile_load<T, kLbChunks>(data, len, tile * kTileElems + lane_off, (tile + 1) * kTileElems <= len, v);
-  for (; tile < nb; tile += gridDim.x) {
+  while (tile < nb) {
+    // The next tile number is asked for now and only looked at after the look-back, which hides the round
+    // trip. One number per request: a workgroup that held two would publish the second tile's sum only
+    // after it had written the first tile out, and every later tile would wait for that (measured: 2.2 ms).
+    unsigned long long next_ticket = 0;
+    if (threadIdx.x == 0) next_ticket = atomicAdd(st.counter, 1ull);
     const int64_t lane_base = tile * kTileElems + lane_off;
     const bool whole = (tile + 1) * kTileElems <= len;
     T excl[kLbChunks];  // sum (mod 2^width) of the tile's elements in front of this lane's vector of chunk c
@@ -218,7 +235,6 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
       excl[c] = carry + inc - mine;
       carry += wave_last(inc);
     }
-    const int64_t next = tile + gridDim.x;
     if (lane == 0) wave_total[wave] = carry;
     __syncthreads();
     uint64_t in_tile = 0, total = 0;
@@ -245,10 +261,14 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
         if (threadIdx.x == 0) sum_publish(st.tiles, tile, total);
         before = tile_lookback(st, tile, total);
       }
-      if (threadIdx.x == 0) shared_before = before;
+      if (threadIdx.x == 0) {
+        shared_before = before;
+        shared_tile = next_ticket;
+      }
     }
     __syncthreads();
     const uint64_t base = shared_before + in_tile;
+    const int64_t next = static_cast<int64_t>(shared_tile);
 #pragma unroll
     for (int c = 0; c < kLbChunks; ++c) {
       const int64_t i = lane_base + static_cast<int64_t>(c) * kWave * V;
@@ -269,6 +289,7 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
       }
     }
     if (next < nb) scan_tile_load<T, kLbChunks>(data, len, next * kTileElems + lane_off, (next + 1) * kTileElems <= len, v);
+    tile = next;
   }  // the barriers above also order the reuse of the LDS words by the next tile
 }
 
@@ -326,10 +347,11 @@ static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, hipS
   SHMT_REQUIRE(nb < (1ll << 31), "scan: input too large");
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(tmp) & 7) == 0, "scan: tmp must be 8-byte aligned");
   ScanState st;
+  st.counter = static_cast<unsigned long long *>(tmp);
   st.tiles = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.tiles_off);
   st.groups = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.groups_off);
   st.runs = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.runs_off);
-  // the words start at zero (a kernel, not a memset, so that the scan can be captured in a graph)
+  // counter and words start at zero (a kernel, not a memset, so that the scan can be captured in a graph)
   hipLaunchKernelGGL(scan_state_clear_kernel, dim3(grid_for(need / 8, 256 * 4)), dim3(256), 0, s,
                      static_cast<uint64_t *>(tmp), need / 8);
   SHMT_LAUNCH_CHECK();
@@ -353,8 +375,8 @@ constexpr int64_t kStaticScanMaxLen = 1ll << 28;  // 268,435,456 elements
 constexpr int64_t kStaticScanTiles = kStaticScanMaxLen / (kLbTileBytes / 8);
 constexpr int64_t kStaticScanGroups = kStaticScanTiles / kLbFan;
 constexpr int64_t kStaticScanRuns = (kStaticScanGroups + kLbFan - 1) / kLbFan;
-constexpr int64_t kStaticScanWords =  // 256 KiB of tile words + 4 KiB of group words + 64 B of run words
-    2 * (kStaticScanTiles + kStaticScanGroups + kStaticScanRuns);
+constexpr int64_t kStaticScanWords =  // header + 256 KiB of tile words + 4 KiB of group words + 64 B of run words
+    kScanHeaderBytes / 8 + 2 * (kStaticScanTiles + kStaticScanGroups + kStaticScanRuns);
 static __device__ __align__(256) uint64_t scratch[kStaticScanWords];
 
 constexpr int kMaxDevices = 64;

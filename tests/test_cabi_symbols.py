@@ -34,7 +34,7 @@ def test_size_queries_and_validation(cabi):
     assert lib.shmt_hashmap_table_bytes(0, 0.5, 8, 8) == 128          # an empty map keeps one empty bucket
     assert lib.shmt_hashmap_table_bytes(10, 0.5, 3, 8) == -1
     assert b"bad arguments" in lib.shmt_last_error()
-    assert lib.shmt_scan_tmp_bytes(1000) == 0 and lib.shmt_scan_tmp_bytes(1 << 20) == (64 + 1 + 1) * 16
+    assert lib.shmt_scan_tmp_bytes(1000) == 0 and lib.shmt_scan_tmp_bytes(1 << 20) == 64 + (64 + 1 + 1) * 16
     assert lib.shmt_relabel_scratch_bytes(1000) >= 2000 * 16 + 4000
     assert lib.shmt_sample_plan_bytes(1024) >= 1024 * 16
     # relabel with 64-bit positions: 16-byte slots at load <= 0.5, 8-byte ranks; shmt_relabel uses it from 2^31 ids
