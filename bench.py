@@ -623,6 +623,7 @@ def bench_sampling(capi, args, result):
         # to drive the GPU path); the merged-launch form of the same batches is given beside it
         res["speedup_vs_cpu"] = round((edges / gpu_t) / best, 2)
         res["speedup_vs_cpu_reference_algorithms"] = round((edges / gpu_t) / (e_ref / t_ref), 2)
+        res["speedup_vs_cpu_chained_hops"] = round(overlapped["1_batches_in_flight"]["sampled_edges_per_s"] / best, 2)
         gpu_best = max(v["sampled_edges_per_s"] for v in overlapped.values())
         res["speedup_vs_cpu_batches_sharing_launches"] = round(gpu_best / best, 2)
     result["extra"]["sampling_config3"] = res
