@@ -26,9 +26,7 @@
 
 namespace shmt {
 
-constexpr int kScanBlock = 256;
-constexpr int kScanItems = 8;
-constexpr int kScanTile = kScanBlock * kScanItems;  // 2048 elements per workgroup
+constexpr int kScanItems = 8;  // elements per thread and step of the one-workgroup scan
 constexpr int64_t kSingleBlockMax = 1 << 16;
 
 // One workgroup scans the partials in place (exclusive).
