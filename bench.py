@@ -885,7 +885,11 @@ def main():
     if "sampling" in todo:
         bench_sampling(capi, args, result)
         s = result["extra"]["sampling_config3"]
+        # config 3 through the reference's operators, one batch at a time; and through sample_blocks with
+        # batches sharing their launches (what the dataloader's prefetch= uses)
         result["sampled_edges_per_s"] = s["sampled_edges_per_s"]
+        result["sampled_edges_per_s_batches_sharing_launches"] = max(
+            v["sampled_edges_per_s"] for v in s["sample_blocks_batches_in_flight"].values())
     if "e2e" in todo:
         torch.cuda.empty_cache()
         bench_e2e(capi, args, result)
