@@ -94,6 +94,29 @@ def test_single_pass_scan_all_three_levels_of_published_sums(cabi):
     assert torch.equal(ones[probe].long() & 0xFFFFFFFF, probe & 0xFFFFFFFF)
 
 
+def test_scans_on_several_streams_at_once(cabi):
+    """Scans queued on four streams without waiting in between share the GPU: every tile number is taken by
+    a running workgroup, so kernels that hold compute units at the same time cannot wait for each other's
+    unstarted workgroups. Each result against torch.cumsum."""
+    lib = cabi.load()
+    g = torch.Generator(device="cuda").manual_seed(4)
+    n = (1 << 24) + 3
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    data, refs, tmps = [], [], []
+    for _ in range(8):
+        a = torch.randint(0, 2**40, (n,), device="cuda", generator=g)
+        refs.append(torch.cumsum(a, 0) - a)
+        data.append(a)
+        tmps.append(torch.empty(lib.shmt_scan_tmp_bytes(n), dtype=torch.uint8, device="cuda"))
+    torch.cuda.synchronize()
+    for i, a in enumerate(data):
+        s = streams[i % 4]
+        cabi.check(lib.shmt_exclusive_scan(a.data_ptr(), n, 8, tmps[i].data_ptr(), tmps[i].numel(), s.cuda_stream))
+    torch.cuda.synchronize()
+    for a, ref in zip(data, refs):
+        assert torch.equal(a, ref)
+
+
 def test_relabel_reference_kat(capi):
     g = load_golden("relabel_kat.json")
     u, labels = capi.tensor_relabel([torch.tensor(x).cuda() for x in g["inputs"]])
