@@ -67,6 +67,39 @@ def test_fetch_query_and_set_replay_in_a_hip_graph(capi, cache):
         assert float(static_out.abs().sum()) > 0
 
 
+def test_one_pass_scans_replay_in_a_hip_graph(capi, cabi):
+    """thrust_scan (workspace from the shim), shmt_exclusive_scan with a caller's workspace and the form
+    without a workspace, each over several tiles, recorded once and replayed on new data: the kernels clear
+    the published sums they use with a kernel of their own, so every replay starts clean."""
+    lib = cabi.load()
+    n = 3_000_017
+    static_a = torch.zeros(n, dtype=torch.int32).cuda()
+    static_b = torch.zeros(n, dtype=torch.int64).cuda()
+    static_c = torch.zeros(n, dtype=torch.int64).cuda()
+    tmp = torch.empty(lib.shmt_scan_tmp_bytes(n), dtype=torch.uint8).cuda()
+    cabi.check(lib.shmt_exclusive_scan_noalloc(None, 0, 8, cabi.current_stream()))     # set-up call outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        capi.thrust_scan(static_a)
+        cabi.check(lib.shmt_exclusive_scan(static_b.data_ptr(), n, 8, tmp.data_ptr(), tmp.numel(), cabi.current_stream()))
+        cabi.check(lib.shmt_exclusive_scan_noalloc(static_c.data_ptr(), n, 8, cabi.current_stream()))
+    g = torch.Generator(device="cuda").manual_seed(3)
+    for it in range(4):
+        a = torch.randint(-1000, 1000, (n,), device="cuda", generator=g, dtype=torch.int32)
+        b = torch.randint(0, 2**40, (n,), device="cuda", generator=g)
+        static_a.copy_(a)
+        static_b.copy_(b)
+        static_c.copy_(b)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_a, torch.cumsum(a, 0, dtype=torch.int32)), it
+        assert torch.equal(static_b, torch.cumsum(b, 0) - b), it
+        assert torch.equal(static_c, static_b), it
+        torch.zeros(1000, device="cuda").sum()       # eager work between the replays
+
+
 def test_fused_hop_replays_in_a_hip_graph(capi, cabi):
     """shmt_sample_hop never waits for the host (sizes go to device memory here), so the whole hop can be
     captured once and replayed on new seeds: every replay is compared with the eager operator, with eager
