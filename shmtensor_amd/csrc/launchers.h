@@ -21,12 +21,12 @@ constexpr int kMaxStages = 12;
 enum StageKind : int {
   kStagePlanSingle = 0,  // + map mode (0: no cache, 1: wide map, 2: narrow map)
   kStagePlanTile = 3,    // + map mode
-  kStagePickNarrowHop = 6,
-  kStageRlSmall = 7,
-  kStageRlInsert = 8,
-  kStageRlFirst = 9,
-  kStageRlUnique = 10,
-  kStageRlLabels = 11,
+  kStagePickNarrowHop = 6,  // + log2(lanes per seed) - 2, i.e. 6 .. 10
+  kStageRlSmall = 11,
+  kStageRlInsert = 12,
+  kStageRlFirst = 13,
+  kStageRlUnique = 14,
+  kStageRlLabels = 15,
 };
 
 struct Stage {

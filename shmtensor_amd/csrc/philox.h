@@ -68,4 +68,16 @@ SHMT_HD uint64_t sample_draw(uint64_t rng_seed, uint32_t rng_stream, int64_t nod
   return mulhi64(bits, range);
 }
 
+// The same draw for a range that fits 32 bits: floor(bits * range / 2^64) from
+// two 32-bit products instead of a 64 x 64-bit one (identical value).
+SHMT_HD uint32_t sample_draw32(uint64_t rng_seed, uint32_t rng_stream, int64_t node, uint32_t draw,
+                               uint32_t range) {
+  const uint64_t n = static_cast<uint64_t>(node);
+  Philox4 r = philox4x32_10(static_cast<uint32_t>(n), static_cast<uint32_t>(n >> 32), draw,
+                            rng_stream, static_cast<uint32_t>(rng_seed),
+                            static_cast<uint32_t>(rng_seed >> 32));
+  const uint64_t low = (static_cast<uint64_t>(r.v[0]) * range) >> 32;
+  return static_cast<uint32_t>((static_cast<uint64_t>(r.v[1]) * range + low) >> 32);
+}
+
 }  // namespace shmt

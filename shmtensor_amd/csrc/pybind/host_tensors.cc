@@ -21,19 +21,30 @@
 
 namespace py = pybind11;
 
+namespace shim {
+bool host_register_enabled();  // module.cc: the opt-in switch for registering existing memory in place
+}
+
 namespace {
 
-// Registers a fresh mapping for GPU access. Some drivers refuse to register
-// memory that already exists; the mapping is then taken down again (and the
-// segment this call created removed) before the error is raised, so a refused
-// request leaves nothing behind.
+// Registers a fresh mapping for GPU access, where that is switched on.
+// Registering memory that already exists is refused by some drivers, and a
+// refused call can leave its error for the next HIP call to report, so the
+// runtime is only asked when in-place registration was requested
+// (set_host_register(True) / SHMT_HOST_REGISTER=1, the switch pin_memory()
+// honours too). Without the request, or when the driver refuses, the mapping is
+// taken down again (and the segment this call created removed) before the
+// error is raised, so a refused request leaves nothing behind.
 void pin_range(void *ptr, int64_t size, int fd, const char *what, const char *unlink_name) {
-  if (shmt_host_register(ptr, size) == SHMT_OK) return;
-  const std::string why = shmt_last_error();
+  const bool asked = shim::host_register_enabled();
+  if (asked && shmt_host_register(ptr, size) == SHMT_OK) return;
+  const std::string why = asked ? std::string("the driver refused: ") + shmt_last_error()
+                                : std::string("in-place registration is switched off; set_host_register(True) or "
+                                              "SHMT_HOST_REGISTER=1 asks the driver for it");
   munmap(ptr, static_cast<size_t>(size));
   close(fd);
   if (unlink_name != nullptr) shm_unlink(unlink_name);
-  TORCH_CHECK(false, what, "(pin_memory=True): this driver does not register an existing mapping for GPU access (",
+  TORCH_CHECK(false, what, "(pin_memory=True): the existing mapping was not registered for GPU access (",
               why, "). Open it with pin_memory=False and hand the GPU operators a staging copy in pinned "
               "memory instead: `staged = obj.pinned()` on a ShmTensor / DiskTensor (`obj.flush()` copies it "
               "back into the mapping), or `tensor.pin_memory()` on the plain tensor.");

@@ -228,6 +228,7 @@ struct PickArgs {
   int ptr_bytes;
   int replace;
   int log2_group;  // lanes per seed (narrow kernel)
+  int rounds;      // seeds a lane group handles per pass (narrow kernel), 1 .. kPickRounds
   // fused hop only (HOP kernels):
   void *sub_indptr_rw;          // tile-local offsets in, final offsets out
   const uint64_t *tile_prefix;  // totals of the plan's seed tiles, or null when offsets are final: scanned
@@ -315,67 +316,186 @@ __device__ __forceinline__ int64_t load_adj(const PickArgs &a, int64_t begin_tag
   return load_int(base, (begin_tagged & ~kCachedTag) + pos, a.idx_bytes);
 }
 
-// k <= 64: group of G = 2^log2_group >= k lanes per seed. (bx, gx): this
-// workgroup's index and the number of workgroups of its job.
-template <bool HOP>
+// Floyd's subset selection resolved inside a group of G lanes, positions of 32
+// bits. Lane j (j < k) brings its draw t_j in [0, top_j], top_j = deg - k + j;
+// the chosen position of step j is t_j unless an earlier step already chose
+// that value, and top_j then (which no earlier step can have chosen). Steps
+// run in order: at step s the choice of lane s is final (it has seen the
+// choices of all steps before it) and is handed to the lanes behind it, which
+// note whether it equals their own draw. Lanes at or beyond k take no part in
+// the result. Groups of 16 lanes and more hand the choice on through scalar
+// registers (one readlane per group of the wave) and keep the "already chosen"
+// flags as one 64-bit lane mask, which costs five vector and eight scalar
+// instructions per step for two groups of 32; smaller groups (at most seven
+// steps) use a lane permute.
+template <int G>
+__device__ __forceinline__ uint32_t floyd_resolve32(uint32_t t, uint32_t top, int gl, int k) {
+  if (G == 32) {
+    uint64_t hit = 0;
+    for (int step = 0; step + 1 < k; ++step) {
+      const uint32_t c = __builtin_amdgcn_inverse_ballot_w64(hit) ? top : t;
+      const uint32_t c0 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c), step));
+      const uint32_t c1 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c), 32 + step));
+      const uint64_t m0 = __builtin_amdgcn_ballot_w64(t == c0), m1 = __builtin_amdgcn_ballot_w64(t == c1);
+      const uint32_t behind = 0xFFFFFFFEu << step;  // lanes of a group with gl > step
+      hit |= (static_cast<uint64_t>(static_cast<uint32_t>(m1 >> 32) & behind) << 32) |
+             (static_cast<uint32_t>(m0) & behind);
+    }
+    return __builtin_amdgcn_inverse_ballot_w64(hit) ? top : t;
+  }
+  if (G >= 16) {
+    constexpr int kGroups = kWave / G;
+    // bit l of `behind`: lane l lies behind the current step in its group (gl > step)
+    constexpr uint64_t kLowBits = G == 64 ? 1ull : G == 32 ? 0x0000000100000001ull : 0x0001000100010001ull;
+    constexpr uint64_t kGroupLanes = G == 64 ? ~0ull : (1ull << (G % 64)) - 1ull;
+    uint64_t behind = ~kLowBits;
+    uint64_t hit = 0;
+    for (int step = 0; step + 1 < k; ++step) {
+      const uint32_t c = __builtin_amdgcn_inverse_ballot_w64(hit) ? top : t;
+      uint64_t same = 0;  // lanes whose draw equals the choice their group just made
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g) {
+        const uint32_t chosen = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(c), g * G + step));
+        same |= __builtin_amdgcn_ballot_w64(t == chosen) & (kGroupLanes << (g * G));
+      }
+      hit |= same & behind;
+      behind = (behind << 1) & ~kLowBits;
+    }
+    return __builtin_amdgcn_inverse_ballot_w64(hit) ? top : t;
+  }
+  bool hit = false;
+  for (int step = 0; step + 1 < k; ++step) {
+    const uint32_t c = hit ? top : t;
+    const uint32_t chosen = static_cast<uint32_t>(__shfl(static_cast<int>(c), (lane_id() & ~(G - 1)) + step, kWave));
+    hit |= (gl > step) && (chosen == t);
+  }
+  return hit ? top : t;
+}
+
+// One adjacency element, issued without touching the loaded value: 4-byte
+// elements come back zero-extended and are sign-extended by adj_value() when
+// they are stored, so that several such loads stay in flight together.
+__device__ __forceinline__ int64_t issue_adj(const PickArgs &a, int64_t begin_tagged, int64_t pos) {
+  const void *base = (begin_tagged & kCachedTag) ? a.cache_indices : a.indices;
+  const int64_t i = (begin_tagged & ~kCachedTag) + pos;
+  if (a.idx_bytes == 8) return static_cast<const int64_t *>(base)[i];
+  return static_cast<int64_t>(static_cast<const uint32_t *>(base)[i]);
+}
+__device__ __forceinline__ int64_t adj_value(const PickArgs &a, int64_t raw) {
+  return a.idx_bytes == 8 ? raw : static_cast<int64_t>(static_cast<int32_t>(static_cast<uint32_t>(raw)));
+}
+
+constexpr int kPickRounds = 4;  // seeds a lane group handles per pass, at most: that many adjacency loads in flight
+
+// k <= 64: group of G = 2^LG >= k lanes per seed. (bx, gx): this workgroup's
+// index and the number of workgroups of its job. A wave takes `rounds` x 64 / G
+// consecutive seeds per pass (a.rounds <= kPickRounds; they share a plan
+// tile): first one lane per seed fetches the seed's plan entry, output offset
+// and id in coalesced loads (and finishes the offset: the fused hop's plan
+// leaves tile-local offsets), then the lane groups take the seeds round by
+// round, choose their positions and issue the adjacency loads of all rounds
+// before the first value is stored. The chain of dependent memory round trips
+// per pass is plan entry -> adjacency -> store whatever the number of rounds;
+// measured on 127,000 seeds with 25 picks each: 98 us with one seed per group
+// and pass (four dependent chains per wave one after the other), 79 us so.
+// Capping the kernel at 64 registers for eight resident waves per SIMD spills
+// and measured 150 us; two rounds per pass instead of four measured the same.
+template <bool HOP, int LG>
 __device__ __forceinline__ void pick_narrow_body(unsigned bx, unsigned gx, const PickArgs &a) {
   pick_clear<HOP>(a, bx, gx);
+  constexpr int G = 1 << LG;
+  constexpr int kGroups = kWave / G;
   const int lane = lane_id();
-  const int G = 1 << a.log2_group;
   const int gl = lane & (G - 1);
-  const int gbase = lane & ~(G - 1);
-  const int groups_per_wave = kWave >> a.log2_group;
+  const int grp = lane >> LG;
   const int64_t waves_per_block = blockDim.x / kWave;
   const int64_t wave = static_cast<int64_t>(bx) * waves_per_block + threadIdx.x / kWave;
   const int64_t nwaves = static_cast<int64_t>(gx) * waves_per_block;
   const int k = static_cast<int>(a.k);
+  const int rounds = a.rounds;
+  const int per_pass = rounds * kGroups;  // <= 64 and a divisor of kPlanBlock
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
   const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
   if (HOP) pick_publish_total(a, S, bx);
 
-  for (int64_t s0 = wave * groups_per_wave; s0 < S; s0 += nwaves * groups_per_wave) {
-    // the seeds of a wave share a plan tile (tiles hold a multiple of groups_per_wave seeds)
-    const int64_t tile_base = HOP ? pick_tile_base(a, s0) : 0;
-    const int64_t s = s0 + (lane >> a.log2_group);
-    if (s >= S) continue;  // uniform within the group
-    const SeedPlan p = a.plan[s];
-    const int64_t deg = p.deg;
-    const int64_t optr = pick_offset<HOP>(a, s, tile_base, gl == 0);
-    if (deg <= 0) continue;
-    if (a.replace) {
-      if (gl < k) {
-        const int64_t node = load_int(a.seeds, s, a.seed_bytes);
-        const uint64_t r = sample_draw(rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg));
-        pick_store<HOP>(a, S, s, optr + gl, load_adj(a, p.begin, static_cast<int64_t>(r)));
+  for (int64_t w0 = wave * per_pass; w0 < S; w0 += nwaves * per_pass) {
+    const int64_t tile_base = HOP ? pick_tile_base(a, w0) : 0;
+    // one lane per seed of the pass
+    const int64_t sl = w0 + lane;
+    const bool seed_live = lane < per_pass && sl < S;
+    SeedPlan pl{0, 0};
+    int64_t optr_l = 0, node_l = 0;
+    if (seed_live) {
+      pl = a.plan[sl];
+      node_l = load_int(a.seeds, sl, a.seed_bytes);
+      if (!HOP) {
+        optr_l = load_int(a.sub_indptr, sl, a.ptr_bytes);
+      } else {
+        optr_l = load_int(a.sub_indptr_rw, sl, a.ptr_bytes);
+        note_wide_id(a, node_l);
+        if (a.tile_prefix) {
+          optr_l += tile_base;
+          store_int(a.sub_indptr_rw, sl, a.ptr_bytes, optr_l);
+        }
       }
-    } else if (deg <= k) {
-      if (gl < deg) pick_store<HOP>(a, S, s, optr + gl, load_adj(a, p.begin, gl));
-    } else {
-      // Floyd: for J = deg-k .. deg-1 draw t in [0, J]; take t unless already
-      // taken, then take J. Draws in parallel, resolution in k ballot steps.
-      const int64_t node = load_int(a.seeds, s, a.seed_bytes);
-      int64_t t = 0;
-      if (gl < k)
-        t = static_cast<int64_t>(sample_draw(rng_seed, a.rng_stream, node, gl,
-                                             static_cast<uint64_t>(deg - k + gl + 1)));
-      int64_t mine = -1;
-      for (int step = 0; step < k; ++step) {
-        const int64_t ts = shfl64(t, gbase + step);
-        const bool taken = group_ballot_dyn(gl < step && mine == ts, G) != 0;
-        if (gl == step) mine = taken ? (deg - k + step) : ts;
-      }
-      if (gl < k) pick_store<HOP>(a, S, s, optr + gl, load_adj(a, p.begin, mine));
     }
+    int64_t raw[kPickRounds], where[kPickRounds];
+#pragma unroll
+    for (int r = 0; r < kPickRounds; ++r) {
+      where[r] = -1;  // nothing to store for this lane in round r
+      if (r >= rounds) continue;
+      const int src = r * kGroups + grp;
+      const int64_t begin = shfl64(pl.begin, src);
+      const int64_t deg = shfl64(pl.deg, src);
+      const int64_t optr = shfl64(optr_l, src);
+      const int64_t node = shfl64(node_l, src);
+      if (w0 + src >= S || deg <= 0) continue;  // uniform within the group
+      int64_t pos = -1;  // position in the row this lane reads
+      if (a.replace) {
+        if (gl < k) pos = static_cast<int64_t>(sample_draw(rng_seed, a.rng_stream, node, gl, static_cast<uint64_t>(deg)));
+      } else if (deg <= k) {
+        if (gl < deg) pos = gl;
+      } else if (deg <= static_cast<int64_t>(0xFFFFFFFFu)) {
+        // Floyd with 32-bit positions (every degree met in practice)
+        const uint32_t top = static_cast<uint32_t>(deg - k + gl);  // J of this lane's step
+        uint32_t t = 0;
+        if (gl < k) t = sample_draw32(rng_seed, a.rng_stream, node, gl, top + 1u);
+        const uint32_t mine = floyd_resolve32<G>(t, top, gl, k);
+        if (gl < k) pos = mine;
+      } else {
+        // Floyd: for J = deg-k .. deg-1 draw t in [0, J]; take t unless already
+        // taken, then take J. Draws in parallel, resolution in k ballot steps.
+        int64_t t = 0;
+        if (gl < k)
+          t = static_cast<int64_t>(sample_draw(rng_seed, a.rng_stream, node, gl,
+                                               static_cast<uint64_t>(deg - k + gl + 1)));
+        int64_t mine = -1;
+        for (int step = 0; step < k; ++step) {
+          const int64_t ts = shfl64(t, (lane & ~(G - 1)) + step);
+          const bool taken = group_ballot<G>(gl < step && mine == ts) != 0;
+          if (gl == step) mine = taken ? (deg - k + step) : ts;
+        }
+        if (gl < k) pos = mine;
+      }
+      if (pos >= 0) {
+        raw[r] = issue_adj(a, begin, pos);
+        where[r] = optr + gl;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kPickRounds; ++r)
+      if (where[r] >= 0) pick_store<HOP>(a, S, w0 + r * kGroups + grp, where[r], adj_value(a, raw[r]));
   }
 }
 
-template <bool HOP>
+template <bool HOP, int LG>
 __global__ __launch_bounds__(256) void pick_narrow_kernel(PickArgs a) {
-  pick_narrow_body<HOP>(blockIdx.x, gridDim.x, a);
+  pick_narrow_body<HOP, LG>(blockIdx.x, gridDim.x, a);
 }
 
+template <int LG>
 __global__ __launch_bounds__(256) void pick_narrow_hop_jobs(Jobs<PickArgs> j) {
-  if (blockIdx.x < j.blocks[blockIdx.y]) pick_narrow_body<true>(blockIdx.x, j.blocks[blockIdx.y], j.a[blockIdx.y]);
+  if (blockIdx.x < j.blocks[blockIdx.y]) pick_narrow_body<true, LG>(blockIdx.x, j.blocks[blockIdx.y], j.a[blockIdx.y]);
 }
 
 // k > 64: one wave (= one 64-thread workgroup) per seed. The chosen positions
@@ -680,14 +800,31 @@ struct PickHopExtras {
 };
 
 template <bool HOP>
-static int pick_launch(const PickArgs &a, Launcher launcher) {
+static void launch_pick_narrow(int lg, unsigned blocks, unsigned threads, hipStream_t s, const PickArgs &a) {
+  switch (lg) {
+    case 2: hipLaunchKernelGGL((pick_narrow_kernel<HOP, 2>), dim3(blocks), dim3(threads), 0, s, a); break;
+    case 3: hipLaunchKernelGGL((pick_narrow_kernel<HOP, 3>), dim3(blocks), dim3(threads), 0, s, a); break;
+    case 4: hipLaunchKernelGGL((pick_narrow_kernel<HOP, 4>), dim3(blocks), dim3(threads), 0, s, a); break;
+    case 5: hipLaunchKernelGGL((pick_narrow_kernel<HOP, 5>), dim3(blocks), dim3(threads), 0, s, a); break;
+    default: hipLaunchKernelGGL((pick_narrow_kernel<HOP, 6>), dim3(blocks), dim3(threads), 0, s, a); break;
+  }
+}
+
+template <bool HOP>
+static int pick_launch(PickArgs a, Launcher launcher) {
   hipStream_t s = launcher.stream;
   StageList *const defer = launcher.defer;
   const int64_t S = a.S, k = a.k;
   if (k <= kWave) {
+    // One seed per lane group and pass while all waves of the launch are resident together (8,192 on
+    // this part); beyond that a group takes 2 or 4 seeds per pass, whose adjacency loads overlap.
+    const int groups_per_wave = kWave >> a.log2_group;
+    int rounds = 1;
+    while (rounds < kPickRounds && (S + groups_per_wave * rounds - 1) / (groups_per_wave * rounds) > 8192) rounds *= 2;
+    a.rounds = rounds;
+    const int seeds_per_wave = groups_per_wave * rounds;
     // Few seeds: one wave per workgroup, so that the cold rows' host-link reads come from as many
     // compute units as possible (a unit keeps only so many of them in flight).
-    const int seeds_per_wave = kWave >> a.log2_group;
     int threads = 256;
     int64_t blocks = (S + 4 * seeds_per_wave - 1) / (4 * seeds_per_wave);
     if (blocks < 512) {
@@ -700,10 +837,13 @@ static int pick_launch(const PickArgs &a, Launcher launcher) {
       if (blocks < for_clear) blocks = for_clear;
     }
     if (defer) {
-      if (HOP) stage_push(defer, kStagePickNarrowHop, grid_for(blocks, 1), threads, a); else defer->mergeable = false;
+      if (HOP)
+        stage_push(defer, kStagePickNarrowHop + a.log2_group - 2, grid_for(blocks, 1), threads, a);
+      else
+        defer->mergeable = false;
       return SHMT_OK;
     }
-    hipLaunchKernelGGL(pick_narrow_kernel<HOP>, dim3(grid_for(blocks, 1)), dim3(threads), 0, s, a);
+    launch_pick_narrow<HOP>(a.log2_group, grid_for(blocks, 1), threads, s, a);
   } else if (defer) {
     defer->mergeable = false;  // the one-wave-per-seed forms have no merged launch
     return SHMT_OK;
@@ -723,10 +863,17 @@ namespace shmt {
 int launch_merged_sampling_stage(int n_jobs, const Stage *const *stages, hipStream_t s) {
   const int kind = stages[0]->kind;
   const unsigned threads = stages[0]->threads;
-  if (kind == kStagePickNarrowHop) {
+  if (kind >= kStagePickNarrowHop && kind < kStagePickNarrowHop + 5) {
     Jobs<PickArgs> j;
     const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
-    hipLaunchKernelGGL(pick_narrow_hop_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
+    const dim3 grid(blocks, n_jobs), block(threads);
+    switch (kind - kStagePickNarrowHop + 2) {
+      case 2: hipLaunchKernelGGL(pick_narrow_hop_jobs<2>, grid, block, 0, s, j); break;
+      case 3: hipLaunchKernelGGL(pick_narrow_hop_jobs<3>, grid, block, 0, s, j); break;
+      case 4: hipLaunchKernelGGL(pick_narrow_hop_jobs<4>, grid, block, 0, s, j); break;
+      case 5: hipLaunchKernelGGL(pick_narrow_hop_jobs<5>, grid, block, 0, s, j); break;
+      default: hipLaunchKernelGGL(pick_narrow_hop_jobs<6>, grid, block, 0, s, j); break;
+    }
   } else if (kind >= kStagePlanSingle && kind < kStagePlanTile + 3) {
     Jobs<PlanArgs> j;
     const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
@@ -777,6 +924,7 @@ static int pick_impl(const void *indices, const void *cache_indices, int idx_byt
   a.ptr_bytes = ptr_bytes;
   a.replace = replace ? 1 : 0;
   a.log2_group = 0;
+  a.rounds = 1;
   if (k <= kWave) {
     int lg = 2;
     while ((1 << lg) < k) ++lg;

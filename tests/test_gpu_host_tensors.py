@@ -99,29 +99,41 @@ def test_shm_tensor_rows_through_the_gpu_operators(capi, shmtensor):
 
 def test_pin_memory_true_works_or_names_the_alternative(capi, shmtensor, tmp_path):
     """In-place registration is the reference's route (include/shm_memory.h:19-21,
-    src/mmap_tensor.cc:42-45). Where the driver provides it the mapping itself is fetched
-    from; where it is refused the error names the staging copy and nothing is left behind."""
+    src/mmap_tensor.cc:42-45). It is asked of the driver only on request (SHMT_HOST_REGISTER=1 /
+    set_host_register(True)): without the request pin_memory=True raises the error that names the
+    staging copy, makes no runtime call and leaves nothing behind; with it, the mapping itself is
+    fetched from where the driver provides registration, and the same error is raised where not."""
+    asked = os.environ.get("SHMT_HOST_REGISTER", "0") not in ("", "0")
     data = np.arange(600, dtype=np.float32).reshape(100, 6)
     path = str(tmp_path / "p.npy")
     np.save(path, data)
     idx = torch.tensor([0, 99, 5]).cuda()
-    try:
-        t = shmtensor.DiskTensor(path, pin_memory=True)
-    except RuntimeError as exc:
-        assert "pinned()" in str(exc) and "pin_memory=False" in str(exc)
-    else:
-        assert np.array_equal(capi.uva_fetch(t.tensor_, idx).cpu().numpy(), data[[0, 99, 5]])
-        del t
     name = "shmt_pin_%s" % uuid.uuid4().hex[:12]
-    try:
-        s = shmtensor.ShmTensor(name, (100, 6), 0, 1, None, torch.float32, pin_memory=True)
-    except RuntimeError as exc:
-        assert "pinned()" in str(exc)
+    if not asked:
+        with pytest.raises(RuntimeError, match="switched off") as exc:
+            shmtensor.DiskTensor(path, pin_memory=True)
+        assert "pinned()" in str(exc.value) and "pin_memory=False" in str(exc.value)
+        with pytest.raises(RuntimeError, match="switched off") as exc:
+            shmtensor.ShmTensor(name, (100, 6), 0, 1, None, torch.float32, pin_memory=True)
+        assert "pinned()" in str(exc.value)
         assert not capi.file_exist(name)                                 # the refused segment was removed
     else:
-        s.tensor_.copy_(torch.from_numpy(data))
-        assert np.array_equal(capi.uva_fetch(s.tensor_, idx).cpu().numpy(), data[[0, 99, 5]])
-        del s
+        try:
+            t = shmtensor.DiskTensor(path, pin_memory=True)
+        except RuntimeError as exc:
+            assert "pinned()" in str(exc) and "pin_memory=False" in str(exc)
+        else:
+            assert np.array_equal(capi.uva_fetch(t.tensor_, idx).cpu().numpy(), data[[0, 99, 5]])
+            del t
+        try:
+            s = shmtensor.ShmTensor(name, (100, 6), 0, 1, None, torch.float32, pin_memory=True)
+        except RuntimeError as exc:
+            assert "pinned()" in str(exc)
+            assert not capi.file_exist(name)
+        else:
+            s.tensor_.copy_(torch.from_numpy(data))
+            assert np.array_equal(capi.uva_fetch(s.tensor_, idx).cpu().numpy(), data[[0, 99, 5]])
+            del s
     # an unpinned mapping handed to a kernel is an error, not a fault
     t = shmtensor.DiskTensor(path)
     with pytest.raises(RuntimeError, match="pin_memory"):

@@ -109,3 +109,21 @@ def test_shm_tensor_two_ranks_gloo():
         p.join(120)
         assert p.exitcode == 0
     assert dict(results) == {0: 24000, 1: 24000}
+
+
+def test_pin_memory_true_needs_the_opt_in(shmtensor, capi, tmp_path):
+    """Registering an existing mapping in place is only asked of the driver on request
+    (set_host_register(True) / SHMT_HOST_REGISTER=1). Without it pin_memory=True raises an error
+    that names the staging copy, before any runtime call (so this runs without a GPU), and takes
+    the mapping and the segment it created down again."""
+    capi.set_host_register(False)
+    f = str(tmp_path / "p.npy")
+    np.save(f, np.arange(12, dtype=np.float32))
+    with pytest.raises(RuntimeError, match="switched off") as exc:
+        shmtensor.DiskTensor(f, pin_memory=True)
+    assert "pinned()" in str(exc.value) and "set_host_register" in str(exc.value)
+    name = "shmt_cpu_pin_%s" % uuid.uuid4().hex[:12]
+    with pytest.raises(RuntimeError, match="switched off"):
+        shmtensor.ShmTensor(name, (4, 3), 0, 1, None, torch.float32, pin_memory=True)
+    assert not capi.file_exist(name)
+    assert shmtensor.DiskTensor(f).tensor_.tolist() == list(range(12))      # the file is still fine
