@@ -842,7 +842,7 @@ def main():
     ap.add_argument("--sampling-scale", type=int, default=21)
     ap.add_argument("--sampling-batches", type=int, default=50)
     ap.add_argument("--e2e-scale", type=int, default=24)
-    ap.add_argument("--e2e-batches", type=int, default=8)
+    ap.add_argument("--e2e-batches", type=int, default=24)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--headline-only", action="store_true",

@@ -178,6 +178,37 @@ int shmt_fetch_counted(const void *miss_data, const void *cache_data,
                        const int64_t *count, int64_t *count_seen,
                        int64_t row_bytes, void *stream);
 
+/* A cached fetch in two launches, for callers that overlap fetches with
+ * other GPU work (the next mini-batch's sampling). CacheTensorFetch
+ * (src/cache_feature_fetch.cu:131-185) moves hits and misses in one kernel;
+ * when the id-addressed table lives in pinned host memory the misses are
+ * host-link reads, and a kernel that spans the whole GPU while it waits for
+ * them keeps every other stream's kernels out and fills the link's queue.
+ *   shmt_fetch_cached_part  moves the rows that hit (out[i,:] =
+ *       cache_data[slot_i,:]) over the first min(max_rows, *count) entries
+ *       (count may be NULL: exactly max_rows) and marks the rows that missed
+ *       in miss_bits: bit (i & 31) of 32-bit word i / 32, room for
+ *       ceil(max_rows / 32) words. Every word that covers an existing row is
+ *       written, so the buffer needs no clearing.
+ *   shmt_fetch_missed_part  moves out[i,:] = miss_data[indices[i],:] for the
+ *       marked rows (same max_rows and count), on at most max_blocks
+ *       workgroups (0: a default that saturates the host link and no more),
+ *       and may run on another stream once the first call's work is done.
+ * Together they give exactly what shmt_fetch[_counted] gives. Rows and
+ * tables must allow 16-byte accesses (row_bytes and all base addresses
+ * multiples of 16) and max_rows must be below 2^32; otherwise SHMT_EINVAL,
+ * and the caller uses shmt_fetch.                                          */
+int shmt_fetch_cached_part(const void *miss_data, const void *cache_data,
+                           const void *indices, int idx_bytes,
+                           const shmt_hashmap_t *map, const void *mask,
+                           int mask_bytes, void *out, int64_t max_rows,
+                           const int64_t *count, int64_t row_bytes,
+                           uint32_t *miss_bits, void *stream);
+int shmt_fetch_missed_part(const void *miss_data, const void *indices,
+                           int idx_bytes, const uint32_t *miss_bits, void *out,
+                           int64_t max_rows, const int64_t *count,
+                           int64_t row_bytes, int max_blocks, void *stream);
+
 /* Feature set: UVATensorSet src/cache_feature_set.cu:39-75, CacheTensorSet
  * :118-165, CacheTensorSetWithMask :209-248. Mirror of shmt_fetch:
  *   (slot_i >= 0 ? cache_data[slot_i,:] : miss_data[indices[i],:]) = update[i,:]

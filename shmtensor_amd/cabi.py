@@ -33,6 +33,8 @@ SIGNATURES = {
     "shmt_hashmap_destroy": (None, [_vp]),
     "shmt_fetch": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
     "shmt_fetch_counted": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _vp, _vp, _i64, _vp]),
+    "shmt_fetch_cached_part": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _vp, _i64, _vp, _vp]),
+    "shmt_fetch_missed_part": (_int, [_vp, _vp, _int, _vp, _vp, _i64, _vp, _i64, _int, _vp]),
     "shmt_set": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
     "shmt_set_through": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _vp, _i64, _i64, _vp]),
     "shmt_scan_tmp_bytes": (_i64, [_i64]),

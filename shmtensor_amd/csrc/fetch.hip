@@ -46,6 +46,7 @@ struct RowArgs {
   int mask_bytes;
   int log2_lanes;      // lanes per row in phase 2 = 1 << log2_lanes, in [8, 64]
   int log2_tile;       // rows per wave tile = 1 << log2_tile, in [64 / lanes, 32]
+  uint32_t *miss_bits;  // DEFER: bit (i & 31) of word i / 32 is set when row i missed the cache
 };
 
 // Native vector types (the non-temporal builtins do not take HIP's struct vectors).
@@ -77,9 +78,13 @@ constexpr int kMaxLog2Tile = 5;
 
 // THROUGH (set only, with a map or mask): rows that hit the cache are written
 // to the id-addressed table as well, so that table never goes stale.
-template <typename VT, int MODE, bool SET, bool ONE_VEC, bool THROUGH = false>
+// DEFER (fetch only, with a map or mask; tiles of exactly 32 rows): rows that
+// miss the cache are not moved; every tile leaves one word of a bitmap that
+// marks them for rows_missed_kernel (no counter, no atomics, nothing to clear).
+template <typename VT, int MODE, bool SET, bool ONE_VEC, bool THROUGH = false, bool DEFER = false>
 __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWavesPerSimd / 2) void rows_kernel(RowArgs a) {
   static_assert(!THROUGH || (SET && MODE != kDirect), "write-through is a cached set");
+  static_assert(!DEFER || (!SET && MODE != kDirect), "only a cached fetch sets its misses aside");
   const int lane = lane_id();
   const int L = 1 << a.log2_lanes;
   const int gl = lane & (L - 1);
@@ -117,8 +122,12 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
       // direct or range form of the map: one 4-byte load, or arithmetic only
       if (live) slot = flat_find(a.map, map_key(a.map, idx));
     }
+    if (DEFER) {
+      const uint64_t missed = __builtin_amdgcn_ballot_w64(live && slot < 0);
+      if (lane == 0) a.miss_bits[base >> 5] = static_cast<uint32_t>(missed);
+    }
     const int64_t my_table_row =
-        reinterpret_cast<int64_t>(slot >= 0 ? a.cache + slot * R : a.miss + idx * R);
+        DEFER && slot < 0 ? 0 : reinterpret_cast<int64_t>(slot >= 0 ? a.cache + slot * R : a.miss + idx * R);
     // write-through: second destination of a row that hit (0: none)
     const int64_t my_second_row =
         THROUGH && slot >= 0 ? reinterpret_cast<int64_t>(a.miss + idx * R) : 0;
@@ -145,7 +154,7 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int row = r0 + u * rows_per_step + grp;
-          if (row < nrows && in) {
+          if (row < nrows && in && (!DEFER || trow[u])) {
             if (SET)
               v[u] = __builtin_nontemporal_load(
                   reinterpret_cast<const VT *>(a.dense + (base + row) * R + my_off));
@@ -156,7 +165,7 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int row = r0 + u * rows_per_step + grp;
-          if (row < nrows && in) {
+          if (row < nrows && in && (!DEFER || trow[u])) {
             if (SET) {
               gstore<VT>(trow[u] + my_off, v[u]);
               if (THROUGH && second[u]) gstore<VT>(second[u] + my_off, v[u]);
@@ -172,7 +181,7 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
         char *trow = reinterpret_cast<char *>(shfl64(my_table_row, row & (kWave - 1)));
         char *second =
             THROUGH ? reinterpret_cast<char *>(shfl64(my_second_row, row & (kWave - 1))) : nullptr;
-        if (row >= nrows) continue;
+        if (row >= nrows || (DEFER && !trow)) continue;
         char *drow = a.dense + (base + row) * R;
         const char *src = SET ? drow : trow;
         char *dst = SET ? trow : drow;
@@ -195,6 +204,124 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
         }
       }
     }
+  }
+}
+
+// Second half of a fetch whose misses were set aside (rows_kernel with DEFER):
+// moves the rows marked in the bitmap from the id-addressed table. These are
+// host-link reads when the table lives in pinned host memory. The link is
+// saturated by the reads of a few dozen waves, and every read beyond that only
+// lengthens the queue that all other link traffic of the GPU (the cold
+// adjacency of the next mini-batch's sampling) and, measured, even its HBM
+// traffic waits in; so the grid is small by design and the rest of the GPU
+// stays free for what other streams have queued.
+// A wave takes kMissedChunk bitmap words (32 rows each) per pass: one lane per
+// word, a wave scan of the popcounts, the set bits expanded into a position
+// list in LDS; then lane groups move kMissedRows rows at a time, all their
+// loads issued before the first store.
+struct MissedArgs {
+  const char *table;
+  char *dense;
+  const void *indices;
+  const uint32_t *bits;
+  const int64_t *count;  // optional: only the first min(rows, *count) rows exist
+  int64_t rows;
+  int64_t row_bytes;
+  int idx_bytes;
+  int log2_lanes;
+};
+
+constexpr int kMissedRows = 2;     // rows a lane group has in flight
+constexpr int kMissedChunk = 32;   // bitmap words per wave pass: 1,024 rows
+constexpr int kMissedBlocks = 48;  // default grid
+
+__global__ __launch_bounds__(kRowsBlock) void rows_missed_kernel(MissedArgs a) {
+  using VT = u32x4;
+  __shared__ uint32_t positions[kRowsBlock / kWave][kMissedChunk * 32];
+  const int lane = lane_id();
+  const int L = 1 << a.log2_lanes;
+  const int gl = lane & (L - 1);
+  const int grp = lane >> a.log2_lanes;
+  const int rows_per_step = kWave >> a.log2_lanes;
+  const int per_pass = kMissedRows * rows_per_step;  // <= 16: lane groups hold 8 lanes at least
+  const int wave_in_block = threadIdx.x / kWave;
+  const int64_t waves_per_block = blockDim.x / kWave;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * waves_per_block + wave_in_block;
+  const int64_t nwaves = static_cast<int64_t>(gridDim.x) * waves_per_block;
+  const int64_t R = a.row_bytes;
+  const int64_t step = static_cast<int64_t>(L) * sizeof(VT);
+  const int64_t my_off = static_cast<int64_t>(gl) * sizeof(VT);
+  int64_t Q = a.rows;
+  if (a.count) {
+    const int64_t counted = *a.count;
+    if (counted < Q) Q = counted < 0 ? 0 : counted;
+  }
+  const int64_t nwords = (Q + 31) >> 5;
+  uint32_t *const mine = positions[wave_in_block];
+  // Words are dealt to the waves one by one (word w0 + lane * nwaves to lane `lane` of wave w0), not in
+  // runs: misses cluster (the first rows of a mini-batch's input nodes are its seeds, mostly cold), and a
+  // wave that owned a run of 1,024 such rows would still be moving them long after the others were done.
+  for (int64_t w0 = wave; w0 < nwords; w0 += nwaves * kMissedChunk) {
+    const int64_t my_word = w0 + lane * nwaves;
+    uint32_t word = 0;
+    if (lane < kMissedChunk && my_word < nwords) word = a.bits[my_word];
+    const uint32_t cnt = __builtin_popcount(word);
+    const uint32_t inc = wave_inclusive_scan(cnt);
+    const int total = static_cast<int>(wave_last(inc));
+    uint32_t at = inc - cnt;
+    while (word) {
+      mine[at++] = static_cast<uint32_t>(my_word << 5) + static_cast<uint32_t>(__builtin_ctz(word));
+      word &= word - 1;
+    }
+    // the list is written and read by this wave only: order its LDS accesses, no workgroup barrier
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int e0 = 0; e0 < total; e0 += per_pass) {
+      int64_t my_src = 0, my_dst = 0;
+      if (lane < per_pass && e0 + lane < total) {
+        const int64_t pos = mine[e0 + lane];
+        const int64_t idx = load_int(a.indices, pos, a.idx_bytes);
+        my_src = reinterpret_cast<int64_t>(a.table + idx * R);
+        my_dst = reinterpret_cast<int64_t>(a.dense + pos * R);
+      }
+      const char *src[kMissedRows];
+      char *dst[kMissedRows];
+#pragma unroll
+      for (int u = 0; u < kMissedRows; ++u) {
+        src[u] = reinterpret_cast<const char *>(shfl64(my_src, u * rows_per_step + grp));
+        dst[u] = reinterpret_cast<char *>(shfl64(my_dst, u * rows_per_step + grp));
+      }
+      for (int64_t off = my_off; off < R; off += step) {
+        VT v[kMissedRows];
+#pragma unroll
+        for (int u = 0; u < kMissedRows; ++u)
+          if (src[u]) v[u] = gload<VT>(src[u] + off);
+#pragma unroll
+        for (int u = 0; u < kMissedRows; ++u)
+          if (src[u]) __builtin_nontemporal_store(v[u], reinterpret_cast<VT *>(dst[u] + off));
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+template <bool ONE_VEC>
+static void launch_defer(int mode, unsigned grid, hipStream_t s, const RowArgs &a) {
+  switch (mode) {
+    case kMap16:
+      hipLaunchKernelGGL((rows_kernel<u32x4, kMap16, false, ONE_VEC, false, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+    case kMap8:
+      hipLaunchKernelGGL((rows_kernel<u32x4, kMap8, false, ONE_VEC, false, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+    case kMapFlat:
+      hipLaunchKernelGGL((rows_kernel<u32x4, kMapFlat, false, ONE_VEC, false, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
+    default:
+      hipLaunchKernelGGL((rows_kernel<u32x4, kMask, false, ONE_VEC, false, true>), dim3(grid), dim3(kRowsBlock), 0, s, a);
+      break;
   }
 }
 
@@ -266,7 +393,8 @@ template <bool SET>
 static int move_rows(const char *who, void *miss, void *cache, const void *indices, int idx_bytes,
                      const shmt_hashmap_t *map, const void *mask, int mask_bytes, void *dense,
                      int64_t Q, int64_t row_bytes, void *stream, bool through = false,
-                     const int64_t *count = nullptr, int64_t *count_seen = nullptr) {
+                     const int64_t *count = nullptr, int64_t *count_seen = nullptr,
+                     uint32_t *miss_bits = nullptr) {
   SHMT_REQUIRE(Q >= 0, "%s: Q must be >= 0", who);
   SHMT_REQUIRE(row_bytes > 0, "%s: row_bytes must be > 0", who);
   SHMT_REQUIRE(width_ok(idx_bytes), "%s: ID can only be int32 or int64 (idx_bytes=%d)", who, idx_bytes);
@@ -298,6 +426,7 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   a.row_bytes = row_bytes;
   a.idx_bytes = idx_bytes;
   a.mask_bytes = mask_bytes;
+  a.miss_bits = miss_bits;
 
   const int vb = pick_vector_bytes(row_bytes, miss, cache, dense);
   const int64_t nvec = row_bytes / vb;
@@ -308,10 +437,20 @@ static int move_rows(const char *who, void *miss, void *cache, const void *indic
   // (256 CUs x 8 waves); fewer rows per wave otherwise, down to one phase-2 step.
   int log2_tile = kMaxLog2Tile;
   while (log2_tile > 6 - log2_lanes && (Q >> log2_tile) < 2048) --log2_tile;
+  if (miss_bits) log2_tile = 5;  // one bitmap word per tile
   a.log2_tile = log2_tile;
   const unsigned grid = grid_for(Q, static_cast<int64_t>(kRowsBlock / kWave) << log2_tile, 256 * 32);
   hipStream_t s = as_stream(stream);
   const bool one_vec = nvec <= (1ll << log2_lanes);
+  if (miss_bits) {
+    SHMT_REQUIRE(!SET && mode != kDirect, "%s: only a fetch through a hashmap or mask sets its misses aside", who);
+    SHMT_REQUIRE(vb == 16, "%s: rows and tables must allow 16-byte accesses (row_bytes %lld)", who,
+                 static_cast<long long>(row_bytes));
+    SHMT_REQUIRE(Q < (1ll << 32), "%s: at most 2^32 - 1 rows", who);
+    if (one_vec) launch_defer<true>(mode, grid, s, a); else launch_defer<false>(mode, grid, s, a);
+    SHMT_LAUNCH_CHECK();
+    return SHMT_OK;
+  }
   switch (vb) {
     case 16: launch_vec<u32x4, SET>(one_vec, through, mode, grid, s, a); break;
     case 8: launch_vec<u32x2, SET>(one_vec, through, mode, grid, s, a); break;
@@ -343,6 +482,48 @@ int shmt_fetch_counted(const void *miss_data, const void *cache_data, const void
   return shmt::move_rows<false>("shmt_fetch_counted", const_cast<void *>(miss_data),
                                 const_cast<void *>(cache_data), indices, idx_bytes, map, mask,
                                 mask_bytes, out, max_rows, row_bytes, stream, false, count, count_seen);
+}
+
+int shmt_fetch_cached_part(const void *miss_data, const void *cache_data, const void *indices, int idx_bytes,
+                           const shmt_hashmap_t *map, const void *mask, int mask_bytes, void *out,
+                           int64_t max_rows, const int64_t *count, int64_t row_bytes, uint32_t *miss_bits,
+                           void *stream) {
+  SHMT_REQUIRE(miss_bits != nullptr || max_rows == 0, "shmt_fetch_cached_part: miss_bits is null");
+  SHMT_REQUIRE(map != nullptr || mask != nullptr, "shmt_fetch_cached_part: needs a hashmap or a mask");
+  return shmt::move_rows<false>("shmt_fetch_cached_part", const_cast<void *>(miss_data),
+                                const_cast<void *>(cache_data), indices, idx_bytes, map, mask, mask_bytes, out,
+                                max_rows, row_bytes, stream, false, count, nullptr, miss_bits);
+}
+
+int shmt_fetch_missed_part(const void *miss_data, const void *indices, int idx_bytes, const uint32_t *miss_bits,
+                           void *out, int64_t max_rows, const int64_t *count, int64_t row_bytes, int max_blocks,
+                           void *stream) {
+  using namespace shmt;
+  SHMT_REQUIRE(width_ok(idx_bytes), "shmt_fetch_missed_part: ID can only be int32 or int64 (idx_bytes=%d)", idx_bytes);
+  SHMT_REQUIRE(max_rows >= 0 && max_rows < (1ll << 32), "shmt_fetch_missed_part: max_rows must be in [0, 2^32)");
+  SHMT_REQUIRE(max_blocks >= 0, "shmt_fetch_missed_part: max_blocks must be >= 0");
+  if (max_rows == 0) return SHMT_OK;
+  SHMT_REQUIRE(miss_data && indices && miss_bits && out, "shmt_fetch_missed_part: null buffer");
+  SHMT_REQUIRE(row_bytes > 0 && pick_vector_bytes(row_bytes, miss_data, out, nullptr) == 16,
+               "shmt_fetch_missed_part: rows and tables must allow 16-byte accesses (row_bytes %lld)",
+               static_cast<long long>(row_bytes));
+  MissedArgs a;
+  a.table = static_cast<const char *>(miss_data);
+  a.dense = static_cast<char *>(out);
+  a.indices = indices;
+  a.bits = miss_bits;
+  a.count = count;
+  a.rows = max_rows;
+  a.row_bytes = row_bytes;
+  a.idx_bytes = idx_bytes;
+  int log2_lanes = 3;
+  while (log2_lanes < 6 && (1ll << log2_lanes) < row_bytes / 16) ++log2_lanes;
+  a.log2_lanes = log2_lanes;
+  const int64_t chunks = ((max_rows + 31) / 32 + kMissedChunk - 1) / kMissedChunk;
+  const unsigned grid = grid_for(chunks, kRowsBlock / kWave, max_blocks > 0 ? max_blocks : kMissedBlocks);
+  hipLaunchKernelGGL(rows_missed_kernel, dim3(grid), dim3(kRowsBlock), 0, as_stream(stream), a);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
 }
 
 int shmt_set(void *miss_data, void *cache_data, const void *indices, int idx_bytes,

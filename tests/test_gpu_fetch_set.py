@@ -353,6 +353,82 @@ def test_c_abi_fetch_with_the_row_count_in_device_memory(cabi, route, count):
         lib.shmt_hashmap_destroy(hnd)
 
 
+@pytest.mark.parametrize("route", ["map", "mask"])
+@pytest.mark.parametrize("D", [4, 48, 256, 1000])
+@pytest.mark.parametrize("count", [None, 0, 1, 700, 9000])
+def test_c_abi_fetch_in_two_launches_equals_fetch(cabi, route, D, count):
+    """shmt_fetch_cached_part (hits now, the misses marked in a bitmap) followed by shmt_fetch_missed_part on
+    another stream gives what shmt_fetch / shmt_fetch_counted gives: every row once, hits from the cache
+    (told apart by content), misses from the pinned host table, rows past the count untouched."""
+    import ctypes
+    lib = cabi.load()
+    g = torch.Generator().manual_seed(D + (count or 3))
+    n, c, max_rows = 6000, 2500, 5000
+    table = torch.randn(n, D, generator=g).pin_memory()
+    table_dev = ctypes.c_void_p()
+    cabi.check(lib.shmt_host_devptr(table.data_ptr(), ctypes.byref(table_dev)))
+    ids = torch.randperm(n, generator=g)[:c]
+    cache = (table[ids] + 1.0).cuda()
+    idx = torch.randint(0, n, (max_rows,), generator=g)
+    slot_of = torch.full((n,), -1, dtype=torch.int64)
+    slot_of[ids] = torch.arange(c)
+    expect = torch.where((slot_of[idx] >= 0)[:, None], table[idx] + 1.0, table[idx])
+    idx_dev = idx.cuda()
+    hnd, mask, keep = None, None, []
+    if route == "map":
+        keys, vals = ids.cuda(), torch.arange(c).cuda()
+        nbytes = lib.shmt_hashmap_table_bytes(c, 0.8, 8, 8)
+        keep.append(torch.empty(nbytes, dtype=torch.uint8).cuda())
+        hnd = ctypes.c_void_p()
+        cabi.check(lib.shmt_hashmap_create(ctypes.byref(hnd), keys.data_ptr(), vals.data_ptr(), c, 8, 8, 0.8,
+                                           keep[0].data_ptr(), nbytes, cabi.current_stream()))
+    else:
+        mask = slot_of[idx].cuda()
+    out = torch.full((max_rows, D), -7.0).cuda()
+    count_dev = torch.tensor([count if count is not None else 0]).cuda()
+    words = (max_rows + 31) // 32
+    marks = torch.full((words,), 0x5A5A5A5A, dtype=torch.int32).cuda()      # needs no clearing
+    side = torch.cuda.Stream()
+    cabi.check(lib.shmt_fetch_cached_part(table_dev, cache.data_ptr(), idx_dev.data_ptr(), 8, hnd,
+                                          mask.data_ptr() if mask is not None else None,
+                                          8 if mask is not None else 0, out.data_ptr(), max_rows,
+                                          count_dev.data_ptr() if count is not None else None, D * 4,
+                                          marks.data_ptr(), cabi.current_stream()))
+    side.wait_stream(torch.cuda.current_stream())
+    cabi.check(lib.shmt_fetch_missed_part(table_dev, idx_dev.data_ptr(), 8, marks.data_ptr(), out.data_ptr(),
+                                          max_rows, count_dev.data_ptr() if count is not None else None, D * 4, 3,
+                                          side.cuda_stream))
+    side.synchronize()
+    torch.cuda.synchronize()
+    moved = max_rows if count is None else min(count, max_rows)
+    miss_np = (slot_of[idx[:moved]] < 0).numpy()
+    got = np.unpackbits(marks.cpu().numpy().view(np.uint8), bitorder="little")[:moved].astype(bool)
+    assert np.array_equal(got, miss_np)                       # every existing row is marked or cleared
+    assert torch.equal(out[:moved].cpu(), expect[:moved])
+    assert bool((out[moved:] == -7.0).all())
+    # the one-launch form on the same input
+    whole = torch.full((max_rows, D), -7.0).cuda()
+    if count is None:
+        cabi.check(lib.shmt_fetch(table_dev, cache.data_ptr(), idx_dev.data_ptr(), 8, hnd,
+                                  mask.data_ptr() if mask is not None else None, 8 if mask is not None else 0,
+                                  whole.data_ptr(), max_rows, D * 4, cabi.current_stream()))
+    else:
+        cabi.check(lib.shmt_fetch_counted(table_dev, cache.data_ptr(), idx_dev.data_ptr(), 8, hnd,
+                                          mask.data_ptr() if mask is not None else None,
+                                          8 if mask is not None else 0, whole.data_ptr(), max_rows,
+                                          count_dev.data_ptr(), None, D * 4, cabi.current_stream()))
+    assert torch.equal(whole, out)
+    # rows that do not allow 16-byte accesses are refused, not mis-read
+    assert lib.shmt_fetch_cached_part(table_dev, cache.data_ptr(), idx_dev.data_ptr(), 8, hnd,
+                                      mask.data_ptr() if mask is not None else None, 8 if mask is not None else 0,
+                                      out.data_ptr(), max_rows, None, D * 4 - 4, marks.data_ptr(),
+                                      cabi.current_stream()) != 0
+    assert b"16-byte" in lib.shmt_last_error()
+    if hnd is not None:
+        torch.cuda.synchronize()
+        lib.shmt_hashmap_destroy(hnd)
+
+
 @pytest.mark.parametrize("D,dtype", [(32, torch.float32), (64, torch.float16), (7, torch.int8), (300, torch.float32)])
 @pytest.mark.parametrize("slots", ["8-byte", "16-byte"])
 def test_fetch_and_set_through_bucket_tables(capi, oracle, D, dtype, slots):
