@@ -715,6 +715,8 @@ def bench_e2e(capi, args, result):
     cap = int(1.25 * inp.numel())
     fetched_ms = {}
     for k_in_flight in (1, 2, 4):
+        # (the warm-up's results are dropped before the timed call, as a training loop drops each batch: the
+        # caching allocator then hands their blocks out again instead of asking the driver for new memory)
         capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats, feat_cache,
                                  feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
         torch.cuda.synchronize()

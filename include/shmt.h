@@ -473,6 +473,14 @@ typedef struct shmt_hop_job {
 } shmt_hop_job;
 int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream);
 
+/* Queues one wave that stays busy for about `microseconds` (0 .. 100,000)
+ * and touches no memory. No counterpart in the reference. For callers that
+ * spread work over several streams: streams share a small number of
+ * hardware queues, two streams on one queue run one after the other, and
+ * the runtime does not say which share; a short wait queued on one stream
+ * and an event on another show it (the shim's side-stream choice).        */
+int shmt_busy_wait(void *stream, int microseconds);
+
 /* Replaying a mini-batch. The hops of a batch, queued with
  * shmt_sample_hop_chained on fixed buffers, never wait for the host, so the
  * whole sequence can be captured once as a HIP graph and replayed for every

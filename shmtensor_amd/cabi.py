@@ -59,6 +59,7 @@ SIGNATURES = {
                                        _c.c_uint64, _vp, _c.c_uint32, _vp, _vp, _vp, _i64, _int, _vp, _vp, _i64,
                                        _vp, _vp, _vp, _vp, _vp, _vp]),
     "shmt_sample_hops_chained": (_int, [_vp, _int, _vp]),
+    "shmt_busy_wait": (_int, [_vp, _int]),
     "shmt_capture_begin": (_int, [_vp]),
     "shmt_capture_end": (_int, [_vp, _c.POINTER(_vp)]),
     "shmt_graph_launch": (_int, [_vp, _vp]),

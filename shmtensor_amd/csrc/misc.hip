@@ -45,9 +45,28 @@ __global__ __launch_bounds__(256) void stage_seeds_kernel(const void *src, int s
 
 }  // namespace shmt
 
+namespace shmt {
+
+// One wave that stays busy for about `ticks` of the 100 MHz wall clock (and at
+// most `max_sleeps` sleep instructions, so it ends whatever the clock does).
+__global__ __launch_bounds__(64) void busy_wait_kernel(unsigned long long ticks, int max_sleeps) {
+  const unsigned long long t0 = wall_clock64();
+  for (int i = 0; i < max_sleeps && wall_clock64() - t0 < ticks; ++i) __builtin_amdgcn_s_sleep(64);
+}
+
+}  // namespace shmt
+
 using namespace shmt;
 
 extern "C" {
+
+int shmt_busy_wait(void *stream, int microseconds) {
+  SHMT_REQUIRE(microseconds >= 0 && microseconds <= 100000, "shmt_busy_wait: 0 .. 100,000 microseconds");
+  hipLaunchKernelGGL(busy_wait_kernel, dim3(1), dim3(64), 0, as_stream(stream),
+                     static_cast<unsigned long long>(microseconds) * 100ull, microseconds + 16);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
+}
 
 int shmt_stage_seeds(const void *seeds, int seed_bytes, int64_t n, void *staged, int staged_bytes,
                      int64_t *len_out, uint64_t rng_seed, uint64_t *rng_seed_out, void *stream) {

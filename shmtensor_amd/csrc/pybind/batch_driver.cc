@@ -506,6 +506,61 @@ std::vector<BatchResult> finish_together(const CsrArgs &g, std::vector<TogetherB
   return out;
 }
 
+// Side streams of the pipelined fetch: two for the host-link launches, taken in turn, and one for the
+// launch that moves the cached rows. Streams share a few hardware queues (four per process by default),
+// work of two streams on one queue runs one after the other, and the runtime does not tell which stream
+// sits on which queue: so the three are chosen, once per calling stream, by trying pool streams until
+// three are found that make progress while the calling stream and the ones chosen before are kept busy
+// (a 300 us wait on each; a stream that shares a queue with any of them cannot finish a kernel before
+// that wait ends). When fewer than three such streams exist the remaining roles take what is left: the
+// results do not depend on the choice, only the overlap does.
+struct SideStreams {
+  c10::hip::HIPStreamMasqueradingAsCUDA link, link2, hits;
+};
+
+bool runs_beside(const c10::hip::HIPStreamMasqueradingAsCUDA &candidate,
+                 const std::vector<c10::hip::HIPStreamMasqueradingAsCUDA> &busy) {
+  std::vector<at::cuda::CUDAEvent> waits(busy.size());
+  for (size_t i = 0; i < busy.size(); ++i) {
+    check(shmt_busy_wait(busy[i].stream(), 300));
+    waits[i].record(busy[i]);
+  }
+  check(shmt_busy_wait(candidate.stream(), 0));
+  at::cuda::CUDAEvent done;
+  done.record(candidate);
+  done.synchronize();
+  bool beside = true;
+  for (auto &w : waits) beside = beside && !w.query();
+  for (auto &w : waits) w.synchronize();
+  return beside;
+}
+
+SideStreams side_streams_for(const c10::hip::HIPStreamMasqueradingAsCUDA &caller) {
+  static std::mutex mutex;
+  static std::unordered_map<uint64_t, SideStreams> chosen;  // by device and calling stream
+  const c10::DeviceIndex device = caller.device_index();
+  const uint64_t key = (static_cast<uint64_t>(device) << 48) ^ static_cast<uint64_t>(caller.id());
+  std::lock_guard<std::mutex> lock(mutex);
+  auto it = chosen.find(key);
+  if (it != chosen.end()) return it->second;
+  std::vector<c10::hip::HIPStreamMasqueradingAsCUDA> pool, busy{caller}, picked;
+  for (int i = 0; i < 12; ++i) pool.push_back(c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, device));
+  for (const auto &s : pool) {
+    if (picked.size() == 3) break;
+    if (s == caller || std::find(picked.begin(), picked.end(), s) != picked.end()) continue;
+    if (runs_beside(s, busy)) {
+      picked.push_back(s);
+      busy.push_back(s);
+    }
+  }
+  for (const auto &s : pool)  // not enough independent queues: any other stream will do
+    if (picked.size() < 3 && !(s == caller) && std::find(picked.begin(), picked.end(), s) == picked.end())
+      picked.push_back(s);
+  const SideStreams side{picked[0], picked[1], picked[2]};
+  chosen.emplace(key, side);
+  return side;
+}
+
 // Multi-hop sampling of several independent seed batches. Every batch is a
 // chain of short, latency-bound kernels with a host read of the sizes at its end,
 // so one batch alone leaves most of the GPU idle. Batches whose hops all chain
@@ -540,11 +595,6 @@ std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch
   // With several batches to drive and the feature table in host memory, the rows that miss the cache
   // are fetched on the device's link stream (see FeatureArgs::link): batch b's host-link reads then
   // run beside batch b + 1's sampling, whatever the number of host threads.
-  static std::mutex link_mutex;
-  struct SideStreams {
-    c10::hip::HIPStreamMasqueradingAsCUDA link, link2, hits;
-  };
-  static std::unordered_map<int, SideStreams> side_streams;
   std::atomic<uint32_t> turn{0};
   FeatureArgs with_link;
   if (features && B > 1 && features->cached() && !features->uva_data.is_cuda()) {
@@ -553,18 +603,10 @@ std::vector<BatchResult> drive_batches(const CsrArgs &g, const std::vector<torch
     with_link.hashmap = features->hashmap;
     with_link.max_rows = features->max_rows;
     with_link.uva_dev = features->uva_dev;
-    std::lock_guard<std::mutex> lock(link_mutex);
-    auto it = side_streams.find(static_cast<int>(device));
-    if (it == side_streams.end())
-      it = side_streams
-               .emplace(static_cast<int>(device),
-                        SideStreams{c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, device),
-                                    c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, device),
-                                    c10::hip::getStreamFromPoolMasqueradingAsCUDA(false, device)})
-               .first;
-    with_link.link = it->second.link;
-    with_link.link2 = it->second.link2;
-    with_link.hits = it->second.hits;
+    const SideStreams side = side_streams_for(caller);
+    with_link.link = side.link;
+    with_link.link2 = side.link2;
+    with_link.hits = side.hits;
     with_link.turn = &turn;
     features = &with_link;
   }

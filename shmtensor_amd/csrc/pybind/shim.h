@@ -10,6 +10,7 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cstdint>
