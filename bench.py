@@ -46,16 +46,19 @@ CONFIG4_PMC_SUMMARY = os.path.join(ROOT, "profiles", "rows_kernel_fetch_config4_
 
 
 def config4_traffic_bytes():
-    """`roofline.traffic`: the figure the counter summary under profiles/ states ("traffic_bytes_per_launch: N"),
-    or None when the summary is absent."""
+    """`roofline.traffic` per map layout: the figures the counter summary under profiles/ states on lines
+    "traffic_bytes_per_launch[<layout>]: N"; an empty dict when the summary is absent."""
+    found = {}
     try:
         with open(CONFIG4_PMC_SUMMARY) as f:
             for line in f:
-                if line.strip().startswith("traffic_bytes_per_launch:"):
-                    return int(line.split(":")[1].split()[0].replace(",", ""))
+                line = line.strip()
+                if line.startswith("traffic_bytes_per_launch["):
+                    layout = line[line.index("[") + 1:line.index("]")]
+                    found[layout] = int(line.split(":")[1].split()[0].replace(",", ""))
     except OSError:
         pass
-    return None
+    return found
 
 
 def log(*a):
@@ -126,47 +129,65 @@ def bench_fetch(capi, args, result):
     log("[fetch] table %d x %d fp16 (%.1f GB pinned), cache %d rows (%.2f GB HBM): %.1f s"
         % (N, D, N * R / 1e9, C, C * R / 1e9, time.time() - t0))
     keys = torch.arange(C, device="cuda")
-    hmap = capi.CUCOStaticHashmap(keys, keys.clone(), 0.8)
+    # The timed map is the general bucket table (int64 -> int64: 16-byte slots, one 128-byte bucket line per
+    # probe), built whatever the keys look like, as the reference's cuco::static_map is. Left to itself the
+    # constructor recognises this configuration's keys (ids 0 .. C-1 -> slot = id) as an id range and builds
+    # no table at all; that form is timed beside it and reported as roofline_auto_layout.
+    hmap = capi.CUCOStaticHashmap(keys, keys.clone(), 0.8, layout="buckets")
+    hmap_auto = capi.CUCOStaticHashmap(keys, keys.clone(), 0.8)
     del keys
     nb = 8
     batches = [zipf_ranks(Q, N, 1.1, seed=100 + i) for i in range(nb)]
     hit_rate = float((batches[0] < C).float().mean())
 
     # correctness of the timed operator on the timed input (bit patterns)
-    out = capi.cache_fetch(host, cache, batches[0], hmap)
     ref = torch.index_select(host.view(torch.int16), 0, batches[0].cpu())
-    assert torch.equal(out.cpu().view(torch.int16), ref), "cache_fetch differs from index_select"
-    del out, ref
+    for m in (hmap, hmap_auto):
+        out = capi.cache_fetch(host, cache, batches[0], m)
+        assert torch.equal(out.cpu().view(torch.int16), ref), "cache_fetch differs from index_select"
+        del out
+    del ref
 
     W, K = args.warmup, args.steps
-    for i in range(W):
-        capi.cache_fetch(host, cache, batches[i % nb], hmap)
-    torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
-    t0 = time.perf_counter()
-    for i in range(K):
-        ev[i][0].record()
-        capi.cache_fetch(host, cache, batches[i % nb], hmap)
-        ev[i][1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kern_ms = sum(a.elapsed_time(b) for a, b in ev) / K
-    ms_per_step = wall * 1e3 / K
-    value = Q * R / (ms_per_step * 1e-3) / 1e9
     algo_bytes = Q * (2 * R + 8)
-    achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
-    result.update({
-        "value": round(value, 2), "ms_per_step": round(ms_per_step, 4),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": config4_traffic_bytes() if N == 100_000_000 else None,
-                     "kernel": "rows_kernel<u32x4, %s, fetch>" % ("map_flat" if hmap.layout() != "buckets" else "map8"),
-                     "kernel_ms": round(kern_ms, 4),
-                     "bytes_per_launch": algo_bytes},
-    })
+
+    def timed_steps(m):
+        for i in range(W):
+            capi.cache_fetch(host, cache, batches[i % nb], m)
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+        t0 = time.perf_counter()
+        for i in range(K):
+            ev[i][0].record()
+            capi.cache_fetch(host, cache, batches[i % nb], m)
+            ev[i][1].record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        kern_ms = sum(a.elapsed_time(b) for a, b in ev) / K
+        return wall * 1e3 / K, kern_ms
+
+    def roofline_of(m, kern_ms, traffic):
+        achieved = algo_bytes / (kern_ms * 1e-3) / 1e9
+        fmt = {"buckets": "map16" if m.memory_usage() >= 16 * 2 * C else "map8"}.get(m.layout(), "map_flat")
+        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "kernel": "rows_kernel<u32x4, %s, fetch>" % fmt, "kernel_ms": round(kern_ms, 4),
+                "bytes_per_launch": algo_bytes, "map_layout": m.layout(), "map_bytes": m.memory_usage()}
+
+    traffic = config4_traffic_bytes() if N == 100_000_000 else {}
+    if args.headline_only and args.headline_map == "auto":      # profiler runs of the id-range form only
+        hmap = hmap_auto
+    ms_per_step, kern_ms = timed_steps(hmap)
+    value = Q * R / (ms_per_step * 1e-3) / 1e9
+    result.update({"value": round(value, 2), "ms_per_step": round(ms_per_step, 4),
+                   "roofline": roofline_of(hmap, kern_ms, traffic.get("range" if hmap is hmap_auto else "buckets"))})
     result["config"].update({"workload": "config 4: cache_fetch, %d x %d fp16 table pinned, %d rows cached, "
-                             "Q=%d Zipf(1.1)" % (N, D, C, Q), "hit_rate": round(hit_rate, 4),
+                             "Q=%d Zipf(1.1), general bucket hashmap" % (N, D, C, Q), "hit_rate": round(hit_rate, 4),
                              "row_bytes": R, "queries_per_step": Q, "map_layout": hmap.layout()})
+    if not args.headline_only:
+        ms_auto, kern_auto = timed_steps(hmap_auto)
+        result["roofline_auto_layout"] = roofline_of(hmap_auto, kern_auto, traffic.get("range"))
+        result["roofline_auto_layout"]["value_GBs"] = round(Q * R / (ms_auto * 1e-3) / 1e9, 2)
     extra = result["extra"]
     if args.headline_only:
         del host, cache, hmap
@@ -209,11 +230,11 @@ def bench_fetch(capi, args, result):
                                             "algorithmic_GBs": round(algo_bytes / t["median"] / 1e6, 1)}
     # all-hit: uniform queries over the cached ids (no locality), HBM bound
     qh = torch.randint(0, C, (Q,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
-    t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qh, hmap), 30)
+    t = gpu_time_ms(lambda: capi.cache_fetch(host, cache, qh, hmap_auto), 30)
     a = algo_bytes / (t["median"] * 1e-3) / 1e9
     extra["fetch_all_hit"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "algorithmic_GBs": round(a, 1),
                               "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4), "payload_GBs": round(Q * R / t["median"] / 1e6, 1),
-                              "map_layout": hmap.layout(),
+                              "map_layout": hmap_auto.layout(),
                               "note": "the configuration's own map: ids 0..C-1 -> slot = id, recognised as an id range"}
     tm = gpu_time_ms(lambda: capi.cache_fetch_with_mask(host, cache, qh, qh), 30)
     a = algo_bytes / (tm["median"] * 1e-3) / 1e9
@@ -317,7 +338,7 @@ def bench_fetch(capi, args, result):
         set_t = (time.perf_counter() - t1) / 5
         extra["cache_set_262144"]["cpu_index_put_ms"] = round(set_t * 1e3, 3)
         extra["cache_set_262144"]["cpu_threads"] = torch.get_num_threads()
-    del host, cache, hmap
+    del host, cache, hmap, hmap_auto
 
 
 # ---------------------------------------------------------------------------
@@ -847,6 +868,8 @@ def main():
     ap.add_argument("--e2e-batches", type=int, default=24)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--headline-map", default="buckets", choices=["buckets", "auto"],
+                    help="with --headline-only: which map's launches to run (for profiler runs)")
     ap.add_argument("--headline-only", action="store_true",
                     help="fetch workload: only the timed config-4 steps (used for profiler runs, so that "
                          "every launch of the fetch kernel in the trace belongs to the headline workload)")

@@ -102,9 +102,13 @@ int shmt_hashmap_create(shmt_hashmap_t **out, const void *keys,
  * bits, whatever their dtype. Every form answers exactly like the general
  * table (same contract as the constructor above: include/cuco_hashmap.cuh:
  * 57-87). shmt_hashmap_plan looks at the keys and values (one sweep, plus a
- * repeat check for range candidates), SYNCHRONISES the stream once and fills
+ * repeat check for range candidates), SYNCHRONISES the stream once (twice
+ * for a range candidate, whose repeat check is a second read-back) and fills
  * `layout`, including the table_bytes the caller has to provide;
- * shmt_hashmap_create_planned then builds that layout (asynchronous).
+ * shmt_hashmap_create_planned then builds that layout (asynchronous). The
+ * layout must come from shmt_hashmap_plan on the same, unchanged keys and
+ * values: the build trusts it (a rank layout is only re-checked for
+ * n < 2^32, the width of its running counts).
  * `scratch` is device memory of shmt_hashmap_plan_scratch_bytes(n) bytes,
  * 16-byte aligned, free again when plan returns.                            */
 #define SHMT_MAP_BUCKETS 0

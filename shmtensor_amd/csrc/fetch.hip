@@ -114,13 +114,23 @@ __global__ __launch_bounds__(kRowsBlock, ONE_VEC ? kRowsWavesPerSimd : kRowsWave
     int64_t slot = -1;
     if (MODE == kMask) {
       if (live) slot = load_int(a.mask, i, a.mask_bytes);
-    } else if (MODE == kMap16) {
-      slot = wave_find<kSlot16, kFindBatch>(a.map, live ? map_key(a.map, idx) : -1);
-    } else if (MODE == kMap8) {
-      slot = wave_find<kSlot8, kFindBatch>(a.map, live ? map_key(a.map, idx) : -1);
+    } else if (MODE == kMap16 || MODE == kMap8) {
+      constexpr int FMT = MODE == kMap16 ? kSlot16 : kSlot8;
+      const int64_t key = live ? map_key(a.map, idx) : -1;
+      if (tile > 32)
+        slot = wave_find<FMT, kFindBatch>(a.map, key);
+      else if (tile_repeats(key, live))
+        slot = half_wave_find<FMT, false>(a.map, key);
+      else
+        slot = half_wave_find<FMT, true>(a.map, key);
     } else if (MODE == kMapFlat) {
-      // direct or range form of the map: one 4-byte load, or arithmetic only
-      if (live) slot = flat_find(a.map, map_key(a.map, idx));
+      // direct, rank or range form of the map: one load, or arithmetic only
+      const int64_t key = live ? map_key(a.map, idx) : -1;
+      if (a.map.kind == kKindDirect && !tile_repeats(key, live)) {
+        if (live) slot = flat_find<true>(a.map, key);
+      } else {
+        if (live) slot = flat_find<false>(a.map, key);
+      }
     }
     if (DEFER) {
       const uint64_t missed = __builtin_amdgcn_ballot_w64(live && slot < 0);

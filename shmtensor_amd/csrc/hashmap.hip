@@ -503,6 +503,8 @@ int shmt_hashmap_create_planned(shmt_hashmap_t **out, const shmt_hashmap_layout 
                "shmt_hashmap_create_planned: unknown layout kind %d", layout->kind);
   SHMT_REQUIRE(n > 0 && keys != nullptr && vals != nullptr && layout->lo >= 0 && layout->span > 0,
                "shmt_hashmap_create_planned: a flat layout needs keys and a non-negative id range");
+  SHMT_REQUIRE(layout->kind != SHMT_MAP_RANK || n < (1ll << 32),
+               "shmt_hashmap_create_planned: a rank layout holds fewer than 2^32 keys (32-bit running counts)");
   hipStream_t s = as_stream(stream);
   if (layout->kind == SHMT_MAP_DIRECT) {
     if (table_mem == nullptr || table_bytes < layout->table_bytes || layout->table_bytes < layout->span * 4) {

@@ -442,7 +442,8 @@ PYBIND11_MODULE(ShmTensorLib, m) {
   register_batch_sampler(m);
 
   py::class_<StaticHashmap>(m, "CUCOStaticHashmap")
-      .def(py::init<torch::Tensor, torch::Tensor, double>())
+      .def(py::init<torch::Tensor, torch::Tensor, double, const std::string &>(), py::arg("keys"), py::arg("values"),
+           py::arg("load_factor"), py::arg("layout") = "auto")
       .def("query", &StaticHashmap::query)
       .def("capacity", &StaticHashmap::capacity)
       .def("memory_usage", &StaticHashmap::memory_usage)

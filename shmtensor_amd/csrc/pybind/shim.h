@@ -141,9 +141,14 @@ inline torch::Tensor device_bytes(int64_t nbytes) {
 
 class StaticHashmap {
  public:
-  StaticHashmap(torch::Tensor keys, torch::Tensor values, double load_factor) {
+  // `layout`: "auto" looks at the keys and builds the cheapest form that answers like the general table
+  // (an id range, a rank bitmap, a direct table, narrow bucket slots); "buckets" builds the general bucket
+  // table in the slot format the dtypes call for, whatever the keys look like (what cuco::static_map holds
+  // in the reference, include/cuco_hashmap.cuh:57-77).
+  StaticHashmap(torch::Tensor keys, torch::Tensor values, double load_factor, const std::string &layout_choice = "auto") {
     TORCH_CHECK(keys.is_cuda(), "keys must be a CUDA tensor");
     TORCH_CHECK(values.is_cuda(), "values must be a CUDA tensor");
+    TORCH_CHECK(layout_choice == "auto" || layout_choice == "buckets", "layout must be \"auto\" or \"buckets\"");
     key_type_ = keys.scalar_type();
     value_type_ = values.scalar_type();
     const int kb = id_bytes(keys, "keys"), vb = id_bytes(values, "values");
@@ -153,6 +158,15 @@ class StaticHashmap {
     values = values.contiguous();
     const int64_t n = keys.numel();
     capacity_ = shmt_hashmap_capacity(n, load_factor);
+    if (layout_choice == "buckets") {
+      const int64_t bytes = shmt_hashmap_table_bytes(n, load_factor, kb, vb);
+      table_ = device_bytes(bytes);
+      memory_usage_ = bytes;
+      kind_ = SHMT_MAP_BUCKETS;
+      check(shmt_hashmap_create(&handle_, keys.data_ptr(), values.data_ptr(), n, kb, vb, load_factor,
+                                table_.data_ptr(), bytes, current_stream()));
+      return;
+    }
     // the layout follows from the keys (dense id range, 32-bit ids ...): look first, then allocate what it needs
     shmt_hashmap_layout layout;
     {
