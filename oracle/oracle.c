@@ -304,29 +304,170 @@ ORC_EXPORT int64_t orc_relabel(const int64_t *total, int64_t N, int64_t *unique,
  * baselines): one sequential sweep, open addressing with a mixed hash, a new
  * id is appended to `unique` the first time it is met. First-occurrence order
  * falls out of the sweep order, so no index table, no counting pass and no
- * scan are needed (src/tensor_relabel.cu:127-130, 206-208 for the contract). */
+ * scan are needed (src/tensor_relabel.cu:127-130, 206-208 for the contract).
+ * The table is kept between calls and emptied by the slots a call used. Not
+ * re-entrant. */
+static int64_t *g_sw_key = NULL, *g_sw_val = NULL; /* kept between calls, emptied by the slots a call used */
+static uint64_t *g_sw_used = NULL;
+static uint64_t g_sw_cap = 0;
+
 ORC_EXPORT int64_t orc_relabel_sweep(const int64_t *total, int64_t N, int64_t *unique, int64_t *labels) {
   if (N == 0) return 0;
   uint64_t cap = 16;
   while (cap < (uint64_t)N * 2) cap <<= 1;
-  int64_t *kt = (int64_t *)malloc(sizeof(int64_t) * cap);
-  int64_t *vt = (int64_t *)malloc(sizeof(int64_t) * cap);
-  memset(kt, 0xff, sizeof(int64_t) * cap); /* -1: empty */
+  if (cap > g_sw_cap) {
+    free(g_sw_key);
+    free(g_sw_val);
+    free(g_sw_used);
+    g_sw_key = (int64_t *)malloc(sizeof(int64_t) * cap);
+    g_sw_val = (int64_t *)malloc(sizeof(int64_t) * cap);
+    g_sw_used = (uint64_t *)malloc(sizeof(uint64_t) * (cap / 2));
+    g_sw_cap = cap;
+    memset(g_sw_key, 0xff, sizeof(int64_t) * cap); /* -1: empty */
+  }
+  int64_t *const kt = g_sw_key, *const vt = g_sw_val;
+  const uint64_t mask = g_sw_cap - 1;
   int64_t count = 0;
   for (int64_t i = 0; i < N; ++i) {
     const int64_t key = total[i];
-    uint64_t pos = mix64((uint64_t)key) & (cap - 1);
-    while (kt[pos] != -1 && kt[pos] != key) pos = (pos + 1) & (cap - 1);
+    uint64_t pos = mix64((uint64_t)key) & mask;
+    while (kt[pos] != -1 && kt[pos] != key) pos = (pos + 1) & mask;
     if (kt[pos] == -1) {
       kt[pos] = key;
       vt[pos] = count;
+      g_sw_used[count] = pos;
       unique[count++] = key;
     }
     labels[i] = vt[pos];
   }
-  free(kt);
-  free(vt);
+  for (int64_t u = 0; u < count; ++u) kt[g_sw_used[u]] = -1;
   return count;
+}
+
+/* The same contract on all host cores (the tuned CPU baseline of bench.py, not
+ * a restatement of the reference's kernel structure), without atomics: ids are dealt to one
+ * partition per thread by the top bits of their mixed hash, each partition in
+ * index order (a counting pass and a scatter pass over the threads' chunks),
+ * every thread then sweeps ITS partition with a private table exactly as
+ * orc_relabel_sweep does (first occurrences fall out of the index order), the
+ * first-occurrence flags are ranked by a two-level prefix sum, and a last pass
+ * maps every element's first index to its rank. All tables and buffers are
+ * kept between calls. Small inputs take the sequential sweep, which wins there.
+ * Not re-entrant. Contract: src/tensor_relabel.cu:127-130, 206-208. */
+typedef struct {
+  uint32_t *items;  /* indices dealt to the partitions, partition after partition */
+  uint32_t *first;  /* per element: index of the first occurrence of its id */
+  uint32_t *rank;   /* per index: number of first occurrences before it */
+  int64_t items_cap;
+  uint64_t *key;    /* private tables, one region per thread */
+  uint32_t *val;
+  uint64_t table_cap; /* slots per thread */
+  int threads;
+} RlPartState;
+static RlPartState g_part = {0};
+
+ORC_EXPORT int64_t orc_relabel_parallel(const int64_t *total, int64_t N, int64_t *unique, int64_t *labels) {
+  if (N < 16384 || N >= ((int64_t)1 << 31)) return orc_relabel_sweep(total, N, unique, labels);
+  const int T = omp_get_max_threads();
+  int shift = 64;
+  int parts = 1;
+  while (parts < T) { parts <<= 1; --shift; } /* partitions: power of two >= threads, dealt round-robin */
+  RlPartState *g = &g_part;
+  if (N > g->items_cap) {
+    free(g->items); free(g->first); free(g->rank);
+    g->items = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)N);
+    g->first = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)N);
+    g->rank = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)(N + 1));
+    g->items_cap = N;
+  }
+  /* a partition holds N / parts ids on average; tables sized for four times that (load <= 0.5 at twice the mean) */
+  uint64_t want = 1024;
+  while (want < (uint64_t)(N / parts + 1) * 4) want <<= 1;
+  if (want > g->table_cap || parts != g->threads) {
+    free(g->key); free(g->val);
+    g->key = (uint64_t *)malloc(sizeof(uint64_t) * want * (size_t)parts);
+    g->val = (uint32_t *)malloc(sizeof(uint32_t) * want * (size_t)parts);
+    g->table_cap = want;
+    g->threads = parts;
+    memset(g->key, 0xff, sizeof(uint64_t) * want * (size_t)parts);
+  }
+  int64_t *counts = (int64_t *)calloc((size_t)T * parts + 1, sizeof(int64_t)); /* [thread][partition] */
+  int64_t *starts = (int64_t *)calloc((size_t)parts + 1, sizeof(int64_t));
+  int64_t *firsts = (int64_t *)calloc((size_t)T + 1, sizeof(int64_t));
+  int overflow = 0;
+  int64_t tot = 0;
+#pragma omp parallel num_threads(T)
+  {
+    const int t = omp_get_thread_num();
+    const int64_t lo = N * t / T, hi = N * (t + 1) / T;
+    int64_t *mine = counts + (size_t)t * parts;
+    for (int64_t i = lo; i < hi; ++i) mine[parts == 1 ? 0 : (mix64((uint64_t)total[i]) >> shift)]++;
+#pragma omp barrier
+#pragma omp single
+    {
+      /* partition p holds the ids of thread 0's chunk first, then thread 1's, ...: index order */
+      int64_t run = 0;
+      for (int p = 0; p < parts; ++p) {
+        starts[p] = run;
+        for (int k = 0; k < T; ++k) {
+          const int64_t c = counts[(size_t)k * parts + p];
+          counts[(size_t)k * parts + p] = run;
+          run += c;
+        }
+      }
+      starts[parts] = run;
+      for (int p = 0; p < parts; ++p)
+        if ((uint64_t)(starts[p + 1] - starts[p]) * 2 > g->table_cap) overflow = 1; /* a very uneven deal */
+    }
+    if (!overflow) {
+      for (int64_t i = lo; i < hi; ++i)
+        g->items[mine[parts == 1 ? 0 : (mix64((uint64_t)total[i]) >> shift)]++] = (uint32_t)i;
+#pragma omp barrier
+      /* sweep the partitions (round-robin over the threads), each with its own table */
+      int64_t nfirst = 0;
+      for (int p = t; p < parts; p += T) {
+        uint64_t *kt = g->key + (size_t)p * g->table_cap;
+        uint32_t *vt = g->val + (size_t)p * g->table_cap;
+        const uint64_t mask = g->table_cap - 1;
+        for (int64_t e = starts[p]; e < starts[p + 1]; ++e) {
+          const uint32_t i = g->items[e];
+          const uint64_t key = (uint64_t)total[i];
+          uint64_t pos = (mix64(key) * 0x9E3779B97F4A7C15ull >> 20) & mask; /* independent of the partition bits */
+          while (kt[pos] != ~0ull && kt[pos] != key) pos = (pos + 1) & mask;
+          if (kt[pos] == ~0ull && key != ~0ull) {
+            kt[pos] = key;
+            vt[pos] = i;
+          }
+          g->first[i] = kt[pos] == key ? vt[pos] : i;
+          g->rank[e] = (uint32_t)pos; /* scratch until the ranks are written: the slot this element used */
+        }
+        /* leave the table empty: only the slots used (by remembered position: emptying while probing
+         * would cut the chains of the ids still to be found) */
+        for (int64_t e = starts[p]; e < starts[p + 1]; ++e) kt[g->rank[e]] = ~0ull;
+      }
+#pragma omp barrier
+      for (int64_t i = lo; i < hi; ++i) nfirst += g->first[i] == (uint32_t)i;
+      firsts[t + 1] = nfirst;
+#pragma omp barrier
+#pragma omp single
+      {
+        for (int k = 0; k < T; ++k) firsts[k + 1] += firsts[k];
+        tot = firsts[T];
+      }
+      int64_t r = firsts[t];
+      for (int64_t i = lo; i < hi; ++i) {
+        g->rank[i] = (uint32_t)r;
+        if (g->first[i] == (uint32_t)i) unique[r++] = total[i];
+      }
+#pragma omp barrier
+      for (int64_t i = lo; i < hi; ++i) labels[i] = (int64_t)g->rank[g->first[i]];
+    }
+  }
+  free(counts);
+  free(starts);
+  free(firsts);
+  if (overflow) return orc_relabel_sweep(total, N, unique, labels);
+  return tot;
 }
 
 /* ------------------------------------------------------------------ */

@@ -48,6 +48,8 @@ def lib():
         L.orc_relabel.argtypes = [_vp, _i64, _vp, _vp]
         L.orc_relabel_sweep.restype = _i64
         L.orc_relabel_sweep.argtypes = [_vp, _i64, _vp, _vp]
+        L.orc_relabel_parallel.restype = _i64
+        L.orc_relabel_parallel.argtypes = [_vp, _i64, _vp, _vp]
         L.orc_philox4x32_10.argtypes = [_vp, _vp, _vp]
         L.orc_sample_counts.restype = _i64
         L.orc_sample_counts.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _vp]
@@ -169,19 +171,21 @@ def relabel(tensors, algo="passes"):
     """tensor_relabel: src/tensor_relabel.cu:125-209. Returns (unique, [labels...])
     with the dtype torch.cat would give (int64 if any input is int64). algo: "passes"
     (the reference's four parallel passes over its low-bit hash table, OpenMP) or
-    "sweep" (one sequential sweep with a mixed hash: the plain CPU way, same results)."""
+    "sweep" (one sequential sweep with a mixed hash: the plain CPU way, same results) or
+    "parallel" (the tuned multi-core form: ids dealt to one partition per thread by their hash, every
+    thread sweeping its own; tables kept between calls)."""
     tensors = [_ids(t) for t in tensors]
     dt = np.result_type(*[t.dtype for t in tensors]) if tensors else np.int64
     total = _i64a(np.concatenate(tensors)) if tensors else np.zeros(0, np.int64)
     unique = np.empty(total.size, np.int64)
     labels = np.empty(total.size, np.int64)
-    fn = {"passes": lib().orc_relabel, "sweep": lib().orc_relabel_sweep}[algo]
+    fn = {"passes": lib().orc_relabel, "sweep": lib().orc_relabel_sweep, "parallel": lib().orc_relabel_parallel}[algo]
     u = fn(_p(total), total.size, _p(unique), _p(labels))
     out, off = [], 0
     for t in tensors:
-        out.append(labels[off:off + t.size].astype(dt))
+        out.append(labels[off:off + t.size].astype(dt, copy=False))
         off += t.size
-    return unique[:u].astype(dt), out
+    return unique[:u].astype(dt, copy=False), out
 
 
 def philox4x32_10(ctr, key):

@@ -113,7 +113,7 @@ def _relabel_closed_form(arrays):
     return list(first.keys()), [first[x] for x in total]
 
 
-@pytest.mark.parametrize("algo", ["passes", "sweep"])
+@pytest.mark.parametrize("algo", ["passes", "sweep", "parallel"])
 def test_relabel_reference_kat(oracle, algo):
     g = load_golden("relabel_kat.json")
     u, labels = oracle.relabel([np.array(x) for x in g["inputs"]], algo=algo)
@@ -121,7 +121,7 @@ def test_relabel_reference_kat(oracle, algo):
     assert [l.tolist() for l in labels] == g["labels"]
 
 
-@pytest.mark.parametrize("algo", ["passes", "sweep"])
+@pytest.mark.parametrize("algo", ["passes", "sweep", "parallel"])
 @pytest.mark.parametrize("n", [1, 2, 7, 8, 9, 255, 256, 257, 5000])
 def test_relabel_closed_form(oracle, n, algo):
     a = RNG.integers(0, max(2, n // 2), size=n)
@@ -130,6 +130,24 @@ def test_relabel_closed_form(oracle, n, algo):
     eu, el = _relabel_closed_form([a, b])
     assert u.tolist() == eu
     assert np.concatenate(labels).tolist() == el
+
+
+@pytest.mark.parametrize("ids", ["narrow", "wide", "negative"])
+@pytest.mark.parametrize("algo", ["parallel", "sweep"])
+def test_relabel_forms_that_keep_their_tables_on_repeated_calls(oracle, ids, algo):
+    """Both tuned forms keep their tables between calls and empty only the slots they used: calls of
+    different sizes one after the other, with ids that fit 32 bits, ids beyond and negative ids (not -1, the
+    reference's empty key, src/tensor_relabel.cu:141), must all equal the closed form."""
+    for n in (50_000, 300, 120_000, 7):
+        a = RNG.integers(0, max(2, n // 3), size=n)
+        if ids == "wide":
+            a = a + (1 << 40)
+        elif ids == "negative":
+            a = a - n // 6 - 2                      # some below -1, some above
+            a[a == -1] = -2
+        u, (labels,) = oracle.relabel([a], algo=algo)
+        eu, el = _relabel_closed_form([a])
+        assert u.tolist() == eu and labels.tolist() == el
 
 
 def test_relabel_mixed_dtypes_and_prefix(oracle):
