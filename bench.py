@@ -26,7 +26,7 @@ Benchmark configurations referred to by number in this file:
      f32 features in pinned host memory, top-degree 25 % cached; 4,096 seeds, fanouts [25,15,10],
      relabel, then fetch of all input nodes
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,scan,sampling,e2e]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workloads fetch,hashmap,scan,harness,sampling,e2e]
 """
 import argparse
 import collections
@@ -856,6 +856,142 @@ def bench_e2e(capi, args, result):
         "fetch_payload_GBs": round(tot_nodes * D * 4 / (t_f * 1e-3) / 1e9, 2)}
 
 
+# ---------------------------------------------------------------------------
+# the reference's own benchmark harnesses, shape for shape (they only print): per-call latency by the wall
+# clock, synchronised on both sides as time_recorder does there (example/test_cache_fetch.py:9-22)
+
+def wall_us(fn, reps):
+    """Median wall-clock microseconds of fn(), device idle before and after each call."""
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        ts.append((time.perf_counter() - t0) * 1e6)
+    ts.sort()
+    return round(ts[len(ts) // 2], 1)
+
+
+def bench_ref_harness(capi, args, result):
+    import torch
+    res = {}
+    g = torch.Generator().manual_seed(123)
+    sizes = [10, 100, 1000, 10_000, 100_000, 300_000, 1_000_000]
+
+    def reps_for(n):
+        return 200 if n <= 10_000 else 30
+
+    # example/test_cache_fetch.py:108-154: 1,000,000 x 128 f32, 90 % of the ids cached in random order
+    N, D = 1_000_000, 128
+    data = torch.randn(N, D, generator=g).pin_memory()
+    full_gpu = data.cuda()
+    ids = torch.randperm(N, generator=g)[: int(N * 0.9)].cuda()
+    cache = full_gpu[ids].contiguous()
+    hmap = capi.CUCOStaticHashmap(ids, torch.arange(ids.numel(), device="cuda"), 0.8)
+    fetch = {"map_layout": hmap.layout(), "by_queries": {}}
+    for n in sizes:
+        q = torch.randint(0, N, (n,), generator=g).cuda()
+        q_cpu = q.cpu()
+        a = capi.cache_fetch(data, cache, q, hmap)
+        assert torch.equal(a, full_gpu[q]) and torch.equal(a, capi.uva_fetch(data, q))
+        r = reps_for(n)
+        row = {"cache_fetch_us": wall_us(lambda: capi.cache_fetch(data, cache, q, hmap), r),
+               "uva_fetch_us": wall_us(lambda: capi.uva_fetch(data, q), r),
+               "mask_fetch_us": wall_us(lambda: capi.cache_fetch_with_mask(data, cache, q, hmap.query(q)), r),
+               "gpu_index_us": wall_us(lambda: full_gpu[q], r),
+               "gpu_index_select_us": wall_us(lambda: torch.index_select(full_gpu, 0, q), r)}
+        if not args.no_cpu:
+            row["cpu_fetch_us"] = wall_us(lambda: data[q_cpu].cuda(), 5 if n >= 100_000 else 30)
+        fetch["by_queries"][str(n)] = row
+    res["fetch_1M_x_128_f32_90pct_cached"] = fetch
+
+    # what a call costs the host (queued back to back, no synchronisation): the floor of the small-n rows
+    # above is one launch plus the synchronisation, and the operator's own share of it is this
+    def host_us(fn, n=2000):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        t = (time.perf_counter() - t0) / n * 1e6
+        torch.cuda.synchronize()
+        return round(t, 2)
+    q10 = torch.randint(0, N, (10,), generator=g).cuda()
+    res["host_cost_per_call_us_10_queries"] = {
+        "cache_fetch_pinned_table": host_us(lambda: capi.cache_fetch(data, cache, q10, hmap)),
+        "cache_fetch_device_table": host_us(lambda: capi.cache_fetch(full_gpu, cache, q10, hmap)),
+        "uva_fetch_pinned_table": host_us(lambda: capi.uva_fetch(data, q10)),
+        "hashmap_query": host_us(lambda: hmap.query(q10)),
+        "torch_index": host_us(lambda: full_gpu[q10]),
+        "torch_index_select": host_us(lambda: torch.index_select(full_gpu, 0, q10)),
+        "torch_empty_output_only": host_us(lambda: torch.empty((10, D), device="cuda"))}
+    del cache, hmap, ids
+
+    # example/test_cache_set.py:150-194: the same table, every id cached in random order
+    ids = torch.randperm(N, generator=g).cuda()
+    cache = full_gpu[ids].contiguous()
+    hmap = capi.CUCOStaticHashmap(ids, torch.arange(N, device="cuda"), 0.8)
+    sets = {"map_layout": hmap.layout(), "by_updates": {}}
+    for n in sizes:
+        idx = torch.randint(0, N, (n,), generator=g).cuda().unique()
+        upd = torch.randn(idx.numel(), D, generator=g).cuda()
+        r = reps_for(n)
+        row = {"rows": idx.numel(),
+               "cache_set_us": wall_us(lambda: capi.cache_set(data, cache, idx, upd, hmap), r),
+               "uva_set_us": wall_us(lambda: capi.uva_set(data, idx, upd), r),
+               "mask_set_us": wall_us(lambda: capi.cache_set_with_mask(data, cache, idx, upd, hmap.query(idx)), r),
+               "gpu_index_put_us": wall_us(lambda: full_gpu.index_put_((idx,), upd), r)}
+        assert torch.equal(capi.cache_fetch(data, cache, idx, hmap), upd)
+        sets["by_updates"][str(n)] = row
+    res["set_1M_x_128_f32_all_cached"] = sets
+    del cache, hmap, ids, full_gpu, data
+
+    # example/simple_bench.py:6-34: ~950,000 distinct int32 keys below 10,000,000, 1,000,000 int32 requests
+    keys = torch.randint(0, 10_000_000, (1_000_000,), generator=g).int().unique().cuda()
+    vals = torch.arange(keys.numel(), dtype=torch.int32, device="cuda")
+    req = torch.randint(0, 10_000_000, (1_000_000,), generator=g).int().cuda()
+    by_lf = {}
+    for lf in (0.1, 0.2, 0.3, 0.4, 0.5, 0.6, 0.7, 0.8, 0.9, 0.99, 1.0):
+        # (sorted keys with consecutive values would make the constructor choose its rank bitmap: the general
+        # table is timed beside the layout it picks)
+        row = {}
+        for layout in ("auto", "buckets"):
+            m = capi.CUCOStaticHashmap(keys, vals, lf, layout=layout)
+            row[layout] = {"layout": m.layout(), "query_us": wall_us(lambda: m.query(req), 50),
+                           "table_bytes": m.memory_usage()}
+            del m
+        by_lf[str(lf)] = row
+    res["hashmap_query_1M_int32_by_load_factor"] = by_lf
+    del keys, vals, req
+
+    # example/test_cache_sampling.py:167-221: 2,000,000 rows of degree U[0, 1000), int64 CSR, the top 30 % by
+    # degree cached, 5 picks without replacement; the reference times 50 calls per entry, here one call
+    if not args.harness_skip_sampling:
+        deg = torch.randint(0, 1000, (2_000_000,), generator=g)
+        indptr = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(deg, 0)])
+        nnz = int(indptr[-1])
+        indices = torch.empty(nnz, dtype=torch.int64, pin_memory=True)
+        torch.arange(nnz, out=indices)
+        indptr = indptr.pin_memory()
+        gpu_full_p, gpu_full_i = indptr.cuda(), indices.cuda()
+        hot = torch.sort(deg, descending=True).indices[: int(2_000_000 * 0.3)].cuda()
+        gp, gi = capi.create_subcsr(indptr, indices, hot)
+        hmap = capi.CUCOStaticHashmap(hot, torch.arange(hot.numel(), device="cuda"), 0.8)
+        samp = {"map_layout": hmap.layout(), "edges": nnz, "by_seeds": {}}
+        for n in [10, 100, 1000, 10_000, 100_000, 300_000, 500_000]:
+            seeds = torch.randperm(2_000_000, generator=g)[:n].cuda()
+            r = reps_for(n)
+            samp["by_seeds"][str(n)] = {
+                "gpu_us": wall_us(lambda: capi.csr_sampling(gpu_full_p, gpu_full_i, seeds, 5, False), r),
+                "uva_us": wall_us(lambda: capi.csr_sampling(indptr, indices, seeds, 5, False), r),
+                "cache_us": wall_us(lambda: capi.csr_cache_sampling(indptr, indices, gp, gi, hmap, seeds, 5, False), r)}
+        res["sampling_2M_rows_deg_u1000_k5_30pct_cached"] = samp
+    result["extra"]["ref_harness"] = res
+
+
 def probe_granularity(capi, args, result):
     """Random rows of 16/32/64/128 bytes from a 4 GiB HBM table: run under
     rocprofv3 --pmc FETCH_SIZE to see how many bytes one small random read costs."""
@@ -877,7 +1013,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workloads", default="fetch,hashmap,scan,sampling,e2e")
+    ap.add_argument("--workloads", default="fetch,hashmap,scan,harness,sampling,e2e")
+    ap.add_argument("--harness-skip-sampling", action="store_true",
+                    help="harness workload: leave out the 8 GB sampling graph of example/test_cache_sampling.py")
     ap.add_argument("--fetch-rows", type=int, default=100_000_000)
     ap.add_argument("--sampling-scale", type=int, default=21)
     ap.add_argument("--sampling-batches", type=int, default=50)
@@ -924,6 +1062,9 @@ def main():
         bench_scan(capi, args, result)
     if "granularity" in todo:
         probe_granularity(capi, args, result)
+    if "harness" in todo:
+        bench_ref_harness(capi, args, result)
+        torch.cuda.empty_cache()
     if "sampling" in todo:
         bench_sampling(capi, args, result)
         s = result["extra"]["sampling_config3"]
