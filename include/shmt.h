@@ -248,6 +248,32 @@ int shmt_exclusive_scan(void *data, int64_t len, int elem_bytes, void *tmp,
                         int64_t tmp_bytes, void *stream);
 int shmt_inclusive_scan_i32(void *data, int64_t len, void *tmp,
                             int64_t tmp_bytes, void *stream);
+/* The same two scans on a workspace that is KEPT clean. The scans above take
+ * any memory for `tmp` and clear it first, one short launch per call (cub's
+ * temporary storage, src/tensor_relabel.cu:15-25, likewise needs no
+ * preparation). A workspace that is all zero when a scan starts is all zero
+ * again when it ends (the last workgroup to finish clears what the scan
+ * used), so a caller that clears its workspace once (shmt_scan_workspace_clear,
+ * or any memset) and then hands it to nothing but these scans, one at a
+ * time, saves that launch on every call. kept_tmp: at least
+ * shmt_scan_tmp_bytes(len) bytes, 8-byte aligned.                           */
+int shmt_scan_workspace_clear(void *tmp, int64_t tmp_bytes, void *stream);
+int shmt_exclusive_scan_kept(void *data, int64_t len, int elem_bytes,
+                             void *kept_tmp, int64_t tmp_bytes, void *stream);
+int shmt_inclusive_scan_i32_kept(void *data, int64_t len, void *kept_tmp,
+                                 int64_t tmp_bytes, void *stream);
+/* Bounded waits. A tile of a device-wide scan waits for the sums of the
+ * tiles before it; that wait is bounded, and a tile that gives up leaves its
+ * part of the array as it was, publishes nothing and sets a bit in an error
+ * word of the current GPU (no counterpart in the reference, whose kernels
+ * have no such waits). shmt_async_error waits for the GPU's queued work,
+ * stores the word in *code_out (0: no kernel gave up; bit 0: a scan's
+ * look-back) and clears it; when it is not 0, shmt_last_error() says what
+ * gave up.                                                                  */
+int shmt_async_error(int *code_out);
+/* Sets bits of that word from the host, as a kernel that gave up would: for
+ * tests of the error path (no kernel has to starve for them).               */
+int shmt_async_error_inject(int bits);
 /* shmt_exclusive_scan without a workspace argument, and without any
  * allocation inside the call. It has no counterpart in the reference (whose
  * cub_exclusiveSum allocates its temporary storage on every call,

@@ -196,6 +196,21 @@ void cache_set_with_mask(torch::Tensor uva_data, torch::Tensor gpu_data, torch::
 
 // ---- scan --------------------------------------------------------------------
 
+// Scan workspace that is kept clean: one per device and stream, all zero when it is made; every scan
+// leaves it all zero again, so no scan has to clear it first (shmt_*_scan_kept). Scans of one stream run
+// one after the other, which is all the sharing such a workspace allows.
+torch::Tensor kept_scan_workspace(int64_t bytes) {
+  static std::mutex mutex;
+  static std::unordered_map<uint64_t, torch::Tensor> kept;
+  const auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+  const uint64_t key = (static_cast<uint64_t>(stream.device_index()) << 48) ^ static_cast<uint64_t>(stream.id());
+  std::lock_guard<std::mutex> lock(mutex);
+  torch::Tensor &w = kept[key];
+  if (!w.defined() || w.numel() < bytes)
+    w = torch::zeros({std::max<int64_t>(bytes, 1 << 16)}, torch::TensorOptions().dtype(torch::kUInt8).device(torch::kCUDA));
+  return w;
+}
+
 // thrust_scan, src/thrust_scan.cu:9-18: in-place inclusive sum over int32.
 void thrust_scan(torch::Tensor tensor) {
   TORCH_CHECK(tensor.scalar_type() == torch::kInt32, "thrust_scan expects an int32 tensor");
@@ -203,9 +218,18 @@ void thrust_scan(torch::Tensor tensor) {
   const int64_t n = tensor.numel();
   if (n == 0) return;
   const int64_t tmp_bytes = shmt_scan_tmp_bytes(n);
-  torch::Tensor tmp = device_bytes(tmp_bytes);
-  check(shmt_inclusive_scan_i32(device_address(tensor, "tensor"), n, tmp.data_ptr(), tmp_bytes,
-                                current_stream()));
+  torch::Tensor tmp = tmp_bytes > 0 ? kept_scan_workspace(tmp_bytes) : torch::Tensor();
+  check(shmt_inclusive_scan_i32_kept(device_address(tensor, "tensor"), n, tmp_bytes > 0 ? tmp.data_ptr() : nullptr,
+                                     tmp_bytes, current_stream()));
+}
+
+// What shmt_async_error reports as an exception (nothing when no kernel gave up a bounded wait).
+// Synchronises the device; meant for the end of a job, for tests, and for the slow path of a size
+// read-back that did not arrive.
+void raise_async_error() {
+  int code = 0;
+  check(shmt_async_error(&code));
+  TORCH_CHECK(code == 0, shmt_last_error());
 }
 
 // ---- sampling ------------------------------------------------------------------
@@ -400,6 +424,9 @@ PYBIND11_MODULE(ShmTensorLib, m) {
 
   m.def("thrust_scan", &thrust_scan, py::arg("tensor"));
 
+  m.def("raise_async_error", &raise_async_error,
+        "Raises RuntimeError if a kernel of this library gave up a bounded wait for another workgroup since the "
+        "last call (a device-wide scan whose look-back starved); synchronises the device.");
   m.def("set_host_register", &set_host_register, py::arg("enabled"),
         "Let pin_memory() try to register existing memory in place (hipHostRegister) before it falls "
         "back to re-homing the tensor's storage in new pinned memory. Off by default; also switched on "

@@ -114,7 +114,11 @@ class Readback {
     }
     sync_current_stream();
     const int64_t v = *s.host;
-    TORCH_CHECK(v != kPending, "the GPU did not report a result size (kernel failed?)");
+    if (v == kPending) {
+      int gave_up = 0;  // a kernel that gave up a bounded wait says so in the GPU's error word
+      const bool known = shmt_async_error(&gave_up) == SHMT_OK && gave_up != 0;
+      TORCH_CHECK(false, known ? shmt_last_error() : "the GPU did not report a result size (kernel failed?)");
+    }
     return v;
   }
 

@@ -78,6 +78,13 @@ int launch_scan_partials(uint64_t *partials, int64_t nb, hipStream_t s) {
 // took 64 us.
 constexpr uint32_t kPublished = 1;
 constexpr uint32_t kLookbackSpinLimit = 1u << 24;  // a wait that long means a tile before this one died
+constexpr uint32_t kErrScanWait = 1;               // bit of the error word: a look-back gave up
+
+// Sticky error word of the library, one copy per GPU (part of the loaded code
+// object, like the static scan workspace below): a kernel that gives up a
+// bounded wait sets a bit here instead of finishing with a wrong result in
+// silence. shmt_async_error() reads and clears it.
+static __device__ uint32_t async_error_word;
 constexpr int kLbBlock = 1024;                 // threads per tile
 constexpr int kLbWaves = kLbBlock / kWave;
 constexpr int kLbChunks = 8;                   // 16-byte vectors per lane
@@ -87,7 +94,9 @@ constexpr int kLbFan = kWave;                  // tiles per group, groups per ru
 constexpr int64_t kScanHeaderBytes = 64;  // tile counter (+ padding) in front of the published sums
 
 struct ScanState {
-  unsigned long long *counter;  // next tile number to hand out
+  unsigned long long *counter;  // next tile number to hand out; counter[1]: workgroups that are done
+  uint32_t *error;              // the GPU's error word
+  int64_t words;                // 64-bit words of the workspace behind the header (tiles, groups, runs)
   uint64_t *tiles;              // 2 words per tile
   uint64_t *groups;             // 2 words per group of 64 tiles
   uint64_t *runs;               // 2 words per run of 64 groups
@@ -132,28 +141,50 @@ __device__ __forceinline__ uint64_t wave_sum_all(uint64_t v) { return wave_last(
 // that end with this tile. A tile only waits for entries that tiles with
 // smaller numbers publish, which were handed out earlier to workgroups that
 // are already running, so the waiting ends.
-__device__ __forceinline__ uint64_t tile_lookback(const ScanState &st, int64_t tile, uint64_t own) {
+__device__ __forceinline__ uint64_t tile_lookback(const ScanState &st, int64_t tile, uint64_t own, bool *gave_up) {
   const int lane = lane_id();
   const int64_t group = tile / kLbFan, run = group / kLbFan;
   const int in_group = static_cast<int>(tile % kLbFan), in_run = static_cast<int>(group % kLbFan);
+  // A wait ends without its value when it has spun for kLookbackSpinLimit rounds, or as soon as any tile
+  // of this GPU has reported such a wait (checked every 256 rounds): the tiles behind a lost one would
+  // otherwise each sit out the full limit, one after the other.
+  auto hopeless = [&](uint32_t spins) {
+    return spins >= kLookbackSpinLimit ||
+           ((spins & 255u) == 255u && __hip_atomic_load(st.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
+  };
   // runs before this tile's run: at most 64 up to 262,144 tiles, in further steps of 64 beyond
   uint64_t far = 0;
   uint32_t spins = 0;
+  bool lost = false;
   for (int64_t first = kWave; first < run; first += kWave) {
     uint64_t part = 0;
-    while (!sum_read(st.runs, first + lane, first + lane < run, &part) && ++spins < kLookbackSpinLimit)
+    bool ok = false;
+    for (;;) {
+      if (!ok) ok = sum_read(st.runs, first + lane, first + lane < run, &part);
+      if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+      if (hopeless(++spins)) {
+        lost = true;
+        break;
+      }
       __builtin_amdgcn_s_sleep(8);
+    }
     far += part;
   }
   // a lane asks again only for what it has not seen published yet
   uint64_t a = 0, b = 0, c = 0;
   bool ok_a = false, ok_b = false, ok_c = false;
-  for (;;) {
+  while (!lost) {
     if (!ok_a) ok_a = sum_read(st.tiles, group * kLbFan + lane, lane < in_group, &a);
     if (!ok_b) ok_b = sum_read(st.groups, run * kLbFan + lane, lane < in_run, &b);
     if (!ok_c) ok_c = sum_read(st.runs, lane, lane < run, &c);
-    if (__builtin_amdgcn_ballot_w64(!(ok_a && ok_b && ok_c)) == 0 || ++spins >= kLookbackSpinLimit) break;
-    __builtin_amdgcn_s_sleep(8);
+    if (__builtin_amdgcn_ballot_w64(!(ok_a && ok_b && ok_c)) == 0) break;
+    if (hopeless(++spins)) lost = true;
+    else __builtin_amdgcn_s_sleep(8);
+  }
+  if (lost) {  // report, publish nothing: the tile is left as it was and so is everything behind it
+    if (lane == 0) __hip_atomic_fetch_or(st.error, kErrScanWait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *gave_up = true;
+    return 0;
   }
   c += far;
   const uint64_t tiles_before = wave_sum_all(a), groups_before = wave_sum_all(b), runs_before = wave_sum_all(c);
@@ -207,10 +238,16 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
   __shared__ uint64_t wave_total[kLbWaves];
   __shared__ uint64_t shared_before;  // the sum of everything before the tile
   __shared__ uint64_t shared_tile;    // the workgroup's next tile number
+  __shared__ int shared_lost;         // the look-back of this tile gave up: leave the tile as it is
+  __shared__ int shared_last;         // this workgroup is the last one to finish its look-backs
   const int wave = threadIdx.x / kWave, lane = lane_id();
   const int64_t lane_off = static_cast<int64_t>(wave) * kLbChunks * kWave * V + lane * V;
   T v[kLbChunks][V];
-  if (threadIdx.x == 0) shared_tile = atomicAdd(st.counter, 1ull);
+  if (threadIdx.x == 0) {
+    shared_tile = atomicAdd(st.counter, 1ull);
+    // a workgroup that comes too late for any tile is done with its look-backs at once
+    shared_last = shared_tile >= static_cast<uint64_t>(nb) && atomicAdd(st.counter + 1, 1ull) == gridDim.x - 1;
+  }
   __syncthreads();
   int64_t tile = static_cast<int64_t>(shared_tile);
   if (tile < nb) scan_tile_load<T, kLbChunks>(data, len, tile * kTileElems + lane_off, (tile + 1) * kTileElems <= len, v);
@@ -244,6 +281,7 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
     }
     if (threadIdx.x < kWave) {  // the first wave talks to the other tiles
       uint64_t before = 0;
+      bool lost = false;
       if (tile == 0) {
         T run = 0;
         if (threadIdx.x == 0) {
@@ -257,11 +295,16 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
         if (threadIdx.x == 0) sum_publish(st.tiles, 0, before + total);
       } else {
         if (threadIdx.x == 0) sum_publish(st.tiles, tile, total);
-        before = tile_lookback(st, tile, total);
+        before = tile_lookback(st, tile, total, &lost);
       }
       if (threadIdx.x == 0) {
         shared_before = before;
         shared_tile = next_ticket;
+        shared_lost = lost;
+        // no tile left for this workgroup: its look-backs are over; the last workgroup to say so
+        // clears the workspace (below), when nobody reads the published words any more
+        if (next_ticket >= static_cast<unsigned long long>(nb))
+          shared_last = atomicAdd(st.counter + 1, 1ull) == gridDim.x - 1;
       }
     }
     __syncthreads();
@@ -269,6 +312,7 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
     const int64_t next = static_cast<int64_t>(shared_tile);
 #pragma unroll
     for (int c = 0; c < kLbChunks; ++c) {
+      if (shared_lost) break;
       const int64_t i = lane_base + static_cast<int64_t>(c) * kWave * V;
       T run = static_cast<T>(base) + excl[c];
       ScanVec<T> out;
@@ -289,6 +333,15 @@ __global__ __launch_bounds__(kLbBlock) void scan_lookback_kernel(T *head, int n_
     if (next < nb) scan_tile_load<T, kLbChunks>(data, len, next * kTileElems + lane_off, (next + 1) * kTileElems <= len, v);
     tile = next;
   }  // the barriers above also order the reuse of the LDS words by the next tile
+  // The workgroup that ends its look-backs last leaves the workspace as it found it, all zero: counter,
+  // done count and every published word. A workspace that starts clean therefore stays clean from scan to
+  // scan and needs no clearing launch in front of the next one (also when this launch is replayed from a
+  // graph). shared_last was written before the last barrier above.
+  if (shared_last) {
+    uint64_t *const words = reinterpret_cast<uint64_t *>(st.counter) + kScanHeaderBytes / 8;
+    for (int64_t i = threadIdx.x; i < st.words; i += kLbBlock) words[i] = 0;
+    if (threadIdx.x < 2) st.counter[threadIdx.x] = 0;
+  }
 }
 
 template <typename T, bool INCLUSIVE>
@@ -320,8 +373,30 @@ static int resident_workgroups(const void *kernel, int *out) {
   return SHMT_OK;
 }
 
+// Device address of this GPU's error word (looked up once per device).
+constexpr int kMaxDevices = 64;
+static std::mutex g_symbol_mutex;
+static uint32_t *g_error_ptr[kMaxDevices];
+
+static int error_word(uint32_t **out) {
+  int dev = -1;
+  SHMT_HIP(hipGetDevice(&dev));
+  SHMT_REQUIRE(dev >= 0 && dev < kMaxDevices, "scan: device ordinal %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_symbol_mutex);
+  if (g_error_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    SHMT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(async_error_word)));
+    SHMT_REQUIRE(p != nullptr, "scan: no device address for the error word");
+    g_error_ptr[dev] = static_cast<uint32_t *>(p);
+  }
+  *out = g_error_ptr[dev];
+  return SHMT_OK;
+}
+
+// kept: the workspace is all zero (it was cleared once and has only been used by scans since, each of
+// which leaves it all zero); otherwise it is cleared first.
 template <typename T, bool INCLUSIVE>
-static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, hipStream_t s) {
+static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, bool kept, hipStream_t s) {
   if (len <= kSingleBlockMax) {
     hipLaunchKernelGGL((scan_single_kernel<T, INCLUSIVE>), dim3(1), dim3(1024), 0, s, data, len);
     SHMT_LAUNCH_CHECK();
@@ -346,15 +421,20 @@ static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, hipS
   SHMT_REQUIRE((reinterpret_cast<uintptr_t>(tmp) & 7) == 0, "scan: tmp must be 8-byte aligned");
   ScanState st;
   st.counter = static_cast<unsigned long long *>(tmp);
+  int rc = error_word(&st.error);
+  if (rc) return rc;
+  st.words = (need - kScanHeaderBytes) / 8;
   st.tiles = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.tiles_off);
   st.groups = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.groups_off);
   st.runs = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.runs_off);
-  // counter and words start at zero (a kernel, not a memset, so that the scan can be captured in a graph)
-  hipLaunchKernelGGL(scan_state_clear_kernel, dim3(grid_for(need / 8, 256 * 4)), dim3(256), 0, s,
-                     static_cast<uint64_t *>(tmp), need / 8);
-  SHMT_LAUNCH_CHECK();
+  if (!kept) {
+    // counter and words start at zero (a kernel, not a memset, so that the scan can be captured in a graph)
+    hipLaunchKernelGGL(scan_state_clear_kernel, dim3(grid_for(need / 8, 256 * 4)), dim3(256), 0, s,
+                       static_cast<uint64_t *>(tmp), need / 8);
+    SHMT_LAUNCH_CHECK();
+  }
   int resident = 0;
-  int rc = resident_workgroups(reinterpret_cast<const void *>(&scan_lookback_kernel<T, INCLUSIVE>), &resident);
+  rc = resident_workgroups(reinterpret_cast<const void *>(&scan_lookback_kernel<T, INCLUSIVE>), &resident);
   if (rc) return rc;
   const unsigned grid = static_cast<unsigned>(nb < resident ? nb : resident);
   hipLaunchKernelGGL((scan_lookback_kernel<T, INCLUSIVE>), dim3(grid), dim3(kLbBlock), 0, s,
@@ -377,8 +457,6 @@ constexpr int64_t kStaticScanWords =  // header + 256 KiB of tile words + 4 KiB 
     kScanHeaderBytes / 8 + 2 * (kStaticScanTiles + kStaticScanGroups + kStaticScanRuns);
 static __device__ __align__(256) uint64_t scratch[kStaticScanWords];
 
-constexpr int kMaxDevices = 64;
-static std::mutex g_scratch_mutex;
 static uint64_t *g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device ordinal
 
 // Device address of this GPU's copy of `scratch` (looked up once per device).
@@ -386,7 +464,7 @@ static int static_scan_scratch(uint64_t **out) {
   int dev = -1;
   SHMT_HIP(hipGetDevice(&dev));
   SHMT_REQUIRE(dev >= 0 && dev < kMaxDevices, "shmt_exclusive_scan_noalloc: device ordinal %d not supported", dev);
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  std::lock_guard<std::mutex> lock(g_symbol_mutex);
   if (g_scratch_ptr[dev] == nullptr) {
     void *p = nullptr;
     SHMT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
@@ -409,17 +487,36 @@ int64_t shmt_scan_tmp_bytes(int64_t len) {
   return scan_tmp_layout((len + tile_elems - 1) / tile_elems).total;
 }
 
+static int exclusive_scan(const char *who, void *data, int64_t len, int elem_bytes, void *tmp, int64_t tmp_bytes,
+                          bool kept, void *stream) {
+  SHMT_REQUIRE(len >= 0, "%s: len must be >= 0", who);
+  SHMT_REQUIRE(width_ok(elem_bytes), "%s: ID can only be int32 or int64", who);
+  if (len == 0) return SHMT_OK;
+  SHMT_REQUIRE(data != nullptr, "%s: data is null", who);
+  if (elem_bytes == 8)
+    return scan_inplace<uint64_t, false>(static_cast<uint64_t *>(data), len, tmp, tmp_bytes, kept, as_stream(stream));
+  return scan_inplace<uint32_t, false>(static_cast<uint32_t *>(data), len, tmp, tmp_bytes, kept, as_stream(stream));
+}
+
 int shmt_exclusive_scan(void *data, int64_t len, int elem_bytes, void *tmp, int64_t tmp_bytes,
                         void *stream) {
-  SHMT_REQUIRE(len >= 0, "shmt_exclusive_scan: len must be >= 0");
-  SHMT_REQUIRE(width_ok(elem_bytes), "shmt_exclusive_scan: ID can only be int32 or int64");
-  if (len == 0) return SHMT_OK;
-  SHMT_REQUIRE(data != nullptr, "shmt_exclusive_scan: data is null");
-  if (elem_bytes == 8)
-    return scan_inplace<uint64_t, false>(static_cast<uint64_t *>(data), len, tmp, tmp_bytes,
-                                         as_stream(stream));
-  return scan_inplace<uint32_t, false>(static_cast<uint32_t *>(data), len, tmp, tmp_bytes,
-                                       as_stream(stream));
+  return exclusive_scan("shmt_exclusive_scan", data, len, elem_bytes, tmp, tmp_bytes, false, stream);
+}
+
+int shmt_exclusive_scan_kept(void *data, int64_t len, int elem_bytes, void *kept_tmp, int64_t tmp_bytes,
+                             void *stream) {
+  return exclusive_scan("shmt_exclusive_scan_kept", data, len, elem_bytes, kept_tmp, tmp_bytes, true, stream);
+}
+
+int shmt_scan_workspace_clear(void *tmp, int64_t tmp_bytes, void *stream) {
+  SHMT_REQUIRE(tmp_bytes >= 0 && (tmp_bytes & 7) == 0, "shmt_scan_workspace_clear: tmp_bytes must be a multiple of 8");
+  if (tmp_bytes == 0) return SHMT_OK;
+  SHMT_REQUIRE(tmp != nullptr && (reinterpret_cast<uintptr_t>(tmp) & 7) == 0,
+               "shmt_scan_workspace_clear: tmp must be 8-byte aligned");
+  hipLaunchKernelGGL(scan_state_clear_kernel, dim3(grid_for(tmp_bytes / 8, 256 * 4)), dim3(256), 0, as_stream(stream),
+                     static_cast<uint64_t *>(tmp), tmp_bytes / 8);
+  SHMT_LAUNCH_CHECK();
+  return SHMT_OK;
 }
 
 int shmt_exclusive_scan_noalloc(void *data, int64_t len, int elem_bytes, void *stream) {
@@ -434,23 +531,59 @@ int shmt_exclusive_scan_noalloc(void *data, int64_t len, int elem_bytes, void *s
   uint64_t *partials = nullptr;
   int rc = static_scan_scratch(&partials);
   if (rc) return rc;
+  uint32_t *err = nullptr;
+  rc = error_word(&err);
+  if (rc) return rc;
   if (len == 0) return SHMT_OK;
-  // The workspace keeps what the last call left in it; every call clears the
-  // words it is going to use before it scans.
+  // The workspace is zero when the library is loaded and every scan leaves it zero again, so no call
+  // has anything to clear (calls that overlap on one GPU share the array and race).
   const int64_t tmp_bytes = kStaticScanWords * static_cast<int64_t>(sizeof(uint64_t));
-  if (elem_bytes == 8)
-    return scan_inplace<uint64_t, false>(static_cast<uint64_t *>(data), len, partials, tmp_bytes,
-                                         as_stream(stream));
-  return scan_inplace<uint32_t, false>(static_cast<uint32_t *>(data), len, partials, tmp_bytes,
-                                       as_stream(stream));
+  return exclusive_scan("shmt_exclusive_scan_noalloc", data, len, elem_bytes, partials, tmp_bytes, true, stream);
 }
 
 int shmt_inclusive_scan_i32(void *data, int64_t len, void *tmp, int64_t tmp_bytes, void *stream) {
   SHMT_REQUIRE(len >= 0, "shmt_inclusive_scan_i32: len must be >= 0");
   if (len == 0) return SHMT_OK;
   SHMT_REQUIRE(data != nullptr, "shmt_inclusive_scan_i32: data is null");
-  return scan_inplace<uint32_t, true>(static_cast<uint32_t *>(data), len, tmp, tmp_bytes,
+  return scan_inplace<uint32_t, true>(static_cast<uint32_t *>(data), len, tmp, tmp_bytes, false,
                                       as_stream(stream));
+}
+
+int shmt_inclusive_scan_i32_kept(void *data, int64_t len, void *kept_tmp, int64_t tmp_bytes, void *stream) {
+  SHMT_REQUIRE(len >= 0, "shmt_inclusive_scan_i32_kept: len must be >= 0");
+  if (len == 0) return SHMT_OK;
+  SHMT_REQUIRE(data != nullptr, "shmt_inclusive_scan_i32_kept: data is null");
+  return scan_inplace<uint32_t, true>(static_cast<uint32_t *>(data), len, kept_tmp, tmp_bytes, true,
+                                      as_stream(stream));
+}
+
+int shmt_async_error(int *code_out) {
+  SHMT_REQUIRE(code_out != nullptr, "shmt_async_error: code_out is null");
+  *code_out = 0;
+  uint32_t *err = nullptr;
+  int rc = error_word(&err);
+  if (rc) return rc;
+  uint32_t seen = 0;
+  SHMT_HIP(hipMemcpy(&seen, err, sizeof(seen), hipMemcpyDeviceToHost));  // waits for the device's queued work
+  if (seen != 0) {
+    const uint32_t zero = 0;
+    SHMT_HIP(hipMemcpy(err, &zero, sizeof(zero), hipMemcpyHostToDevice));
+    set_error("a kernel gave up a bounded wait for another workgroup (error bits 0x%x): %s", seen,
+              (seen & kErrScanWait) ? "the look-back of a device-wide scan; the scanned array is incomplete" : "unknown");
+  }
+  *code_out = static_cast<int>(seen);
+  return SHMT_OK;
+}
+
+int shmt_async_error_inject(int bits) {
+  uint32_t *err = nullptr;
+  int rc = error_word(&err);
+  if (rc) return rc;
+  uint32_t seen = 0;
+  SHMT_HIP(hipMemcpy(&seen, err, sizeof(seen), hipMemcpyDeviceToHost));
+  seen |= static_cast<uint32_t>(bits);
+  SHMT_HIP(hipMemcpy(err, &seen, sizeof(seen), hipMemcpyHostToDevice));
+  return SHMT_OK;
 }
 
 }  // extern "C"

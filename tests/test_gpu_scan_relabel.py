@@ -312,3 +312,49 @@ def test_relabel_beyond_2_31_ids(capi):
         assert torch.equal(labels[lo:hi], torch.arange(lo, hi, device="cuda") % m), lo
     del total, unique, labels
     torch.cuda.empty_cache()
+
+
+def test_kept_workspace_scans_need_no_clearing_and_stay_clean(cabi, oracle):
+    """A workspace that is all zero once stays all zero from scan to scan (the last workgroup clears what the
+    scan used), so shmt_*_scan_kept runs without the clearing launch: several scans of different lengths and
+    widths on one workspace, each against the oracle, and the workspace read back as zeros in between."""
+    lib = cabi.load()
+    sizes = [3_000_017, 70_001, 1 << 24, 200_000]
+    tmp_bytes = max(lib.shmt_scan_tmp_bytes(n) for n in sizes)
+    tmp = torch.full((tmp_bytes,), 0x5A, dtype=torch.uint8).cuda()          # dirty on purpose ...
+    cabi.check(lib.shmt_scan_workspace_clear(tmp.data_ptr(), tmp_bytes, cabi.current_stream()))   # ... cleared once
+    rng = np.random.default_rng(5)
+    for n in sizes:
+        a64 = rng.integers(-2**40, 2**40, size=n)
+        d = torch.from_numpy(a64).cuda()
+        cabi.check(lib.shmt_exclusive_scan_kept(d.data_ptr(), n, 8, tmp.data_ptr(), tmp_bytes, cabi.current_stream()))
+        assert np.array_equal(d.cpu().numpy(), oracle.exclusive_scan(a64))
+        assert int(tmp.count_nonzero()) == 0
+        a32 = rng.integers(-1000, 1000, size=n).astype(np.int32)
+        d = torch.from_numpy(a32).cuda()
+        cabi.check(lib.shmt_inclusive_scan_i32_kept(d.data_ptr(), n, tmp.data_ptr(), tmp_bytes, cabi.current_stream()))
+        assert np.array_equal(d.cpu().numpy(), np.cumsum(a32, dtype=np.int32))
+        assert int(tmp.count_nonzero()) == 0
+    # too small a workspace is an argument error
+    assert lib.shmt_exclusive_scan_kept(d.data_ptr(), 1 << 24, 8, tmp.data_ptr(), 64, cabi.current_stream()) != 0
+
+
+def test_a_wait_that_gave_up_is_reported(capi, cabi):
+    """A scan tile whose look-back gives up sets a bit in the GPU's error word instead of finishing with a wrong
+    result in silence. The word is set from the host here (no kernel has to starve): shmt_async_error returns
+    and clears it, the shim turns it into a RuntimeError that names the scan."""
+    import ctypes
+    lib = cabi.load()
+    code = ctypes.c_int(-1)
+    cabi.check(lib.shmt_async_error(ctypes.byref(code)))
+    assert code.value == 0
+    capi.raise_async_error()                                    # nothing to report
+    cabi.check(lib.shmt_async_error_inject(1))
+    with pytest.raises(RuntimeError, match="look-back of a device-wide scan"):
+        capi.raise_async_error()
+    capi.raise_async_error()                                    # reading it cleared it
+    cabi.check(lib.shmt_async_error_inject(1))
+    cabi.check(lib.shmt_async_error(ctypes.byref(code)))
+    assert code.value == 1 and b"gave up a bounded wait" in lib.shmt_last_error()
+    cabi.check(lib.shmt_async_error(ctypes.byref(code)))
+    assert code.value == 0

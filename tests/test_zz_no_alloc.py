@@ -29,9 +29,14 @@ def _both(cabi, a, bytes_):
                                        cabi.current_stream()))
     no_alloc = torch.from_numpy(a.copy()).cuda()
     torch.cuda.synchronize()
+    # nothing allocated: neither through torch's caching allocator nor behind its back (the driver's own
+    # count of free device memory, which a hipMalloc inside the library would lower)
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info()[0]
     cabi.check(lib.shmt_exclusive_scan_noalloc(no_alloc.data_ptr(), n, bytes_, cabi.current_stream()))
+    torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return with_ws.cpu().numpy(), no_alloc.cpu().numpy()
 
 
@@ -42,7 +47,7 @@ def test_no_alloc_scan_equals_workspace_scan_twice_in_a_row(cabi, oracle):
     cabi.check(lib.shmt_exclusive_scan_noalloc(None, 0, 8, cabi.current_stream()))
     rng = np.random.default_rng(11)
     # first call: 5,000,001 int64 (306 tiles of 16,384 elements); second, smaller: 300,001 int32 (10 tiles of
-    # 32,768), which finds the first call's tile words in the workspace; third: one workgroup, no workspace use
+    # 32,768), on the workspace the first call used and left clean; third: one workgroup, no workspace use
     for n, dt in ((5_000_001, np.int64), (300_001, np.int32), (4_097, np.int64)):
         hi = 2**61 if dt is np.int64 else 2**30                  # sums wrap around
         a = rng.integers(0, hi, size=n).astype(dt)
