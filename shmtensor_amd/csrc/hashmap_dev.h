@@ -71,18 +71,74 @@ __device__ __forceinline__ int64_t map_key(const MapView &m, int64_t req) {
   return req;
 }
 
-// Lookup in a flat map (kind != kKindBuckets); every lane for itself. STREAM:
-// the entry of a direct table is read with a non-temporal load (see
-// half_wave_find for when a row fetch asks for that).
+// Table entries that will not be looked at again soon (the probe of a row
+// fetch) are read with the non-temporal cache policy, so that they do not push
+// table rows out of the caches. They go through buffer loads, whose cache
+// policy is an operand of the instruction: the same hint as metadata on an
+// ordinary load is dropped whenever the optimiser merges the load with its
+// plain twin on the other side of a branch. Buffer loads address with 32-bit
+// byte offsets, so a table must stay below 4 GiB to be read this way
+// (streamable()); larger ones are read with plain loads.
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kCachePolicyNonTemporal = 2;  // gfx94x / gfx950: bit 1 of the cache-policy operand
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t table_resource(const void *table) {
+  // raw buffer over [table, table + 4 GiB): no stride, no swizzle; word 3 as gfx90a .. gfx950 want it for
+  // untyped 32-bit data
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(table), 0, -1, 0x00020000);
+}
+
+__device__ __forceinline__ bool streamable(const MapView &m) {
+  if (m.kind == kKindBuckets) return m.nbuckets < (1u << 25);  // 128-byte buckets
+  if (m.kind == kKindDirect) return m.span < (1ll << 30);      // 4-byte entries
+  return false;
+}
+
+__device__ __forceinline__ uint4 load_bucket_streaming(const MapView &m, uint32_t bucket, int sub) {
+  const uint32_t offset = (bucket * kProbeGroup + static_cast<uint32_t>(sub)) * 16u;
+  const probe_u32x4 v =
+      __builtin_amdgcn_raw_buffer_load_b128(table_resource(m.buckets), offset, 0, kCachePolicyNonTemporal);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// Lookup in a flat map (kind != kKindBuckets); every lane for itself, in two
+// steps so that a caller can put other work between the load and its use:
+// flat_issue starts the one load a rank or direct map needs, flat_finish turns
+// what came back into the value. STREAM: the entry of a direct table is read
+// with a non-temporal load (see half_wave_issue for when a row fetch asks for
+// that).
+struct FlatPending {
+  uint4 block;     // rank form: the 16-byte block of the key
+  int32_t direct;  // direct form: the table entry
+  bool inside;     // the key lies in [lo, lo + span)
+};
+
 template <bool STREAM = false>
-__device__ __forceinline__ int64_t flat_find(const MapView &m, int64_t key) {
+__device__ __forceinline__ FlatPending flat_issue(const MapView &m, int64_t key) {
+  FlatPending p;
+  p.block = make_uint4(0, 0, 0, 0);
+  p.direct = -1;
   const uint64_t off = static_cast<uint64_t>(key) - static_cast<uint64_t>(m.lo);  // key < lo wraps around
-  if (off >= static_cast<uint64_t>(m.span)) return -1;
+  p.inside = off < static_cast<uint64_t>(m.span);
+  if (!p.inside || m.kind == kKindRange) return p;
+  if (m.kind == kKindRank) {
+    p.block = m.buckets[off / kRankIdsPerBlock];  // x: keys below this block; y, z, w: presence of ids 0-31, 32-63, 64-95
+  } else {
+    const int32_t *direct = reinterpret_cast<const int32_t *>(m.buckets);
+    p.direct = STREAM ? static_cast<int32_t>(__builtin_amdgcn_raw_buffer_load_b32(
+                            table_resource(m.buckets), static_cast<uint32_t>(off) * 4u, 0, kCachePolicyNonTemporal))
+                      : direct[off];
+  }
+  return p;
+}
+
+__device__ __forceinline__ int64_t flat_finish(const MapView &m, int64_t key, const FlatPending &p) {
+  if (!p.inside) return -1;
   if (m.kind == kKindRange) return key + m.delta;
   if (m.kind == kKindRank) {
-    const uint64_t blk = off / kRankIdsPerBlock;
-    const uint32_t r = static_cast<uint32_t>(off - blk * kRankIdsPerBlock);
-    const uint4 b = m.buckets[blk];  // x: keys below this block; y, z, w: presence of ids 0-31, 32-63, 64-95
+    const uint64_t off = static_cast<uint64_t>(key) - static_cast<uint64_t>(m.lo);
+    const uint32_t r = static_cast<uint32_t>(off % kRankIdsPerBlock);
+    const uint4 b = p.block;
     const uint32_t word = r < 32 ? b.y : (r < 64 ? b.z : b.w);
     const uint32_t bit = r & 31;
     if (((word >> bit) & 1u) == 0) return -1;
@@ -91,17 +147,12 @@ __device__ __forceinline__ int64_t flat_find(const MapView &m, int64_t key) {
     if (r >= 64) below += __builtin_popcount(b.z);
     return static_cast<int64_t>(b.x + below) + m.delta;
   }
-  const int32_t *direct = reinterpret_cast<const int32_t *>(m.buckets);
-  return static_cast<int64_t>(STREAM ? __builtin_nontemporal_load(direct + off) : direct[off]);
+  return static_cast<int64_t>(p.direct);
 }
 
-// A bucket fragment that will not be looked at again soon (the probe of a
-// row fetch): a non-temporal load, so that probe lines do not push table rows
-// out of the caches.
-typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 load_bucket_streaming(const uint4 *p) {
-  const probe_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4 *>(p));
-  return make_uint4(v.x, v.y, v.z, v.w);
+template <bool STREAM = false>
+__device__ __forceinline__ int64_t flat_find(const MapView &m, int64_t key) {
+  return flat_finish(m, key, flat_issue<STREAM>(m, key));
 }
 
 __device__ __forceinline__ uint32_t map_bucket(const MapView &m, int64_t key) {
@@ -236,42 +287,70 @@ __device__ __forceinline__ bool tile_repeats(int64_t mykey, bool has_key) {
 // streaming only for tiles that show no sign of skew (tile_repeats).
 // Every lane below 32 gets the value for its own key (or -1). All 64 lanes
 // must be active. Flat maps are answered by every lane for itself.
+constexpr int kHalfWaveKeys = 4;  // keys per probe group of a 32-key lookup
+
+// The lookup in two steps, so that a caller can put other work (moving the
+// rows of the tile before) between the loads and their use: half_wave_issue
+// deals the keys to the groups and starts the load of every key's first
+// bucket; half_wave_finish examines what came back and walks on, bucket by
+// bucket, for the few keys whose first bucket was full of other keys.
+struct HalfWaveProbe {
+  uint4 frag[kHalfWaveKeys];  // (the keys are dealt again by half_wave_finish: cheaper than keeping them in registers)
+};
+
 template <int FMT, bool STREAM>
-__device__ __forceinline__ int64_t half_wave_find(const MapView &m, int64_t mykey) {
-  if (m.kind != kKindBuckets) return lane_id() < 32 ? flat_find<STREAM>(m, mykey) : -1;
-  constexpr int kKeys = 4;  // keys per probe group
+__device__ __forceinline__ void half_wave_issue(const MapView &m, int64_t mykey, HalfWaveProbe *p) {
+  const int sub = lane_id() & (kProbeGroup - 1);
+  const int grp = lane_id() / kProbeGroup;
+#pragma unroll
+  for (int j = 0; j < kHalfWaveKeys; ++j) {
+    const int64_t key = shfl64(mykey, grp * kHalfWaveKeys + j);
+    const uint32_t b = map_bucket(m, key);
+    p->frag[j] = STREAM ? load_bucket_streaming(m, b, sub) : m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
+  }
+}
+
+template <int FMT>
+__device__ __forceinline__ int64_t half_wave_finish(const MapView &m, int64_t mykey, const HalfWaveProbe &p) {
   const int lane = lane_id();
   const int sub = lane & (kProbeGroup - 1);
   const int grp = lane / kProbeGroup;
-  int64_t key[kKeys];
-#pragma unroll
-  for (int j = 0; j < kKeys; ++j) key[j] = shfl64(mykey, grp * kKeys + j);
   int64_t res = -1;  // lane 8g + j ends up with the value of key lane 4g + j
-  uint32_t pending = (1u << kKeys) - 1;
-  for (uint32_t round = 0; round < m.nbuckets; ++round) {
-    uint4 frag[kKeys];
+  uint32_t pending = 0;
 #pragma unroll
-    for (int j = 0; j < kKeys; ++j) {
-      if (pending & (1u << j)) {
-        uint32_t b = map_bucket(m, key[j]) + round;
-        if (b >= m.nbuckets) b -= m.nbuckets;
-        const uint4 *at = &m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
-        frag[j] = STREAM ? load_bucket_streaming(at) : *at;
-      }
+  for (int j = 0; j < kHalfWaveKeys; ++j) {
+    int64_t val;
+    if (probe_step<FMT>(p.frag[j], shfl64(mykey, grp * kHalfWaveKeys + j), &val)) {
+      if (sub == j) res = val;
+    } else {
+      pending |= 1u << j;
     }
+  }
+  if (__builtin_amdgcn_ballot_w64(pending != 0) != 0) {  // some first bucket was full of other keys: walk on
 #pragma unroll
-    for (int j = 0; j < kKeys; ++j) {
-      if (pending & (1u << j)) {
+    for (int j = 0; j < kHalfWaveKeys; ++j) {
+      const int64_t key = shfl64(mykey, grp * kHalfWaveKeys + j);  // (all lanes take part in the shuffle)
+      for (uint32_t round = 1; (pending & (1u << j)) && round < m.nbuckets; ++round) {
+        uint32_t b = map_bucket(m, key) + round;
+        if (b >= m.nbuckets) b -= m.nbuckets;
+        const uint4 frag = m.buckets[static_cast<size_t>(b) * kProbeGroup + sub];
         int64_t val;
-        if (probe_step<FMT>(frag[j], key[j], &val)) {
+        if (probe_step<FMT>(frag, key, &val)) {
           pending &= ~(1u << j);
           if (sub == j) res = val;
         }
       }
     }
-    if (pending == 0) break;
   }
-  return shfl64(res, (lane / kKeys) * kProbeGroup + (lane & (kKeys - 1)));
+  return shfl64(res, (lane / kHalfWaveKeys) * kProbeGroup + (lane & (kHalfWaveKeys - 1)));
+}
+
+template <int FMT, bool STREAM>
+__device__ __forceinline__ int64_t half_wave_find(const MapView &m, int64_t mykey) {
+  if (m.kind != kKindBuckets) return lane_id() < 32 ? flat_find<STREAM>(m, mykey) : -1;
+  HalfWaveProbe p;
+  half_wave_issue<FMT, STREAM>(m, mykey, &p);
+  return half_wave_finish<FMT>(m, mykey, p);
 }
 
 }  // namespace shmt
