@@ -293,8 +293,10 @@ def bench_fetch(capi, args, result):
     a = ns * (2 * R + 8) / (t["median"] * 1e-3) / 1e9
     # floor: the same bytes at the rate the 1,048,576-row all-hit fetch sustains (a launch four times shorter
     # spends a larger share of its time filling and draining the chip)
+    t_auto = gpu_time_ms(lambda: capi.cache_set(host, cache, sidx, upd, hmap_auto), 30)
     extra["cache_set_262144"] = {"ms": round(t["median"], 4), "ms_min": round(t["min"], 4), "algorithmic_GBs": round(a, 1),
-                                 "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4),
+                                 "frac_hbm_peak": round(a / HBM_PEAK_GBS, 4), "map_layout": hmap.layout(),
+                                 "ms_through_the_id_range_map": round(t_auto["median"], 4),
                                  "floor_ms_at_all_hit_fetch_rate": round(tm["median"] * ns / Q, 4),
                                  "floor_ms_at_hbm_peak": round(ns * (2 * R + 8) / HBM_PEAK_GBS / 1e6, 4)}
 

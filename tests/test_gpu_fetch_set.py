@@ -462,3 +462,47 @@ def test_fetch_and_set_through_bucket_tables(capi, oracle, D, dtype, slots):
     capi.cache_set(data, gpu_data, torch.from_numpy(w_np + shift).cuda(), upd.cuda(), h)
     torch.cuda.synchronize()
     assert np.array_equal(data.view(view).numpy(), host_ref) and np.array_equal(gpu_data.cpu().view(view).numpy(), gpu_ref)
+
+
+@pytest.mark.parametrize("layout", ["buckets16", "buckets8", "direct"])
+def test_fetch_and_set_through_tables_larger_than_the_caches(capi, layout):
+    """Map tables beyond 64 MiB are read with the streaming cache policy (buffer loads) as long as a wave sees
+    no repeated id, with plain loads afterwards: uniform queries (no repeats), skewed ones (repeats in nearly
+    every tile) and a batch that is half and half must all give what indexing gives, for 16-byte and 8-byte
+    bucket slots and for the direct table."""
+    g = torch.Generator(device="cuda").manual_seed(41)
+    n, D, c = 17_000_000, 8, 4_500_000
+    table_d = torch.arange(n * D, dtype=torch.int32, device="cuda").view(n, D)
+    table = table_d.cpu().pin_memory()
+    ids = torch.randperm(n, device="cuda", generator=g)[:c].contiguous()
+    cache = (table_d[ids] + 1).contiguous()                       # a hit is told from a miss by its content
+    slots = torch.arange(c, device="cuda")
+    if layout == "buckets16":
+        h = capi.CUCOStaticHashmap(ids, slots, 0.5, layout="buckets")
+        assert h.layout() == "buckets" and h.memory_usage() >= 64 << 20
+    elif layout == "buckets8":
+        h = capi.CUCOStaticHashmap(ids.int(), slots.int(), 0.5, layout="buckets")
+        assert h.layout() == "buckets" and 64 << 20 <= h.memory_usage() < 100 << 20
+    else:
+        h = capi.CUCOStaticHashmap(ids, slots, 0.8)
+        assert h.layout() == "direct" and h.memory_usage() >= 64 << 20
+    slot_of = torch.full((n,), -1, dtype=torch.int64, device="cuda")
+    slot_of[ids] = slots
+    q_uniform = torch.randint(0, n, (150_000,), device="cuda", generator=g)
+    hot = ids[:50]                                                  # fifty ids take nearly all requests
+    q_skewed = torch.where(torch.rand(150_000, device="cuda", generator=g) < 0.9,
+                           hot[torch.randint(0, 50, (150_000,), device="cuda", generator=g)], q_uniform)
+    for q in (q_uniform, q_skewed, torch.cat([q_uniform[:70_001], q_skewed[:70_001]])):
+        s = slot_of[q]
+        expect = torch.where((s >= 0)[:, None], cache[s.clamp(min=0)], table_d[q])
+        assert torch.equal(capi.cache_fetch(table, cache, q, h), expect)
+        assert torch.equal(h.query(q).long(), s)
+    # set through the same table: hits land in the cache, misses in the host table
+    uq = torch.unique(q_uniform)[:50_000].contiguous()
+    upd = torch.randint(-1000, 0, (uq.numel(), D), dtype=torch.int32, device="cuda", generator=g)
+    capi.cache_set(table, cache, uq, upd, h)
+    assert torch.equal(capi.cache_fetch(table, cache, uq, h), upd)
+    torch.cuda.synchronize()
+    s = slot_of[uq]
+    assert torch.equal(cache[s[s >= 0]], upd[s >= 0])
+    assert torch.equal(table[uq[s < 0].cpu()], upd[s < 0].cpu())
