@@ -745,72 +745,76 @@ def bench_e2e(capi, args, result):
         tot_nodes += inp.numel()
         del x
     wall = time.perf_counter() - w0
-    # the same batches with each hop issued as one fused call
-    _, inp_f, x = one(batches[nbatch], nbatch, fused=True)
-    del x
-    torch.cuda.synchronize()
-    w0 = time.perf_counter()
-    for b in range(nbatch):
-        _, inp_f, x = one(batches[b], b, fused=True)
+    # (--e2e-operators-only: the reference's operator sequence alone, the form a profile of single kernels wants)
+    wall_fused = wall_pipe = None
+    fetched_ms, in_flight_ms = {}, {}
+    if not args.e2e_operators_only:
+        # the same batches with each hop issued as one fused call
+        _, inp_f, x = one(batches[nbatch], nbatch, fused=True)
         del x
-    torch.cuda.synchronize()
-    wall_fused = time.perf_counter() - w0
-    assert torch.equal(inp_f, inp), "fused hops gave different input nodes"
-    # the same again with the feature fetch queued behind the last relabel (row count read on the device)
-    rng = [7777 + b for b in range(nbatch)]
-    picks = list(reversed(fanouts))
-    cap = int(1.25 * inp.numel())
-    fetched_ms = {}
-    for k_in_flight in (1, 2, 4):
-        # (the warm-up's results are dropped before the timed call, as a training loop drops each batch: the
-        # caching allocator then hands their blocks out again instead of asking the driver for new memory)
-        capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats, feat_cache,
-                                 feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
         torch.cuda.synchronize()
         w0 = time.perf_counter()
-        got = capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats,
-                                       feat_cache, feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
-        torch.cuda.synchronize()
-        fetched_ms[str(k_in_flight)] = round((time.perf_counter() - w0) * 1e3 / nbatch, 3)
-        hops_l, x_l = got[nbatch - 1]
-        assert torch.equal(hops_l[-1][2], inp), "sample_blocks_fetch gave different input nodes"
-        assert torch.equal(x_l, capi.cache_fetch(feats, feat_cache, inp, feat_map)), "sample_blocks_fetch rows differ"
-        del got, hops_l, x_l
-    # sampling + relabel only, several batches advancing concurrently
-    in_flight_ms = {}
-    for k_in_flight in (1, 4, 8):
-        rng = [7777 + b for b in range(nbatch)]
-        capi.sample_blocks(indptr, indices, gp, gi, adj_map, batches[:nbatch], list(reversed(fanouts)), False,
-                           seeds_rng=rng, max_in_flight=k_in_flight)
-        torch.cuda.synchronize()
-        w0 = time.perf_counter()
-        chains = capi.sample_blocks(indptr, indices, gp, gi, adj_map, batches[:nbatch], list(reversed(fanouts)), False,
-                                    seeds_rng=rng, max_in_flight=k_in_flight)
-        torch.cuda.synchronize()
-        in_flight_ms[str(k_in_flight)] = round((time.perf_counter() - w0) * 1e3 / nbatch, 3)
-        assert torch.equal(chains[nbatch - 1][-1][2], inp), "sample_blocks gave different input nodes"
-        del chains
-    # the dataloader sampling ahead on a background thread (4 batches in flight) while this thread fetches
-    import shmtensor
-    dl = shmtensor.GPUSamplingDataloader(indptr, indices, torch.cat(batches[:nbatch]), S, fanouts, shuffle=False,
-                                         rng_seed=7777, prefetch=4, background=True)
-    dl.gpu_indptr, dl.gpu_indices, dl.hashmap, dl.has_cache = gp, gi, adj_map, True
-
-    def epoch():
-        last = None
-        for input_nodes, _, _ in dl:
-            x = capi.cache_fetch(feats, feat_cache, input_nodes, feat_map)
-            last = input_nodes
+        for b in range(nbatch):
+            _, inp_f, x = one(batches[b], b, fused=True)
             del x
         torch.cuda.synchronize()
-        return last
+        wall_fused = time.perf_counter() - w0
+        assert torch.equal(inp_f, inp), "fused hops gave different input nodes"
+        # the same again with the feature fetch queued behind the last relabel (row count read on the device)
+        rng = [7777 + b for b in range(nbatch)]
+        picks = list(reversed(fanouts))
+        cap = int(1.25 * inp.numel())
+        fetched_ms = {}
+        for k_in_flight in (1, 2, 4):
+            # (the warm-up's results are dropped before the timed call, as a training loop drops each batch: the
+            # caching allocator then hands their blocks out again instead of asking the driver for new memory)
+            capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats, feat_cache,
+                                     feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
+            torch.cuda.synchronize()
+            w0 = time.perf_counter()
+            got = capi.sample_blocks_fetch(indptr, indices, gp, gi, adj_map, batches[:nbatch], picks, False, feats,
+                                           feat_cache, feat_map, seeds_rng=rng, max_in_flight=k_in_flight, max_rows=cap)
+            torch.cuda.synchronize()
+            fetched_ms[str(k_in_flight)] = round((time.perf_counter() - w0) * 1e3 / nbatch, 3)
+            hops_l, x_l = got[nbatch - 1]
+            assert torch.equal(hops_l[-1][2], inp), "sample_blocks_fetch gave different input nodes"
+            assert torch.equal(x_l, capi.cache_fetch(feats, feat_cache, inp, feat_map)), "sample_blocks_fetch rows differ"
+            del got, hops_l, x_l
+        # sampling + relabel only, several batches advancing concurrently
+        in_flight_ms = {}
+        for k_in_flight in (1, 4, 8):
+            rng = [7777 + b for b in range(nbatch)]
+            capi.sample_blocks(indptr, indices, gp, gi, adj_map, batches[:nbatch], list(reversed(fanouts)), False,
+                               seeds_rng=rng, max_in_flight=k_in_flight)
+            torch.cuda.synchronize()
+            w0 = time.perf_counter()
+            chains = capi.sample_blocks(indptr, indices, gp, gi, adj_map, batches[:nbatch], list(reversed(fanouts)), False,
+                                        seeds_rng=rng, max_in_flight=k_in_flight)
+            torch.cuda.synchronize()
+            in_flight_ms[str(k_in_flight)] = round((time.perf_counter() - w0) * 1e3 / nbatch, 3)
+            assert torch.equal(chains[nbatch - 1][-1][2], inp), "sample_blocks gave different input nodes"
+            del chains
+        # the dataloader sampling ahead on a background thread (4 batches in flight) while this thread fetches
+        import shmtensor
+        dl = shmtensor.GPUSamplingDataloader(indptr, indices, torch.cat(batches[:nbatch]), S, fanouts, shuffle=False,
+                                             rng_seed=7777, prefetch=4, background=True)
+        dl.gpu_indptr, dl.gpu_indices, dl.hashmap, dl.has_cache = gp, gi, adj_map, True
 
-    # first epoch: batch b draws from seed 7777 + b like the loops above (later epochs continue the count)
-    assert torch.equal(epoch(), inp), "prefetching dataloader gave different input nodes"
-    w0 = time.perf_counter()
-    epoch()
-    wall_pipe = time.perf_counter() - w0
-    dl.close()          # the producer thread has ended with its epoch; this only makes that explicit
+        def epoch():
+            last = None
+            for input_nodes, _, _ in dl:
+                x = capi.cache_fetch(feats, feat_cache, input_nodes, feat_map)
+                last = input_nodes
+                del x
+            torch.cuda.synchronize()
+            return last
+
+        # first epoch: batch b draws from seed 7777 + b like the loops above (later epochs continue the count)
+        assert torch.equal(epoch(), inp), "prefetching dataloader gave different input nodes"
+        w0 = time.perf_counter()
+        epoch()
+        wall_pipe = time.perf_counter() - w0
+        dl.close()          # the producer thread has ended with its epoch; this only makes that explicit
     cpu = None
     if not args.no_cpu:
         import numpy as np
@@ -857,8 +861,8 @@ def bench_e2e(capi, args, result):
         "feature_hit_rate": round(hit, 4),
         "sample_relabel_ms": round(t_s / nbatch, 3), "fetch_ms": round(t_f / nbatch, 3),
         "batch_ms_wall": round(wall * 1e3 / nbatch, 3), "batches_per_s": round(nbatch / wall, 2),
-        "fused_hop_batch_ms_wall": round(wall_fused * 1e3 / nbatch, 3),
-        "background_prefetch_batch_ms_wall": round(wall_pipe * 1e3 / nbatch, 3),
+        "fused_hop_batch_ms_wall": wall_fused and round(wall_fused * 1e3 / nbatch, 3),
+        "background_prefetch_batch_ms_wall": wall_pipe and round(wall_pipe * 1e3 / nbatch, 3),
         "sample_blocks_fetch_batch_ms_wall_by_batches_in_flight": fetched_ms,
         "sample_blocks_ms_per_batch_by_batches_in_flight": in_flight_ms,
         "sampled_edges_per_s": round(tot_edges / (t_s * 1e-3), 1),
@@ -1030,6 +1034,9 @@ def main():
     ap.add_argument("--sampling-batches", type=int, default=50)
     ap.add_argument("--e2e-scale", type=int, default=24)
     ap.add_argument("--e2e-batches", type=int, default=24)
+    ap.add_argument("--e2e-operators-only", action="store_true",
+                    help="e2e workload: only the batches issued operator by operator (no fused, pipelined or "
+                         "prefetching forms)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--headline-map", default="buckets", choices=["buckets", "auto"],
