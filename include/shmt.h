@@ -274,6 +274,14 @@ int shmt_async_error(int *code_out);
 /* Sets bits of that word from the host, as a kernel that gave up would: for
  * tests of the error path (no kernel has to starve for them).               */
 int shmt_async_error_inject(int bits);
+/* Optional: a 4-byte word in pinned host memory (its host address and the
+ * address the current GPU reaches it at, shmt_host_devptr) that a kernel
+ * giving up also sets to non-zero, so that a host loop which polls pinned
+ * memory anyway learns of it without a device call; shmt_async_error clears
+ * it together with the GPU's word. The word must outlive every later launch
+ * on that GPU, or be withdrawn first (null, null). No counterpart in the
+ * reference.                                                                */
+int shmt_async_error_mirror(void *host_word, void *device_alias);
 /* shmt_exclusive_scan without a workspace argument, and without any
  * allocation inside the call. It has no counterpart in the reference (whose
  * cub_exclusiveSum allocates its temporary storage on every call,

@@ -46,6 +46,7 @@ SIGNATURES = {
     "shmt_inclusive_scan_i32_kept": (_int, [_vp, _i64, _vp, _i64, _vp]),
     "shmt_async_error": (_int, [_c.POINTER(_int)]),
     "shmt_async_error_inject": (_int, [_int]),
+    "shmt_async_error_mirror": (_int, [_vp, _vp]),
     "shmt_relabel_scratch_bytes": (_i64, [_i64]),
     "shmt_relabel": (_int, [_vp, _i64, _int, _vp, _i64, _vp, _vp, _vp, _vp]),
     "shmt_relabel_wide_scratch_bytes": (_i64, [_i64]),

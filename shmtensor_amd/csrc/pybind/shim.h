@@ -77,7 +77,10 @@ inline void *device_address(const torch::Tensor &t, const char *name) {
 // soon as the kernel that computes it has run, while later kernels of the
 // same operator are still queued or running. If the value does not show up
 // within the spin budget (a failed launch, a hung device) the wait falls back
-// to a stream synchronisation, which surfaces the error.
+// to a stream synchronisation, which surfaces the error. One more pinned word
+// mirrors the GPU's error word (shmt_async_error_mirror): a kernel that gave
+// up a bounded wait sets it, and every wait here looks at it, so the failure
+// surfaces as an exception at the next size read-back at no cost otherwise.
 class Readback {
  public:
   static constexpr int kSlots = 4096;  // a ring: more than all operators together keep pending at once
@@ -89,10 +92,16 @@ class Readback {
   Slot acquire() {
     std::lock_guard<std::mutex> lock(mutex_);
     if (!host_.defined()) {
-      host_ = torch::zeros({kSlots}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+      host_ = torch::zeros({kSlots + 1}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
       void *d = nullptr;
       check(shmt_host_devptr(host_.data_ptr(), &d));
       dev_ = static_cast<int64_t *>(d);
+      gave_up_ = reinterpret_cast<volatile uint32_t *>(host_.data_ptr<int64_t>() + kSlots);
+    }
+    const int device = static_cast<int>(c10::hip::current_device());
+    if (device >= 0 && device < 64 && !(mirrored_ >> device & 1)) {  // once per GPU this process launches on
+      check(shmt_async_error_mirror(const_cast<uint32_t *>(gave_up_), dev_ + kSlots));
+      mirrored_ |= 1ull << device;
     }
     const uint32_t i = next_;
     next_ = (next_ + 1) % kSlots;  // stays in [0, kSlots): nothing counts up without bound
@@ -106,7 +115,10 @@ class Readback {
     const auto t0 = std::chrono::steady_clock::now();
     for (uint64_t spins = 0;; ++spins) {
       const int64_t v = *s.host;
-      if (v != kPending) return v;
+      if (v != kPending) {
+        if (gave_up_ && *gave_up_ != 0) report_gave_up();
+        return v;
+      }
       if ((spins & 1023) == 1023 &&
           std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(kSpinBudgetMs))
         break;
@@ -119,15 +131,25 @@ class Readback {
       const bool known = shmt_async_error(&gave_up) == SHMT_OK && gave_up != 0;
       TORCH_CHECK(false, known ? shmt_last_error() : "the GPU did not report a result size (kernel failed?)");
     }
+    if (gave_up_ && *gave_up_ != 0) report_gave_up();
     return v;
   }
 
  private:
+  // Reads and clears the GPU's error word (which also clears the mirror) and raises what it says.
+  static void report_gave_up() {
+    int code = 0;
+    check(shmt_async_error(&code));
+    TORCH_CHECK(code == 0, shmt_last_error());
+  }
+
   static constexpr int64_t kPending = INT64_MIN;
   static constexpr int kSpinBudgetMs = 200;
   std::mutex mutex_;  // operators may run on several host threads (sample_blocks)
   torch::Tensor host_;
   int64_t *dev_ = nullptr;
+  static inline volatile uint32_t *gave_up_ = nullptr;  // the mirror word, behind the slots
+  uint64_t mirrored_ = 0;                 // bit d: the mirror is registered with GPU d
   uint32_t next_ = 0;
 };
 

@@ -96,6 +96,7 @@ constexpr int64_t kScanHeaderBytes = 64;  // tile counter (+ padding) in front o
 struct ScanState {
   unsigned long long *counter;  // next tile number to hand out; counter[1]: workgroups that are done
   uint32_t *error;              // the GPU's error word
+  uint32_t *error_mirror;       // where the host watches for it (device alias of a pinned host word), or null
   int64_t words;                // 64-bit words of the workspace behind the header (tiles, groups, runs)
   uint64_t *tiles;              // 2 words per tile
   uint64_t *groups;             // 2 words per group of 64 tiles
@@ -182,7 +183,11 @@ __device__ __forceinline__ uint64_t tile_lookback(const ScanState &st, int64_t t
     else __builtin_amdgcn_s_sleep(8);
   }
   if (lost) {  // report, publish nothing: the tile is left as it was and so is everything behind it
-    if (lane == 0) __hip_atomic_fetch_or(st.error, kErrScanWait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) {
+      __hip_atomic_fetch_or(st.error, kErrScanWait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // a plain system-scope store: the host only asks whether the word is zero, the bits are in st.error
+      if (st.error_mirror) __hip_atomic_store(st.error_mirror, kErrScanWait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
     *gave_up = true;
     return 0;
   }
@@ -377,6 +382,8 @@ static int resident_workgroups(const void *kernel, int *out) {
 constexpr int kMaxDevices = 64;
 static std::mutex g_symbol_mutex;
 static uint32_t *g_error_ptr[kMaxDevices];
+static uint32_t *g_mirror_dev[kMaxDevices];            // shmt_async_error_mirror: the pinned word as the GPU addresses it
+static volatile uint32_t *g_mirror_host[kMaxDevices];  // and as the host does
 
 static int error_word(uint32_t **out) {
   int dev = -1;
@@ -391,6 +398,13 @@ static int error_word(uint32_t **out) {
   }
   *out = g_error_ptr[dev];
   return SHMT_OK;
+}
+
+static uint32_t *error_mirror() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_symbol_mutex);
+  return g_mirror_dev[dev];
 }
 
 // kept: the workspace is all zero (it was cleared once and has only been used by scans since, each of
@@ -423,6 +437,7 @@ static int scan_inplace(T *data, int64_t len, void *tmp, int64_t tmp_bytes, bool
   st.counter = static_cast<unsigned long long *>(tmp);
   int rc = error_word(&st.error);
   if (rc) return rc;
+  st.error_mirror = error_mirror();
   st.words = (need - kScanHeaderBytes) / 8;
   st.tiles = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.tiles_off);
   st.groups = reinterpret_cast<uint64_t *>(static_cast<char *>(tmp) + l.groups_off);
@@ -568,6 +583,12 @@ int shmt_async_error(int *code_out) {
   if (seen != 0) {
     const uint32_t zero = 0;
     SHMT_HIP(hipMemcpy(err, &zero, sizeof(zero), hipMemcpyHostToDevice));
+    int dev = -1;
+    SHMT_HIP(hipGetDevice(&dev));
+    {
+      std::lock_guard<std::mutex> lock(g_symbol_mutex);
+      if (dev >= 0 && dev < kMaxDevices && g_mirror_host[dev]) *g_mirror_host[dev] = 0;
+    }
     set_error("a kernel gave up a bounded wait for another workgroup (error bits 0x%x): %s", seen,
               (seen & kErrScanWait) ? "the look-back of a device-wide scan; the scanned array is incomplete" : "unknown");
   }
@@ -583,6 +604,25 @@ int shmt_async_error_inject(int bits) {
   SHMT_HIP(hipMemcpy(&seen, err, sizeof(seen), hipMemcpyDeviceToHost));
   seen |= static_cast<uint32_t>(bits);
   SHMT_HIP(hipMemcpy(err, &seen, sizeof(seen), hipMemcpyHostToDevice));
+  int dev = -1;
+  SHMT_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_symbol_mutex);
+  if (bits != 0 && dev >= 0 && dev < kMaxDevices && g_mirror_host[dev]) *g_mirror_host[dev] = seen;
+  return SHMT_OK;
+}
+
+int shmt_async_error_mirror(void *host_word, void *device_alias) {
+  SHMT_REQUIRE((host_word == nullptr) == (device_alias == nullptr),
+               "shmt_async_error_mirror: pass both addresses of the word, or null twice");
+  SHMT_REQUIRE((reinterpret_cast<uintptr_t>(host_word) & 3) == 0 && (reinterpret_cast<uintptr_t>(device_alias) & 3) == 0,
+               "shmt_async_error_mirror: the word must be 4-byte aligned");
+  int dev = -1;
+  SHMT_HIP(hipGetDevice(&dev));
+  SHMT_REQUIRE(dev >= 0 && dev < kMaxDevices, "shmt_async_error_mirror: device ordinal %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_symbol_mutex);
+  g_mirror_host[dev] = static_cast<volatile uint32_t *>(host_word);
+  g_mirror_dev[dev] = static_cast<uint32_t *>(device_alias);
+  if (host_word) *g_mirror_host[dev] = 0;
   return SHMT_OK;
 }
 

@@ -358,3 +358,13 @@ def test_a_wait_that_gave_up_is_reported(capi, cabi):
     assert code.value == 1 and b"gave up a bounded wait" in lib.shmt_last_error()
     cabi.check(lib.shmt_async_error(ctypes.byref(code)))
     assert code.value == 0
+    # the shim also watches a pinned mirror of the word: the next operator that reads a size back raises, the
+    # one after it works again
+    a = torch.arange(100_000, device="cuda") % 977
+    capi.tensor_relabel([a])                                    # first read-back registers the mirror word
+    cabi.check(lib.shmt_async_error_inject(1))
+    with pytest.raises(RuntimeError, match="look-back of a device-wide scan"):
+        capi.tensor_relabel([a])
+    uniq, _ = capi.tensor_relabel([a])
+    assert uniq.numel() == 977
+    capi.raise_async_error()
