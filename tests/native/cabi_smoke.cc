@@ -7,6 +7,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include <algorithm>
 #include <numeric>
@@ -152,6 +153,37 @@ int main() {
   EXPECT(shmt_fetch_counted(table_alias, d_cache, d_q, 4, fmap, nullptr, 0, d_out, Q, nullptr, nullptr,
                             row_bytes, stream) == SHMT_EINVAL);
   HIP_OK(hipFree(d_count));
+  // the same fetch in two launches: the rows that hit on this stream, the rows that missed from a few
+  // workgroups on a second stream once an event says the first part is done; the bitmap is never cleared
+  {
+    hipStream_t side = nullptr;
+    hipEvent_t hits_done = nullptr, misses_done = nullptr;
+    HIP_OK(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
+    HIP_OK(hipEventCreateWithFlags(&hits_done, hipEventDisableTiming));
+    HIP_OK(hipEventCreateWithFlags(&misses_done, hipEventDisableTiming));
+    uint32_t *d_bits = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_bits), ((Q + 31) / 32) * 4));
+    HIP_OK(hipMemsetAsync(d_bits, 0xA5, ((Q + 31) / 32) * 4, stream));   // stale content must not matter
+    HIP_OK(hipMemsetAsync(d_out, 0x5A, Q * row_bytes, stream));
+    SHMT_OK_(shmt_fetch_cached_part(table_alias, d_cache, d_q, 4, fmap, nullptr, 0, d_out, Q, nullptr, row_bytes,
+                                    d_bits, stream));
+    HIP_OK(hipEventRecord(hits_done, stream));
+    HIP_OK(hipStreamWaitEvent(side, hits_done, 0));
+    SHMT_OK_(shmt_fetch_missed_part(table_alias, d_q, 4, d_bits, d_out, Q, nullptr, row_bytes, 8, side));
+    HIP_OK(hipEventRecord(misses_done, side));
+    HIP_OK(hipStreamWaitEvent(stream, misses_done, 0));
+    HIP_OK(hipStreamSynchronize(stream));
+    EXPECT(to_host(d_out, Q * row_bytes) == out);
+    std::vector<uint32_t> bits = to_host(d_bits, (Q + 31) / 32);
+    for (int64_t i = 0; i < Q; ++i) EXPECT(((bits[i / 32] >> (i % 32)) & 1u) == (slot_of.count(q[i]) ? 0u : 1u));
+    // rows that do not allow 16-byte accesses are refused
+    EXPECT(shmt_fetch_cached_part(table_alias, d_cache, d_q, 4, fmap, nullptr, 0, d_out, Q, nullptr, 24, d_bits,
+                                  stream) == SHMT_EINVAL);
+    HIP_OK(hipFree(d_bits));
+    HIP_OK(hipEventDestroy(hits_done));
+    HIP_OK(hipEventDestroy(misses_done));
+    HIP_OK(hipStreamDestroy(side));
+  }
   // pageable host memory is refused instead of faulting
   std::vector<char> pageable(4096);
   void *alias = nullptr;
@@ -333,6 +365,68 @@ int main() {
       r2 += static_cast<uint32_t>(b2[i]);
     }
     EXPECT(shmt_exclusive_scan_noalloc(d_b1, SHMT_SCAN_NOALLOC_MAX_LEN + 1, 8, stream) == SHMT_EINVAL);
+  }
+
+  // ---- scans on a workspace that is cleared once and then kept: no clearing launch, left all zero ----
+  {
+    const int64_t l1 = 2500003, l2 = 900001;
+    std::vector<int64_t> b1(l1);
+    for (auto &x : b1) x = static_cast<int64_t>(rnd() >> 8);
+    std::vector<uint32_t> b2(l2);
+    for (auto &x : b2) x = static_cast<uint32_t>(rnd() % 1000);
+    int64_t *d_b1 = to_device(b1);
+    uint32_t *d_b2 = to_device(b2);
+    const int64_t wbytes = std::max(shmt_scan_tmp_bytes(l1), shmt_scan_tmp_bytes(l2));
+    char *d_ws = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_ws), wbytes));
+    HIP_OK(hipMemsetAsync(d_ws, 0xEE, wbytes, stream));
+    SHMT_OK_(shmt_scan_workspace_clear(d_ws, wbytes, stream));
+    SHMT_OK_(shmt_exclusive_scan_kept(d_b1, l1, 8, d_ws, wbytes, stream));
+    SHMT_OK_(shmt_inclusive_scan_i32_kept(d_b2, l2, d_ws, wbytes, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<int64_t> s1 = to_host(d_b1, l1);
+    uint64_t r1 = 0;
+    for (int64_t i = 0; i < l1; ++i) {
+      EXPECT(static_cast<uint64_t>(s1[i]) == r1);
+      r1 += static_cast<uint64_t>(b1[i]);
+    }
+    std::vector<uint32_t> s2 = to_host(d_b2, l2);
+    uint32_t r2 = 0;
+    for (int64_t i = 0; i < l2; ++i) {
+      r2 += b2[i];
+      EXPECT(s2[i] == r2);
+    }
+    for (char c : to_host(d_ws, wbytes)) EXPECT(c == 0);
+    HIP_OK(hipFree(d_ws));
+    HIP_OK(hipFree(d_b1));
+    HIP_OK(hipFree(d_b2));
+  }
+
+  // ---- the error word of bounded waits, set from the host: read-and-clear, and its pinned mirror ----
+  {
+    int code = -1;
+    SHMT_OK_(shmt_async_error(&code));
+    EXPECT(code == 0);
+    uint32_t *h_word = nullptr;
+    HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&h_word), 4, hipHostMallocDefault));
+    void *word_alias = nullptr;
+    SHMT_OK_(shmt_host_devptr(h_word, &word_alias));
+    *h_word = 0xFFFFFFFFu;
+    SHMT_OK_(shmt_async_error_mirror(h_word, word_alias));
+    EXPECT(*h_word == 0);
+    EXPECT(shmt_async_error_mirror(h_word, nullptr) == SHMT_EINVAL);
+    SHMT_OK_(shmt_async_error_inject(1));
+    EXPECT(*static_cast<volatile uint32_t *>(h_word) != 0);
+    SHMT_OK_(shmt_async_error(&code));
+    EXPECT(code == 1 && strstr(shmt_last_error(), "look-back of a device-wide scan") != nullptr);
+    EXPECT(*static_cast<volatile uint32_t *>(h_word) == 0);
+    SHMT_OK_(shmt_async_error(&code));
+    EXPECT(code == 0);
+    SHMT_OK_(shmt_async_error_mirror(nullptr, nullptr));   // withdrawn before the word is freed
+    HIP_OK(hipHostFree(h_word));
+    // a kernel that only passes time (the probe for streams that run side by side)
+    SHMT_OK_(shmt_busy_wait(stream, 50));
+    HIP_OK(hipStreamSynchronize(stream));
   }
 
   // ---- coordinate form: destination position of every sampled id, from a hop job and from sub_indptr ----
