@@ -328,8 +328,79 @@ __device__ __forceinline__ int64_t load_adj(const PickArgs &a, int64_t begin_tag
 // flags as one 64-bit lane mask, which costs five vector and eight scalar
 // instructions per step for two groups of 32; smaller groups (at most seven
 // steps) use a lane permute.
+// Sorting network for the resolution below: bitonic sort, ascending, of one
+// 32-bit key per lane within every group of G lanes (G = 16 or 32). A stage
+// exchanges keys between lanes l and l ^ STRIDE (ds_swizzle in bit mode: no
+// memory is touched) and keeps the smaller or the larger one; which lanes keep
+// the smaller one is a constant of the stage.
+template <int G>
+constexpr uint64_t bitonic_keeps_min(int size, int stride) {
+  uint64_t m = 0;
+  for (int l = 0; l < kWave; ++l) {
+    const int gl = l & (G - 1);
+    const bool up = (gl & size) == 0, lower = (gl & stride) == 0;
+    if (up == lower) m |= 1ull << l;
+  }
+  return m;
+}
+
+template <int G, int SIZE, int STRIDE>
+__device__ __forceinline__ uint32_t bitonic_sort_from(uint32_t key) {
+  constexpr int kPattern = (STRIDE << 10) | 0x1F;  // bit mode: and 0x1F, or 0, xor STRIDE
+  constexpr uint64_t kKeepsMin = bitonic_keeps_min<G>(SIZE, STRIDE);
+  const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_ds_swizzle(static_cast<int>(key), kPattern));
+  const uint32_t lo = key < other ? key : other, hi = key < other ? other : key;
+  key = __builtin_amdgcn_inverse_ballot_w64(kKeepsMin) ? lo : hi;
+  if constexpr (STRIDE > 1) return bitonic_sort_from<G, SIZE, STRIDE / 2>(key);
+  else if constexpr (SIZE < G) return bitonic_sort_from<G, SIZE * 2, SIZE>(key);
+  else return key;
+}
+
+// "Some lane before mine in my group drew the same value": the flag that
+// decides Floyd's selection whenever no draw lies among the k largest
+// positions (see floyd_resolve32). The draws are sorted together with their
+// lane numbers ((t << 5) | gl, which needs t < 2^27 - 1), equal draws then
+// stand side by side in lane order, every one but the first is such a repeat,
+// and the flag travels back to its lane with one permute. 15 exchange stages
+// for 32 lanes (10 for 16) instead of one dependent step per pick.
+template <int G>
+__device__ __forceinline__ bool repeats_earlier_draw(uint32_t t, bool live, int gl) {
+  static_assert(G == 16 || G == 32, "one swizzle domain holds one or two whole groups");
+  const uint32_t key = live ? ((t << 5) | static_cast<uint32_t>(gl)) : (0xFFFFFFE0u | static_cast<uint32_t>(gl));
+  const uint32_t sorted = bitonic_sort_from<G, 2, 1>(key);
+  const uint32_t before = static_cast<uint32_t>(__shfl_up(static_cast<int>(sorted), 1, kWave));
+  const bool repeat = gl != 0 && (before >> 5) == (sorted >> 5) && sorted < 0xFFFFFFE0u;
+  const int home = (lane_id() & ~(G - 1)) + static_cast<int>(sorted & 31u);
+  return __builtin_amdgcn_ds_permute(home << 2, repeat ? 1 : 0) != 0;
+}
+
 template <int G>
 __device__ __forceinline__ uint32_t floyd_resolve32(uint32_t t, uint32_t top, int gl, int k) {
+  if constexpr (G == 16 || G == 32) {
+    // Step j falls back to J = top_j exactly when t_j is among the earlier choices, and that is the case
+    // when (a) an earlier lane drew the same value (its choice, or an earlier one, is that value), or
+    // (b) t_j is the J of an earlier step i = t_j - (deg - k) < j that fell back itself. (a) needs no
+    // step to wait for another; (b) hangs a lane on one earlier lane, needs a draw among the k largest
+    // positions (probability about k / deg) and is settled by following those links until nothing
+    // changes: a link leads to a smaller lane, so every round settles at least one more lane.
+    const uint32_t base = top - static_cast<uint32_t>(gl);  // deg - k, the same for the whole group
+    const bool live = gl < k;
+    const bool packs = base < (1u << 27) - 64u;
+    if (__builtin_amdgcn_ballot_w64(!packs) == 0) {
+      bool hit = repeats_earlier_draw<G>(t, live, gl) && live;
+      const bool linked = live && t >= base && static_cast<int>(t - base) < gl;
+      const int from = (lane_id() & ~(G - 1)) + static_cast<int>(linked ? t - base : 0u);
+      if (__builtin_amdgcn_ballot_w64(linked) != 0) {
+        for (;;) {
+          const uint64_t hits = __builtin_amdgcn_ballot_w64(hit);
+          const bool now = hit || (linked && ((hits >> from) & 1ull) != 0);
+          if (__builtin_amdgcn_ballot_w64(now != hit) == 0) break;
+          hit = now;
+        }
+      }
+      return hit ? top : t;
+    }
+  }
   if (G == 32) {
     uint64_t hit = 0;
     for (int step = 0; step + 1 < k; ++step) {
