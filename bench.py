@@ -1092,6 +1092,39 @@ def main():
     if "e2e" in todo:
         torch.cuda.empty_cache()
         bench_e2e(capi, args, result)
+    # the figures a reader wants without digging through `extra`, and `extra` last
+    extra = result.pop("extra")
+    summary = {}
+    by_map = extra.get("fetch_all_hit_by_map_layout")
+    if by_map:
+        summary["fetch_all_hit_frac_hbm_peak_by_map_layout"] = dict(
+            {k: v["frac_hbm_peak"] for k, v in by_map.items()},
+            id_range=extra["fetch_all_hit"]["frac_hbm_peak"], mask=extra["fetch_all_hit_with_mask"]["frac_hbm_peak"])
+    if "scan" in extra:
+        summary["scan_frac_hbm_peak"] = {"exclusive_int64": extra["scan"]["exclusive_int64_16777216"]["frac_hbm_peak"],
+                                         "inclusive_int32": extra["scan"]["thrust_scan_int32_16777216"]["frac_hbm_peak"]}
+    if "hashmap_config2" in extra:
+        summary["hashmap_query_line_traffic_frac_hbm_peak"] = extra["hashmap_config2"]["query_line_traffic_frac_hbm_peak"]
+    if "sampling_config3" in extra:
+        s3 = extra["sampling_config3"]
+        summary["config3_ms_per_batch"] = {"operators": s3["ms_per_batch"], "fused_hop": s3["fused_hop_ms_per_batch"],
+                                           "chained_hops": s3["chained_hops_ms_per_batch"],
+                                           "batches_sharing_launches": min(
+                                               v["ms_per_batch"] for v in s3["sample_blocks_batches_in_flight"].values())}
+        speedups = {k: s3[k] for k in ("speedup_vs_cpu", "speedup_vs_cpu_chained_hops",
+                                       "speedup_vs_cpu_batches_sharing_launches") if k in s3}
+        if speedups:
+            summary["config3_speedup_vs_fastest_cpu_baseline"] = speedups
+    if "e2e_config5" in extra:
+        e5 = extra["e2e_config5"]
+        summary["config5_ms_per_batch"] = {"operators": e5["batch_ms_wall"], "sample_relabel": e5["sample_relabel_ms"],
+                                           "fetch": e5["fetch_ms"]}
+        if e5["sample_blocks_fetch_batch_ms_wall_by_batches_in_flight"]:
+            summary["config5_ms_per_batch"]["sampler_and_fetch_pipelined"] = min(
+                e5["sample_blocks_fetch_batch_ms_wall_by_batches_in_flight"].values())
+    if summary:
+        result["summary"] = summary
+    result["extra"] = extra
     print(json.dumps(result), flush=True)
 
 
