@@ -9,8 +9,10 @@
 //   first    first[i] = smallest index holding the same key (kept in the
 //            labels buffer); per-tile count of i with first[i] == i
 //   partials exclusive scan of the per-tile counts (own launch only beyond 2 M ids)
-//   unique   rank of every first occurrence; unique[rank] = key; rank_of[i]
-//   labels   labels[i] = rank_of[first[i]]
+//   unique   rank of every first occurrence; unique[rank] = key; per 64
+//            elements a bitmap of the first occurrences among them and the
+//            number of first occurrences before them (RlRanks)
+//   labels   labels[i] = rank of element first[i], from that bitmap
 // The table is touched only by `insert` and `first`; the last two passes read
 // dense arrays. Slots are 16 bytes {int64 key, uint32 first, pad} at load
 // factor <= 0.5 with a mixed hash (the reference hashes with the low bits of
@@ -339,6 +341,19 @@ __global__ __launch_bounds__(kRlTile) void rl_first_jobs(Jobs<RlFirstArgs> j) {
   if (blockIdx.x < j.blocks[blockIdx.y]) rl_first_body(blockIdx.x, j.a[blockIdx.y]);
 }
 
+// Ranks of the first occurrences, 16 bytes per 64 consecutive elements: bit b of `firsts` says that
+// element 64 w + b is the first occurrence of its id, `before` is the number of first occurrences in
+// front of element 64 w. The rank of a first occurrence f is before + popcount(firsts below bit f & 63):
+// one 16-byte load from an array of N / 4 bytes, which stays in the L2s where an array of one rank per
+// element (4 N bytes, read at random positions by the labels pass) did not.
+struct RlRanks {
+  uint64_t firsts;
+  uint32_t before;
+  uint32_t pad;
+};
+static_assert(sizeof(RlRanks) == 16, "one 16-byte load per lookup");
+static_assert(kRlTile % kWave == 0 && kRlItems * kWave * (kRlBlock / kWave) == kRlTile, "a wave ranks whole 64-element words");
+
 struct RlUniqueArgs {
   const void *total;
   int eb;
@@ -346,7 +361,7 @@ struct RlUniqueArgs {
   const void *labels;
   const uint64_t *partials;
   void *unique_out;
-  uint32_t *rank_of;
+  RlRanks *ranks;
   int64_t *count_out;
   int64_t *count_copy;
   int scanned;
@@ -358,11 +373,10 @@ __device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &
   const void *const labels = a.labels;
   const uint64_t *const partials = a.partials;
   void *const unique_out = a.unique_out;
-  uint32_t *const rank_of = a.rank_of;
   const int64_t N = rl_count(a.n);
   // launched for a bound of N: only the tiles that hold ids work (tile 0 reports N = 0)
   if (bx > 0 && static_cast<int64_t>(bx) * kRlTile >= N) return;
-  __shared__ uint32_t lds[kRlBlock / kWave];
+  __shared__ uint32_t wave_firsts[kRlBlock / kWave];
   __shared__ uint64_t lds64[kRlBlock / kWave];
   // Tile prefix: either already scanned by a separate launch, or (few tiles)
   // summed here from the raw per-tile counts.
@@ -376,36 +390,46 @@ __device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &
     block_exclusive_scan<uint64_t, kRlBlock>(part, lds64, &below);
     tile_prefix = below;
   }
-  const int64_t first_i = static_cast<int64_t>(bx) * kRlTile +
-                          static_cast<int64_t>(threadIdx.x) * kRlItems;
+  // a wave takes kRlItems words of 64 consecutive elements: element = word start + lane
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int64_t wave_first = static_cast<int64_t>(bx) * kRlTile + static_cast<int64_t>(wave) * (kRlItems * kWave);
   bool win[kRlItems], ok[kRlItems];
   int64_t idx[kRlItems], lab[kRlItems], val[kRlItems];
-  uint32_t mine = 0;
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
-    idx[j] = first_i + j;
+    idx[j] = wave_first + j * kWave + lane;
     ok[j] = idx[j] < N;
     lab[j] = -1;
     val[j] = 0;
   }
   load_ints<kRlItems>(labels, idx, ok, eb, lab);
+  uint64_t firsts[kRlItems];
+  uint32_t mine = 0;  // first occurrences of this wave
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
     win[j] = ok[j] && lab[j] == idx[j];
-    mine += win[j];
+    firsts[j] = __builtin_amdgcn_ballot_w64(win[j]);
+    mine += static_cast<uint32_t>(__builtin_popcountll(firsts[j]));
   }
   load_ints<kRlItems>(total, idx, win, eb, val);
-  uint32_t tile_total;
-  uint32_t ex = block_exclusive_scan<uint32_t, kRlBlock>(mine, lds, &tile_total);
-  uint64_t rank = tile_prefix + ex;
+  if (lane == 0) wave_firsts[wave] = mine;
+  __syncthreads();
+  uint32_t before_wave = 0, tile_total = 0;
+#pragma unroll
+  for (int w = 0; w < kRlBlock / kWave; ++w) {
+    const uint32_t c = wave_firsts[w];
+    if (w < wave) before_wave += c;
+    tile_total += c;
+  }
+  uint64_t word_rank = tile_prefix + before_wave;  // rank of the first first-occurrence of the word
+  const uint64_t below_lane = (1ull << lane) - 1ull;
 #pragma unroll
   for (int j = 0; j < kRlItems; ++j) {
-    const int64_t i = first_i + j;
-    if (win[j]) {
-      store_int(unique_out, static_cast<int64_t>(rank), eb, val[j]);
-      rank_of[i] = static_cast<uint32_t>(rank);
-      ++rank;
-    }
+    if (win[j])
+      store_int(unique_out, static_cast<int64_t>(word_rank + __builtin_popcountll(firsts[j] & below_lane)), eb, val[j]);
+    const int64_t word_start = wave_first + j * kWave;
+    if (lane == 0 && word_start < N) a.ranks[word_start / kWave] = RlRanks{firsts[j], static_cast<uint32_t>(word_rank), 0u};
+    word_rank += static_cast<uint64_t>(__builtin_popcountll(firsts[j]));
   }
   // the workgroup holding the last id reports the number of distinct ids
   const int64_t last_tile = N > 0 ? (N - 1) / kRlTile : 0;
@@ -425,7 +449,7 @@ struct RlLabelsArgs {
   void *labels;
   int eb;
   RlCount n;
-  const uint32_t *rank_of;
+  const RlRanks *ranks;
 };
 
 __device__ __forceinline__ void rl_labels_body(unsigned bx, unsigned gx, const RlLabelsArgs &a) {
@@ -434,7 +458,10 @@ __device__ __forceinline__ void rl_labels_body(unsigned bx, unsigned gx, const R
   const int64_t stride = static_cast<int64_t>(gx) * blockDim.x;
   for (; i < N; i += stride) {
     const int64_t f = load_int(a.labels, i, a.eb);
-    store_int(a.labels, i, a.eb, static_cast<int64_t>(a.rank_of[f]));
+    const uint4 r = *reinterpret_cast<const uint4 *>(&a.ranks[f >> 6]);
+    const uint64_t firsts = (static_cast<uint64_t>(r.y) << 32) | r.x;
+    const uint32_t rank = r.z + static_cast<uint32_t>(__builtin_popcountll(firsts & ((1ull << (f & 63)) - 1ull)));
+    store_int(a.labels, i, a.eb, static_cast<int64_t>(rank));
   }
 }
 
@@ -857,7 +884,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
                "shmt_relabel: scratch must be 16-byte aligned");
   char *base = static_cast<char *>(scratch);
   RlSlot *tbl = reinterpret_cast<RlSlot *>(base + l.table_off);
-  uint32_t *rank_of = reinterpret_cast<uint32_t *>(base + l.rank_off);
+  RlRanks *ranks = reinterpret_cast<RlRanks *>(base + l.rank_off);  // N / 4 bytes of the N * 4 set aside
   uint64_t *partials = reinterpret_cast<uint64_t *>(base + l.partial_off);
   const int64_t nb = (N + kRlTile - 1) / kRlTile;
   // a caller that emptied the table itself says how much of it (relabel_table)
@@ -887,9 +914,9 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   const int scanned = nb > kRlSelfPrefixTiles;
   const RlInsertArgs ins{tbl, cap, total, elem_bytes, n, path};
   const RlFirstArgs fst{tbl, cap, total, elem_bytes, n, labels_out, partials, path};
-  const RlUniqueArgs unq{total, elem_bytes, n, labels_out, partials, unique_out, rank_of, count_out, count_copy,
+  const RlUniqueArgs unq{total, elem_bytes, n, labels_out, partials, unique_out, ranks, count_out, count_copy,
                          scanned};
-  const RlLabelsArgs lab{labels_out, elem_bytes, n, rank_of};
+  const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks};
   // At most 1,024 workgroups insert, each walking its tiles in turn: random global atomics run at 20-26 G/s on
   // this part whatever the grid (a third of the rate of plain stores), and a workgroup's later tiles then find
   // the ids of hub nodes already in the table with a smaller index and skip their atomics, where 8,192
