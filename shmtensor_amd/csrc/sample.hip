@@ -72,9 +72,18 @@ struct PlanArgs {
 
 // Number of seeds a kernel works on: the host's figure, or the device-side
 // count clamped to it.
+// A value every lane holds alike (loaded from one address), moved to scalar registers: what is compared
+// with it, counted up to it or fed from it into the random number generator then stays scalar too. (The
+// pick kernel needed 104 vector registers with its seed count and RNG seed in vector registers and 73 so.)
+__device__ __forceinline__ int64_t wave_uniform(int64_t v) {
+  const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint64_t>(v))));
+  const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(static_cast<uint64_t>(v) >> 32)));
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 __device__ __forceinline__ int64_t seed_count(int64_t bound, const int64_t *len) {
   if (!len) return bound;
-  const int64_t n = *len;
+  const int64_t n = wave_uniform(*len);
   return n < 0 ? 0 : (n < bound ? n : bound);
 }
 
@@ -489,7 +498,8 @@ __device__ __forceinline__ void pick_narrow_body(unsigned bx, unsigned gx, const
   const int rounds = a.rounds;
   const int per_pass = rounds * kGroups;  // <= 64 and a divisor of kPlanBlock
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
-  const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
+  const uint64_t rng_seed =
+      HOP && a.rng_seed_dev ? static_cast<uint64_t>(wave_uniform(static_cast<int64_t>(*a.rng_seed_dev))) : a.rng_seed;
   if (HOP) pick_publish_total(a, S, bx);
 
   for (int64_t w0 = wave * per_pass; w0 < S; w0 += nwaves * per_pass) {
@@ -583,7 +593,8 @@ __global__ __launch_bounds__(64) void pick_wide_kernel(PickArgs a) {
   const int lane = threadIdx.x;
   const int64_t k = a.k;
   const int64_t S = HOP ? seed_count(a.S, a.S_len) : a.S;
-  const uint64_t rng_seed = HOP && a.rng_seed_dev ? *a.rng_seed_dev : a.rng_seed;
+  const uint64_t rng_seed =
+      HOP && a.rng_seed_dev ? static_cast<uint64_t>(wave_uniform(static_cast<int64_t>(*a.rng_seed_dev))) : a.rng_seed;
   if (HOP) pick_publish_total(a, S, blockIdx.x);
   for (int64_t s = blockIdx.x; s < S; s += gridDim.x) {
     const SeedPlan p = a.plan[s];
