@@ -326,6 +326,20 @@ int64_t shmt_relabel_wide_scratch_bytes(int64_t N);
 int shmt_relabel_wide(const void *total, int64_t N, void *scratch,
                       int64_t scratch_bytes, void *unique_out,
                       void *labels_out, int64_t *count_out, void *stream);
+/* How large inputs are relabelled (no counterpart in the reference, whose
+ * four passes all probe one table in memory, src/tensor_relabel.cu:147-203).
+ * From partition_min_ids ids on (and up to 2^26) the first-occurrence index of
+ * every id is found by partitioning the ids by hash and giving every
+ * partition a table in LDS, which reads and writes memory in streams instead
+ * of touching one random line per id and pass; results are identical.
+ * partition_min_ids <= 0 restores the default (2,097,153: inputs whose tile
+ * counts need a scan launch of their own). lds_slots_log2 (0 = default, 14)
+ * and max_rounds_log2 (-1 = default, 10) shrink a partition's table and the
+ * number of rounds a partition may take before all pairs of its ids are
+ * compared; they exist so that tests can drive those rare paths. Process-wide,
+ * not synchronised with calls in flight on other threads.                    */
+int shmt_relabel_tuning(int64_t partition_min_ids, int lds_slots_log2,
+                        int max_rounds_log2);
 /* Same, with the concatenation of the caller's tensors (torch::cat,
  * src/tensor_relabel.cu:131) done on the way in: nseg <= SHMT_RELABEL_MAX_SEGMENTS
  * segments seg_ptrs[s] of seg_lens[s] ids, seg_bytes[s] in {4,8} wide, are

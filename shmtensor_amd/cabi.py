@@ -51,6 +51,7 @@ SIGNATURES = {
     "shmt_relabel": (_int, [_vp, _i64, _int, _vp, _i64, _vp, _vp, _vp, _vp]),
     "shmt_relabel_wide_scratch_bytes": (_i64, [_i64]),
     "shmt_relabel_wide": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp]),
+    "shmt_relabel_tuning": (_int, [_i64, _int, _int]),
     "shmt_relabel_segments": (_int, [_c.POINTER(_vp), _c.POINTER(_i64), _c.POINTER(_int), _int, _vp, _int, _int,
                                      _vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "shmt_sample_plan_bytes": (_i64, [_i64]),

@@ -25,6 +25,7 @@
 #include "scan_dev.h"
 
 #include <atomic>
+#include <type_traits>
 
 namespace shmt {
 
@@ -358,7 +359,8 @@ struct RlUniqueArgs {
   const void *total;
   int eb;
   RlCount n;
-  const void *labels;
+  const void *first;  // first-occurrence index of every element, fb bytes wide (the labels buffer, or an array of its own)
+  int fb;
   const uint64_t *partials;
   void *unique_out;
   RlRanks *ranks;
@@ -370,7 +372,7 @@ struct RlUniqueArgs {
 __device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &a) {
   const void *const total = a.total;
   const int eb = a.eb;
-  const void *const labels = a.labels;
+  const void *const labels = a.first;
   const uint64_t *const partials = a.partials;
   void *const unique_out = a.unique_out;
   const int64_t N = rl_count(a.n);
@@ -402,7 +404,7 @@ __device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &
     lab[j] = -1;
     val[j] = 0;
   }
-  load_ints<kRlItems>(labels, idx, ok, eb, lab);
+  load_ints<kRlItems>(labels, idx, ok, a.fb, lab);
   uint64_t firsts[kRlItems];
   uint32_t mine = 0;  // first occurrences of this wave
 #pragma unroll
@@ -450,6 +452,8 @@ struct RlLabelsArgs {
   int eb;
   RlCount n;
   const RlRanks *ranks;
+  const void *first;  // see RlUniqueArgs
+  int fb;
 };
 
 __device__ __forceinline__ void rl_labels_body(unsigned bx, unsigned gx, const RlLabelsArgs &a) {
@@ -457,7 +461,7 @@ __device__ __forceinline__ void rl_labels_body(unsigned bx, unsigned gx, const R
   int64_t i = static_cast<int64_t>(bx) * blockDim.x + threadIdx.x;
   const int64_t stride = static_cast<int64_t>(gx) * blockDim.x;
   for (; i < N; i += stride) {
-    const int64_t f = load_int(a.labels, i, a.eb);
+    const int64_t f = load_int(a.first, i, a.fb);
     const uint4 r = *reinterpret_cast<const uint4 *>(&a.ranks[f >> 6]);
     const uint64_t firsts = (static_cast<uint64_t>(r.y) << 32) | r.x;
     const uint32_t rank = r.z + static_cast<uint32_t>(__builtin_popcountll(firsts & ((1ull << (f & 63)) - 1ull)));
@@ -651,6 +655,499 @@ __global__ __launch_bounds__(kRlSmallBlock) void rl_small_jobs(Jobs<RlSmallArgs>
 __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
   if (count_copy) *count_copy = 0;
   publish_size(count_out, 0);
+}
+
+// ---- large inputs: partition by hash, one workgroup per bin, table in LDS --------
+// The insert and first-occurrence passes above touch a random line of a table
+// that no cache holds once per id and pass, and the part moves such lines at
+// 50 G per second whatever the kernel does (3.1 M ids: 74 + 54 us, plus 22 us to
+// empty the table). From kRpDefaultMin ids on the same two results -- the
+// first-occurrence index of every element and the number of first occurrences
+// per tile of kRlTile ids -- come from five passes that read and write memory
+// in runs instead:
+//   count    a workgroup per tile of kRpTile ids: histogram of the ids over P
+//            bins (bin = top bits of the id's hash), one column of the P x W
+//            matrix; ids that repeat within the tile are counted once
+//   rows     exclusive prefix along every row of the matrix, bin totals
+//   scatter  a workgroup per tile again: record {id, index} of every element
+//            to its bin's run for this tile (bins are contiguous, runs in tile
+//            order), position of the record kept per element
+//   bins     a workgroup per bin: smallest index per id through a table in
+//            LDS (the low bits of the hash address it), written per record
+//   gather   a workgroup per tile: first[i] = result of element i's record,
+//            kept in the 4-byte array that held the positions
+// Few, large bins: a tile's workgroup writes into P runs at a time, and the
+// lines of those runs have to stay in its L2 until they are full (measured on
+// 3.1 M ids, scatter / gather: 42 / 29 us with 1,024 bins, 29 / 18 us with 256).
+// P = 256 up to 4 M ids, 512 up to 8 M; larger inputs keep the table in memory.
+// A bin's table has 16,384 slots (8,192 for ids beyond 32 bits); the ids of a
+// bin that do not fit (more than that many distinct ones, or ids crafted to
+// collide) are worked through in 2, 4, ... rounds over classes of a second
+// hash, and by comparing all pairs when 2^kRpMaxRoundsLog2 rounds do not do:
+// slower, never wrong. Records are {id : 32 | index : 32} when the ids fit 32
+// bits and 16 bytes otherwise; everything lives in the memory the table in
+// memory would have had.
+constexpr int kRpBlock = 1024;
+constexpr int kRpSlotsLog2 = 14;     // 16,384 slots of 4 + 4 bytes = 128 KB of LDS
+constexpr int kRpMinBinsLog2 = 8, kRpMaxBinsLog2 = 9;
+constexpr int64_t kRpBinIds = 16384; // ids per bin from which on the number of bins grows
+constexpr int64_t kRpTile = 8192;    // ids per tile of the count / scatter / gather passes
+constexpr int kRpMaxRoundsLog2 = 10;
+constexpr int64_t kRpDefaultMin = kRlSelfPrefixTiles * kRlTile + 1;
+
+struct RpTuning {
+  int64_t min_ids;
+  int slots_log2, max_rounds_log2;
+};
+static RpTuning g_rp_tuning{kRpDefaultMin, kRpSlotsLog2, kRpMaxRoundsLog2};
+
+struct RpPlan {
+  bool ok;
+  int log2P;
+  uint32_t P, W;
+  int64_t rec_off, pos_off, firstp_off, hist_off, bintot_off, binstart_off, end;
+};
+
+// Where the partition passes keep their arrays inside the table memory (16 * cap bytes) of a
+// scratch buffer sized for N ids; ok = false when N is outside the range this path serves.
+static RpPlan rp_plan(int64_t N) {
+  RpPlan p{};
+  if (N < g_rp_tuning.min_ids || N <= kRlSmallMax) return p;
+  int lg = kRpMinBinsLog2;
+  while ((kRpBinIds << lg) < N) ++lg;
+  if (lg > kRpMaxBinsLog2) return p;
+  p.log2P = lg;
+  p.P = 1u << lg;
+  p.W = static_cast<uint32_t>((N + kRpTile - 1) / kRpTile);
+  auto up = [](int64_t x) { return (x + 255) & ~255ll; };
+  p.rec_off = 0;
+  p.pos_off = up(16 * N);
+  p.firstp_off = p.pos_off + up(4 * N);
+  p.hist_off = p.firstp_off + up(4 * N);
+  p.bintot_off = p.hist_off + up(4ll * p.P * p.W);
+  p.binstart_off = p.bintot_off + up(4ll * p.P);
+  p.end = p.binstart_off + up(4ll * (p.P + 1));
+  p.ok = p.end <= rl_capacity(N) * 16;
+  return p;
+}
+
+struct RpArgs {
+  const void *total;
+  int eb;
+  RlCount n;
+  RlPath path;
+  uint64_t *wide_mark;  // == path.wide_mark, writable: the count pass sets it itself
+  int log2P;
+  uint32_t W;
+  void *rec;
+  uint32_t *pos, *firstp, *hist, *bintot, *binstart;
+  void *labels;
+  uint64_t *partials;
+  int slots_log2, max_rounds_log2;
+};
+
+// A second hash of the id, independent of hash_id(): ids that collide there spread here.
+__device__ __forceinline__ uint32_t rp_class(int64_t key) {
+  return hash_id(static_cast<int64_t>(static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull + 0xD6E8FEB86659FD93ull));
+}
+
+constexpr int kRpItems = static_cast<int>(kRpTile / kRpBlock);  // ids a thread keeps in flight
+static_assert(kRpItems * kRpBlock == kRpTile && kRpTile % kRlTile == 0, "tiles are whole chunks of kRpTile ids");
+
+// The ids of one chunk of kRpTile, element j * kRpBlock + t for thread t: all loads issued before any is used.
+__device__ __forceinline__ void rp_load_chunk(const RpArgs &a, int64_t base, int64_t hi, int64_t (&idx)[kRpItems],
+                                              bool (&ok)[kRpItems], int64_t (&key)[kRpItems]) {
+#pragma unroll
+  for (int j = 0; j < kRpItems; ++j) {
+    idx[j] = base + j * kRpBlock + threadIdx.x;
+    ok[j] = idx[j] < hi;
+    key[j] = 0;
+  }
+  load_ints<kRpItems>(a.total, idx, ok, a.eb, key);
+}
+
+// Repeats within a tile. Ids of hub nodes come thousands of times in a sampled batch and would all land in
+// one bin; within a tile only the occurrence with the smallest index becomes a record, and the others take
+// over its position (and so its result) in the scatter pass. Found through a small direct-mapped table:
+// slot = low bits of the hash, value = {index | low 32 bits of the id} of the element with the smallest index
+// that maps there, so an id that comes often is the likely owner of its slot. An element is covered when
+// the slot names an earlier element of the same id; an id that shares its slot with an earlier one of
+// another id is simply not de-duplicated. The table's final content depends on the tile alone, so the
+// count and the scatter pass decide alike.
+constexpr int kRpDedupSlots = 2048;
+
+__device__ __forceinline__ unsigned long long rp_dedup_word(int64_t key, int64_t idx) {
+  return (static_cast<unsigned long long>(static_cast<uint32_t>(idx)) << 32) | static_cast<uint32_t>(key);
+}
+
+__device__ __forceinline__ void rp_dedup_clear(unsigned long long *dedup) {
+  for (int t = threadIdx.x; t < kRpDedupSlots; t += kRpBlock) dedup[t] = ~0ull;
+}
+
+__device__ __forceinline__ bool rp_covered(const RpArgs &a, const unsigned long long *dedup, int64_t key,
+                                           int64_t idx, uint32_t hash) {
+  const unsigned long long v = dedup[hash & (kRpDedupSlots - 1)];
+  if (static_cast<uint32_t>(v) != static_cast<uint32_t>(key) || static_cast<uint32_t>(v >> 32) == static_cast<uint32_t>(idx))
+    return false;
+  // same low half: 4-byte ids are then equal, 8-byte ids are compared in full
+  return a.eb == 4 || static_cast<const int64_t *>(a.total)[static_cast<uint32_t>(v >> 32)] == key;
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_count_kernel(RpArgs a) {
+  extern __shared__ uint32_t hist[];  // P counters
+  __shared__ unsigned long long dedup[kRpDedupSlots];
+  const int64_t N = rl_count(a.n);
+  const uint32_t P = 1u << a.log2P;
+  for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) hist[b] = 0;
+  rp_dedup_clear(dedup);
+  __syncthreads();
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
+  const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
+  int64_t idx[kRpItems], key[kRpItems];
+  bool ok[kRpItems];
+  uint32_t hash[kRpItems];
+  rp_load_chunk(a, lo, hi, idx, ok, key);
+  bool wide = false;
+#pragma unroll
+  for (int j = 0; j < kRpItems; ++j) {
+    hash[j] = hash_id(key[j]);
+    if (ok[j]) {
+      wide |= (static_cast<uint64_t>(key[j]) >> 32) != 0;
+      atomicMin(&dedup[hash[j] & (kRpDedupSlots - 1)], rp_dedup_word(key[j], idx[j]));
+    }
+  }
+  if (wide && a.path.mode == 2) *a.wide_mark = a.path.nonce;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kRpItems; ++j)
+    if (ok[j] && !rp_covered(a, dedup, key[j], idx[j], hash[j])) atomicAdd(&hist[hash[j] >> (32 - a.log2P)], 1u);
+  __syncthreads();
+  for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) a.hist[static_cast<size_t>(b) * a.W + blockIdx.x] = hist[b];
+}
+
+// One wave per bin: the row's counts become the offsets of the tiles' runs inside the bin.
+__global__ __launch_bounds__(256) void rp_rows_kernel(RpArgs a) {
+  const uint32_t b = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  if (b >= (1u << a.log2P)) return;
+  uint32_t *const row = a.hist + static_cast<size_t>(b) * a.W;
+  const uint32_t lane = lane_id();
+  uint32_t carry = 0;
+  for (uint32_t w0 = 0; w0 < a.W; w0 += kWave) {
+    const uint32_t w = w0 + lane;
+    const uint32_t v = w < a.W ? row[w] : 0u;
+    const uint32_t inc = wave_inclusive_scan(v);
+    if (w < a.W) row[w] = carry + inc - v;
+    carry += wave_last(inc);
+  }
+  if (lane == 0) a.bintot[b] = carry;
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
+  extern __shared__ uint32_t off[];  // P cursors
+  __shared__ uint32_t scan_lds[kRpBlock / kWave];
+  __shared__ unsigned long long dedup[kRpDedupSlots];
+  __shared__ uint32_t rep_pos[kRpDedupSlots];
+  const int64_t N = rl_count(a.n);
+  rp_dedup_clear(dedup);
+  const uint32_t P = 1u << a.log2P;
+  // where every bin starts: thread t sums `per` consecutive bin totals
+  const uint32_t per = P > kRpBlock ? P / kRpBlock : 1u;
+  const uint32_t b0 = threadIdx.x * per;
+  uint32_t sum = 0;
+  for (uint32_t j = 0; j < per; ++j)
+    if (b0 + j < P) sum += a.bintot[b0 + j];
+  uint32_t all;
+  uint32_t run = block_exclusive_scan<uint32_t, kRpBlock>(sum, scan_lds, &all);
+  for (uint32_t j = 0; j < per; ++j) {
+    const uint32_t b = b0 + j;
+    if (b < P) {
+      off[b] = run + a.hist[static_cast<size_t>(b) * a.W + blockIdx.x];
+      if (blockIdx.x == 0) a.binstart[b] = run;
+      run += a.bintot[b];
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) a.binstart[P] = all;
+  __syncthreads();
+  const bool packed = rl_packed(a.path);
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
+  const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
+  int64_t idx[kRpItems], key[kRpItems];
+  bool ok[kRpItems];
+  uint32_t hash[kRpItems], p[kRpItems];
+  rp_load_chunk(a, lo, hi, idx, ok, key);
+#pragma unroll
+  for (int j = 0; j < kRpItems; ++j) {
+    hash[j] = hash_id(key[j]);
+    if (ok[j]) atomicMin(&dedup[hash[j] & (kRpDedupSlots - 1)], rp_dedup_word(key[j], idx[j]));
+  }
+  __syncthreads();
+  bool covered[kRpItems];
+#pragma unroll
+  for (int j = 0; j < kRpItems; ++j) {
+    covered[j] = ok[j] && rp_covered(a, dedup, key[j], idx[j], hash[j]);
+    if (ok[j] && !covered[j]) {
+      p[j] = atomicAdd(&off[hash[j] >> (32 - a.log2P)], 1u);
+      // the element a slot names tells the ones it covers where its record went
+      if (dedup[hash[j] & (kRpDedupSlots - 1)] == rp_dedup_word(key[j], idx[j])) rep_pos[hash[j] & (kRpDedupSlots - 1)] = p[j];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kRpItems; ++j) {
+    if (!ok[j]) continue;
+    if (covered[j]) {
+      a.pos[idx[j]] = rep_pos[hash[j] & (kRpDedupSlots - 1)];
+      continue;
+    }
+    if (packed)
+      static_cast<unsigned long long *>(a.rec)[p[j]] =
+          (static_cast<unsigned long long>(static_cast<uint32_t>(key[j])) << 32) | static_cast<uint32_t>(idx[j]);
+    else
+      static_cast<uint4 *>(a.rec)[p[j]] =
+          make_uint4(static_cast<uint32_t>(static_cast<uint64_t>(key[j])),
+                     static_cast<uint32_t>(static_cast<uint64_t>(key[j]) >> 32), static_cast<uint32_t>(idx[j]), 0u);
+    a.pos[idx[j]] = p[j];
+  }
+}
+
+// The table of a bin: ids in the first part of the memory, claimed by a compare-and-swap, and the smallest
+// index seen for each behind them, lowered by an atomic minimum after a look (32-bit atomics, which the LDS
+// executes several times faster than 64-bit ones: a table of {id : 32 | index : 32} words under one 64-bit
+// atomic minimum per id measured 12 us per bin of 12,000 records for the inserts alone). Ids that fit 32 bits
+// are kept as such (16,384 slots in 128 KB), others in full (8,192 slots in 96 KB). The id that looks like
+// an empty slot (all ones) is kept in a word of its own.
+template <bool PACKED>
+struct RpTable {
+  using Key = typename std::conditional<PACKED, uint32_t, unsigned long long>::type;
+  static constexpr Key kEmpty = static_cast<Key>(~0ull);
+  Key *keys;
+  uint32_t *index;
+  uint32_t *all_ones;  // smallest index of the id kEmpty
+  uint32_t mask;       // slots - 1
+
+  __device__ __forceinline__ void clear() const {
+    for (uint32_t t = threadIdx.x; t <= mask; t += kRpBlock) {
+      keys[t] = kEmpty;
+      index[t] = 0xFFFFFFFFu;
+    }
+    if (threadIdx.x == 0) *all_ones = 0xFFFFFFFFu;
+  }
+
+  // From slot p on (key != kEmpty).
+  __device__ __forceinline__ bool insert_from(Key key, uint32_t i, uint32_t p) const {
+    p &= mask;
+    for (uint32_t probes = 0; probes <= mask; ++probes) {
+      Key k = keys[p];
+      if (k == kEmpty) k = atomicCAS(&keys[p], kEmpty, key);
+      if (k == kEmpty || k == key) {
+        if (index[p] > i) atomicMin(&index[p], i);
+        return true;
+      }
+      p = (p + 1) & mask;
+    }
+    return false;
+  }
+
+  __device__ __forceinline__ uint32_t first_from(Key key, uint32_t p) const {
+    p &= mask;
+    for (uint32_t probes = 0; probes <= mask; ++probes) {
+      if (keys[p] == key) return index[p];
+      p = (p + 1) & mask;
+    }
+    return 0xFFFFFFFFu;  // cannot happen: every id was inserted
+  }
+};
+
+template <bool PACKED>
+struct RpRecord {
+  int64_t key;
+  uint32_t i;
+  __device__ __forceinline__ void load(const void *rec, uint32_t at) {
+    if (PACKED) {
+      const unsigned long long r = static_cast<const unsigned long long *>(rec)[at];
+      key = static_cast<int64_t>(r >> 32);
+      i = static_cast<uint32_t>(r);
+    } else {
+      const uint4 r = static_cast<const uint4 *>(rec)[at];
+      key = static_cast<int64_t>((static_cast<uint64_t>(r.y) << 32) | r.x);
+      i = r.z;
+    }
+  }
+};
+
+constexpr int kRpBinItems = 8;  // records a thread has in flight while it walks over a bin
+
+// A bin whose ids do not fit its table is worked through in 2, 4, ... rounds over classes of its ids (bits
+// of the second hash).
+__device__ __forceinline__ bool rp_mine(int64_t key, uint32_t round_mask, uint32_t round) {
+  return round_mask == 0 || (rp_class(key) & round_mask) == round;
+}
+
+// kRpBinItems records of a bin, element e0 + j * kRpBlock for j = 0 .., all loads in flight together.
+template <bool PACKED>
+__device__ __forceinline__ void rp_load_records(const RpArgs &a, uint32_t start, uint32_t cnt, uint32_t e0,
+                                                uint32_t round_mask, uint32_t round,
+                                                RpRecord<PACKED> (&rec)[kRpBinItems], uint32_t (&hash)[kRpBinItems],
+                                                bool (&on)[kRpBinItems]) {
+#pragma unroll
+  for (int j = 0; j < kRpBinItems; ++j) {
+    rec[j].key = 0;
+    rec[j].i = 0;
+    on[j] = e0 + j * kRpBlock < cnt;
+    if (on[j]) rec[j].load(a.rec, start + e0 + j * kRpBlock);
+  }
+#pragma unroll
+  for (int j = 0; j < kRpBinItems; ++j) {
+    hash[j] = hash_id(rec[j].key);
+    on[j] = on[j] && rp_mine(rec[j].key, round_mask, round);
+  }
+}
+
+template <bool PACKED>
+__device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long *mem, uint32_t *shared_words) {
+  using Table = RpTable<PACKED>;
+  using Key = typename Table::Key;
+  const uint32_t start = a.binstart[blockIdx.x];
+  const uint32_t cnt = a.binstart[blockIdx.x + 1] - start;
+  if (cnt == 0) return;
+  uint32_t *const overflow = &shared_words[0];
+  const uint32_t slots = PACKED ? (1u << a.slots_log2) : (1u << (a.slots_log2 - 1));
+  Key *const keys = reinterpret_cast<Key *>(mem);
+  const Table tbl{keys, reinterpret_cast<uint32_t *>(keys + slots), &shared_words[1], slots - 1};
+  for (int lg = 0; lg <= a.max_rounds_log2; ++lg) {
+    const uint32_t round_mask = (1u << lg) - 1u;
+    bool done = true;
+    for (uint32_t r = 0; r <= round_mask && done; ++r) {
+      tbl.clear();
+      if (threadIdx.x == 0) *overflow = 0;
+      __syncthreads();
+      bool fits = true;
+      for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * kRpBlock) {
+        RpRecord<PACKED> rec[kRpBinItems];
+        uint32_t hash[kRpBinItems];
+        bool on[kRpBinItems];
+        rp_load_records<PACKED>(a, start, cnt, e0, round_mask, r, rec, hash, on);
+        // the home slots of all records are looked at together, then claimed together, then their indices
+        // looked at and lowered together; only a record that met another id goes on along its probe sequence
+        Key k[kRpBinItems];
+        uint32_t cur[kRpBinItems];
+#pragma unroll
+        for (int j = 0; j < kRpBinItems; ++j) {
+          const Key key = static_cast<Key>(rec[j].key);
+          if (on[j] && key == Table::kEmpty) {
+            atomicMin(tbl.all_ones, rec[j].i);
+            on[j] = false;
+          }
+          k[j] = on[j] ? tbl.keys[hash[j] & tbl.mask] : static_cast<Key>(0);
+        }
+#pragma unroll
+        for (int j = 0; j < kRpBinItems; ++j)
+          if (on[j] && k[j] == Table::kEmpty)
+            k[j] = atomicCAS(&tbl.keys[hash[j] & tbl.mask], Table::kEmpty, static_cast<Key>(rec[j].key));
+#pragma unroll
+        for (int j = 0; j < kRpBinItems; ++j) {
+          const bool home = on[j] && (k[j] == Table::kEmpty || k[j] == static_cast<Key>(rec[j].key));
+          if (on[j] && !home) {
+            fits &= tbl.insert_from(static_cast<Key>(rec[j].key), rec[j].i, hash[j] + 1);
+            on[j] = false;
+          }
+          cur[j] = home ? tbl.index[hash[j] & tbl.mask] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kRpBinItems; ++j)
+          if (on[j] && cur[j] > rec[j].i) atomicMin(&tbl.index[hash[j] & tbl.mask], rec[j].i);
+      }
+      if (!fits) *overflow = 1;
+      __syncthreads();
+      done = *overflow == 0;
+      if (done) {
+        for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * kRpBlock) {
+          RpRecord<PACKED> rec[kRpBinItems];
+          uint32_t hash[kRpBinItems];
+          bool on[kRpBinItems];
+          rp_load_records<PACKED>(a, start, cnt, e0, round_mask, r, rec, hash, on);
+          Key k[kRpBinItems];
+          uint32_t f[kRpBinItems];
+#pragma unroll
+          for (int j = 0; j < kRpBinItems; ++j) {
+            k[j] = on[j] ? tbl.keys[hash[j] & tbl.mask] : static_cast<Key>(0);
+            f[j] = on[j] ? tbl.index[hash[j] & tbl.mask] : 0u;
+          }
+#pragma unroll
+          for (int j = 0; j < kRpBinItems; ++j) {
+            if (!on[j]) continue;
+            const Key key = static_cast<Key>(rec[j].key);
+            if (key == Table::kEmpty)
+              f[j] = *tbl.all_ones;
+            else if (k[j] != key)
+              f[j] = tbl.first_from(key, hash[j] + 1);
+            a.firstp[start + e0 + j * kRpBlock] = f[j];
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (done) return;
+  }
+  // every pair: the ids of this bin defeat both hashes
+  for (uint32_t e = threadIdx.x; e < cnt; e += kRpBlock) {
+    RpRecord<PACKED> mine;
+    mine.load(a.rec, start + e);
+    uint32_t first = mine.i;
+    for (uint32_t o = 0; o < cnt; ++o) {
+      RpRecord<PACKED> other;
+      other.load(a.rec, start + o);
+      if (other.key == mine.key && other.i < first) first = other.i;
+    }
+    a.firstp[start + e] = first;
+  }
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_bins_kernel(RpArgs a) {
+  __shared__ unsigned long long mem[1 << kRpSlotsLog2];
+  __shared__ uint32_t shared_words[2];
+  if (rl_packed(a.path))
+    rp_bin_body<true>(a, mem, shared_words);
+  else
+    rp_bin_body<false>(a, mem, shared_words);
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) {
+  __shared__ uint32_t firsts[kRpTile / kRlTile];
+  const int64_t N = rl_count(a.n);
+  const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
+  if (lo >= N) return;
+  const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
+  const int sub_tiles = static_cast<int>(kRpTile / kRlTile);
+  for (int t = threadIdx.x; t < sub_tiles; t += kRpBlock) firsts[t] = 0;
+  __syncthreads();
+  for (int64_t base = lo; base < hi; base += kRpTile) {
+    uint32_t p[kRpItems], f[kRpItems];
+#pragma unroll
+    for (int j = 0; j < kRpItems; ++j) {
+      const int64_t i = base + j * kRpBlock + threadIdx.x;
+      p[j] = i < hi ? a.pos[i] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < kRpItems; ++j) {
+      const int64_t i = base + j * kRpBlock + threadIdx.x;
+      f[j] = i < hi ? a.firstp[p[j]] : 0xFFFFFFFFu;
+    }
+#pragma unroll
+    for (int j = 0; j < kRpItems; ++j) {
+      const int64_t i = base + j * kRpBlock + threadIdx.x;
+      if (i < hi) a.pos[i] = f[j];  // the record's position is not needed any more: the slot takes the result
+      // a wave's 64 elements lie in one tile of kRlTile ids
+      const uint64_t wins = __builtin_amdgcn_ballot_w64(i < hi && f[j] == static_cast<uint32_t>(i));
+      if (lane_id() == 0 && wins)
+        atomicAdd(&firsts[(i - lo) / kRlTile], static_cast<uint32_t>(__builtin_popcountll(wins)));
+    }
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < sub_tiles; t += kRpBlock) {
+    const int64_t tile = lo / kRlTile + t;
+    if (tile * kRlTile < N) a.partials[tile] = firsts[t];
+  }
 }
 
 // A value no earlier call has used (and that uninitialised memory is unlikely to hold).
@@ -912,11 +1409,55 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
 
   int rc = SHMT_OK;
   const int scanned = nb > kRlSelfPrefixTiles;
+  const RpPlan rp = rp_plan(N);
+  if (rp.ok && defer) {
+    defer->mergeable = false;
+    return SHMT_OK;
+  }
+  if (rp.ok) {
+    // 8-byte ids: the count pass looks at every id itself, so it can vouch for them like the kernels of a
+    // fused hop do (and an earlier kernel that stored the mark already is just as good)
+    if (path.mode == 0) path.mode = 2;
+    RpArgs a{total, elem_bytes, n, path, wide_mark, rp.log2P, rp.W, base + rp.rec_off,
+             reinterpret_cast<uint32_t *>(base + rp.pos_off), reinterpret_cast<uint32_t *>(base + rp.firstp_off),
+             reinterpret_cast<uint32_t *>(base + rp.hist_off), reinterpret_cast<uint32_t *>(base + rp.bintot_off),
+             reinterpret_cast<uint32_t *>(base + rp.binstart_off), labels_out, partials,
+             g_rp_tuning.slots_log2, g_rp_tuning.max_rounds_log2};
+    if (segs && !prepared) {
+      // concatenation only: there is no table to empty
+      hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(N, 256 * 4)), dim3(256), 0, s,
+                         static_cast<uint4 *>(nullptr), static_cast<int64_t>(0), *segs, const_cast<void *>(total),
+                         elem_bytes, n, wide_mark, nonce);
+      SHMT_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(rp_count_kernel, dim3(rp.W), dim3(kRpBlock), rp.P * sizeof(uint32_t), s, a);
+    SHMT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(rp_rows_kernel, dim3((rp.P + 3) / 4), dim3(256), 0, s, a);
+    SHMT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(rp_scatter_kernel, dim3(rp.W), dim3(kRpBlock), rp.P * sizeof(uint32_t), s, a);
+    SHMT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(rp_bins_kernel, dim3(rp.P), dim3(kRpBlock), 0, s, a);
+    SHMT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(rp_gather_kernel, dim3(rp.W), dim3(kRpBlock), 0, s, a);
+    SHMT_LAUNCH_CHECK();
+    if (scanned) {
+      rc = launch_scan_partials(partials, nb, s);
+      if (rc) return rc;
+    }
+    const RlUniqueArgs unq{total, elem_bytes, n, a.pos, 4, partials, unique_out, ranks, count_out, count_copy,
+                           scanned};
+    const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, a.pos, 4};
+    hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, unq);
+    SHMT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, lab);
+    SHMT_LAUNCH_CHECK();
+    return SHMT_OK;
+  }
   const RlInsertArgs ins{tbl, cap, total, elem_bytes, n, path};
   const RlFirstArgs fst{tbl, cap, total, elem_bytes, n, labels_out, partials, path};
-  const RlUniqueArgs unq{total, elem_bytes, n, labels_out, partials, unique_out, ranks, count_out, count_copy,
-                         scanned};
-  const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks};
+  const RlUniqueArgs unq{total, elem_bytes, n, labels_out, elem_bytes, partials, unique_out, ranks, count_out,
+                         count_copy, scanned};
+  const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, labels_out, elem_bytes};
   // At most 1,024 workgroups insert, each walking its tiles in turn: random global atomics run at 20-26 G/s on
   // this part whatever the grid (a third of the rate of plain stores), and a workgroup's later tiles then find
   // the ids of hub nodes already in the table with a smaller index and skip their atomics, where 8,192
@@ -978,7 +1519,8 @@ int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scrat
   // chained hop sized for every seed the hop before could have produced, typically three times what
   // it did produce) half the slots are used: still one 16-byte slot per id in the worst case, and
   // half as much to empty.
-  out->n16 = N <= kRlSmallMax ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
+  // Nor is there when the partition passes take the input (rp_plan).
+  out->n16 = (N <= kRlSmallMax || rp_plan(N).ok) ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
   out->wide_mark = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + l.flag_off);
   out->nonce = relabel_nonce();
   return SHMT_OK;
@@ -1044,6 +1586,17 @@ int shmt_relabel(const void *total, int64_t N, int elem_bytes, void *scratch,
                  void *stream) {
   return relabel_impl(total, nullptr, N, RlCount{N, nullptr, nullptr, 8, N}, elem_bytes, scratch, scratch_bytes,
                       unique_out, labels_out, count_out, Launcher{as_stream(stream), nullptr});
+}
+
+int shmt_relabel_tuning(int64_t partition_min_ids, int lds_slots_log2, int max_rounds_log2) {
+  SHMT_REQUIRE(lds_slots_log2 >= 0 && lds_slots_log2 <= kRpSlotsLog2 && lds_slots_log2 != 1,
+               "shmt_relabel_tuning: lds_slots_log2 must be 0 (default) or in [2, %d]", kRpSlotsLog2);
+  SHMT_REQUIRE(max_rounds_log2 >= -1 && max_rounds_log2 <= 20,
+               "shmt_relabel_tuning: max_rounds_log2 must be -1 (default) or in [0, 20]");
+  g_rp_tuning.min_ids = partition_min_ids <= 0 ? kRpDefaultMin : partition_min_ids;
+  g_rp_tuning.slots_log2 = lds_slots_log2 == 0 ? kRpSlotsLog2 : lds_slots_log2;
+  g_rp_tuning.max_rounds_log2 = max_rounds_log2 < 0 ? kRpMaxRoundsLog2 : max_rounds_log2;
+  return SHMT_OK;
 }
 
 int shmt_relabel_wide(const void *total, int64_t N, void *scratch, int64_t scratch_bytes, void *unique_out,

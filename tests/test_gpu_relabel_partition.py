@@ -1,0 +1,145 @@
+"""Relabel of large inputs through hash partitions with their tables in LDS: the size from
+which that form is used is lowered (shmt_relabel_tuning) so that inputs the oracle finishes
+quickly take it, through every entry point that relabels. Bit-exact against the oracle and
+against the same call with the default setting; the rare paths of a partition whose ids do
+not fit its table (rounds, all pairs) are driven by shrinking the table."""
+import numpy as np
+import pytest
+import torch
+
+from shmtensor_amd.synthetic import rmat_csr
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def tuning(cabi):
+    lib = cabi.load()
+
+    def set_(min_ids, slots_log2=0, rounds_log2=-1):
+        cabi.check(lib.shmt_relabel_tuning(min_ids, slots_log2, rounds_log2))
+
+    yield set_
+    lib.shmt_relabel_tuning(0, 0, -1)
+
+
+def _ids(kind, n, rng, dt):
+    a = rng.integers(0, max(2, n // 3), size=n).astype(np.int64)
+    if kind == "spread32":
+        a[::5] = rng.integers(0, 2**32 if dt == np.int64 else 2**31, size=a[::5].size)
+    elif kind == "wide":
+        a[1::3] += 2**40
+    elif kind == "one_wide_id_at_the_end":
+        a[-1] = 2**32
+    elif kind == "negative":
+        a[::7] = -a[::7] - 2
+    elif kind == "minus_one":
+        a[::11] = -1
+    elif kind == "hub":
+        a[rng.random(n) < 0.3] = 5
+    elif kind == "all_equal":
+        a[:] = 123456
+    elif kind == "all_distinct":
+        a = rng.permutation(n).astype(np.int64) * 3 + 1
+    elif kind == "uint32_max":
+        a[::9] = 2**32 - 1
+    return a.astype(dt)
+
+
+KINDS64 = ["spread32", "wide", "one_wide_id_at_the_end", "negative", "minus_one", "hub", "all_equal", "all_distinct",
+           "uint32_max"]
+KINDS32 = ["spread32", "negative", "hub", "all_equal", "all_distinct"]
+
+
+@pytest.mark.parametrize("n", [5462, 9000, 70_001, 600_000])
+@pytest.mark.parametrize("dt,kind", [(np.int64, k) for k in KINDS64] + [(np.int32, k) for k in KINDS32])
+def test_partitioned_relabel_matches_oracle(capi, oracle, tuning, n, dt, kind):
+    rng = np.random.default_rng(n)
+    a = _ids(kind, n, rng, dt)
+    b = rng.integers(0, max(2, n // 3), size=n // 2 + 1).astype(dt)
+    tuning(8193)
+    u, (la, lb) = capi.tensor_relabel([torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()])
+    eu, (ea, eb) = oracle.relabel([a, b])
+    assert np.array_equal(u.cpu().numpy(), eu)
+    assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
+
+
+@pytest.mark.parametrize("n", [8193, 100_000, 1_000_000])
+@pytest.mark.parametrize("bytes_,kind", [(8, "spread32"), (8, "wide"), (8, "negative"), (4, "spread32"), (4, "negative")])
+def test_c_abi_partitioned_relabel_of_one_array(cabi, oracle, tuning, n, bytes_, kind):
+    """shmt_relabel: no earlier kernel has seen the ids, the count pass decides the record format."""
+    lib = cabi.load()
+    ids = _ids(kind, n, np.random.default_rng(n + bytes_), np.int32 if bytes_ == 4 else np.int64)
+    total = torch.from_numpy(ids).cuda()
+    sbytes = lib.shmt_relabel_scratch_bytes(n)
+    outs = []
+    for min_ids in (8193, 0):
+        tuning(min_ids)
+        unique, labels = torch.full_like(total, -7), torch.full_like(total, -7)
+        scratch = torch.empty(sbytes, dtype=torch.uint8).cuda()
+        count = torch.full((1,), -1, dtype=torch.int64).cuda()
+        cabi.check(lib.shmt_relabel(total.data_ptr(), n, bytes_, scratch.data_ptr(), sbytes, unique.data_ptr(),
+                                    labels.data_ptr(), count.data_ptr(), cabi.current_stream()))
+        torch.cuda.synchronize()
+        outs.append((int(count.item()), unique.cpu().numpy(), labels.cpu().numpy()))
+    eu, (el,) = oracle.relabel([ids])
+    for cnt, unique, labels in outs:
+        assert cnt == eu.size
+        assert np.array_equal(unique[:cnt], eu) and np.array_equal(labels, el)
+
+
+@pytest.mark.parametrize("slots_log2,rounds_log2", [(6, -1), (3, -1), (4, 2), (2, 0)])
+@pytest.mark.parametrize("kind", ["spread32", "wide", "minus_one", "hub"])
+def test_partition_that_does_not_fit_its_table(capi, oracle, tuning, slots_log2, rounds_log2, kind):
+    """Tables of 64 / 8 / 16 / 4 slots for partitions of some 300 distinct ids: the partition is worked
+    through in rounds over classes of its ids, and by comparing all pairs once the rounds are used up."""
+    n = 40_000
+    rng = np.random.default_rng(slots_log2)
+    a = _ids(kind, n, rng, np.int64)
+    b = rng.integers(0, n // 3, size=n // 2).astype(np.int64)
+    tuning(8193, slots_log2, rounds_log2)
+    u, (la, lb) = capi.tensor_relabel([torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()])
+    eu, (ea, eb) = oracle.relabel([a, b])
+    assert np.array_equal(u.cpu().numpy(), eu)
+    assert np.array_equal(la.cpu().numpy(), ea) and np.array_equal(lb.cpu().numpy(), eb)
+
+
+def _same(a, b):
+    assert len(a) == len(b)
+    for x, y in zip(a, b):
+        assert x.dtype == y.dtype and x.shape == y.shape and torch.equal(x, y)
+
+
+@pytest.mark.parametrize("idx_dt", [torch.int32, torch.int64])
+def test_fused_hop_and_chained_batches_through_partitions(capi, tuning, idx_dt):
+    """The fused hop (the pick kernel writes the relabel input and would have emptied the table) and
+    sample_blocks (hops chained on the device, launches shared between batches) give what they give
+    with the default setting."""
+    indptr, indices = rmat_csr(15, 12, 3)
+    indptr, indices = indptr.cuda(), indices.to(idx_dt).cuda()
+    n = indptr.numel() - 1
+    g = torch.Generator().manual_seed(4)
+    seeds = torch.randint(0, n, (3000,), generator=g).to(idx_dt).cuda()
+    batches = [torch.randperm(n, generator=g)[:700].to(idx_dt).cuda() for _ in range(4)]
+    got = {}
+    for min_ids in (0, 8193):
+        tuning(min_ids)
+        hop = capi.sample_hop(indptr, indices, None, None, None, seeds, 10, False, seed=5)
+        blocks = capi.sample_blocks(indptr, indices, None, None, None, batches, [5, 6, 7], False,
+                                    seeds_rng=[5, 6, 7, 8], max_in_flight=4)
+        torch.cuda.synchronize()
+        got[min_ids] = (hop, blocks)
+    _same(got[0][0], got[8193][0])
+    assert len(got[0][1]) == len(got[8193][1]) == len(batches)
+    for x, y in zip(got[0][1], got[8193][1]):
+        assert len(x) == len(y) == 3
+        for hop_x, hop_y in zip(x, y):
+            _same(hop_x, hop_y)
+
+
+def test_tuning_rejects_bad_values(cabi):
+    lib = cabi.load()
+    assert lib.shmt_relabel_tuning(0, 1, -1) != 0
+    assert lib.shmt_relabel_tuning(0, 15, -1) != 0
+    assert lib.shmt_relabel_tuning(0, 0, 21) != 0
+    assert lib.shmt_relabel_tuning(0, 0, -1) == 0
