@@ -366,7 +366,9 @@ struct RlUniqueArgs {
   RlRanks *ranks;
   int64_t *count_out;
   int64_t *count_copy;
-  int scanned;
+  int scanned;             // 0: partials are raw tile counts, 1: scanned, 2: raw, with the sums of whole groups in `coarse`
+  const uint32_t *coarse;  // scanned == 2: coarse[g] = sum of the counts of tiles [g * group, (g + 1) * group)
+  int group;
 };
 
 __device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &a) {
@@ -383,11 +385,17 @@ __device__ __forceinline__ void rl_unique_body(unsigned bx, const RlUniqueArgs &
   // Tile prefix: either already scanned by a separate launch, or (few tiles)
   // summed here from the raw per-tile counts.
   uint64_t tile_prefix;
-  if (a.scanned) {
+  if (a.scanned == 1) {
     tile_prefix = partials[bx];
   } else {
     uint64_t part = 0;
-    for (int t = threadIdx.x; t < static_cast<int>(bx); t += kRlBlock) part += partials[t];
+    int from = 0;
+    if (a.scanned == 2) {
+      const int groups = static_cast<int>(bx) / a.group;
+      for (int t = threadIdx.x; t < groups; t += kRlBlock) part += a.coarse[t];
+      from = groups * a.group;
+    }
+    for (int t = from + threadIdx.x; t < static_cast<int>(bx); t += kRlBlock) part += partials[t];
     uint64_t below;
     block_exclusive_scan<uint64_t, kRlBlock>(part, lds64, &below);
     tile_prefix = below;
@@ -705,7 +713,7 @@ struct RpPlan {
   bool ok;
   int log2P;
   uint32_t P, W;
-  int64_t rec_off, pos_off, firstp_off, hist_off, bintot_off, binstart_off, end;
+  int64_t rec_off, pos_off, firstp_off, hist_off, bintot_off, binstart_off, coarse_off, end;
 };
 
 // Where the partition passes keep their arrays inside the table memory (16 * cap bytes) of a
@@ -726,7 +734,8 @@ static RpPlan rp_plan(int64_t N) {
   p.hist_off = p.firstp_off + up(4 * N);
   p.bintot_off = p.hist_off + up(4ll * p.P * p.W);
   p.binstart_off = p.bintot_off + up(4ll * p.P);
-  p.end = p.binstart_off + up(4ll * (p.P + 1));
+  p.coarse_off = p.binstart_off + up(4ll * (p.P + 1));
+  p.end = p.coarse_off + up(4ll * p.W);
   p.ok = p.end <= rl_capacity(N) * 16;
   return p;
 }
@@ -740,8 +749,7 @@ struct RpArgs {
   int log2P;
   uint32_t W;
   void *rec;
-  uint32_t *pos, *firstp, *hist, *bintot, *binstart;
-  void *labels;
+  uint32_t *pos, *firstp, *hist, *bintot, *binstart, *coarse;
   uint64_t *partials;
   int slots_log2, max_rounds_log2;
 };
@@ -1144,9 +1152,17 @@ __global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) {
     }
   }
   __syncthreads();
+  uint32_t all = 0;
   for (int t = threadIdx.x; t < sub_tiles; t += kRpBlock) {
     const int64_t tile = lo / kRlTile + t;
     if (tile * kRlTile < N) a.partials[tile] = firsts[t];
+    all += firsts[t];
+  }
+  // (one wave covers all sub-tiles) the tile's own total, so that the unique pass needs no scan of the counts
+  static_assert(kRpTile / kRlTile <= kWave, "the first wave sums a tile's counts");
+  if (threadIdx.x < kWave) {
+    all = wave_last(wave_inclusive_scan(all));
+    if (threadIdx.x == 0) a.coarse[blockIdx.x] = all;
   }
 }
 
@@ -1421,7 +1437,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     RpArgs a{total, elem_bytes, n, path, wide_mark, rp.log2P, rp.W, base + rp.rec_off,
              reinterpret_cast<uint32_t *>(base + rp.pos_off), reinterpret_cast<uint32_t *>(base + rp.firstp_off),
              reinterpret_cast<uint32_t *>(base + rp.hist_off), reinterpret_cast<uint32_t *>(base + rp.bintot_off),
-             reinterpret_cast<uint32_t *>(base + rp.binstart_off), labels_out, partials,
+             reinterpret_cast<uint32_t *>(base + rp.binstart_off), reinterpret_cast<uint32_t *>(base + rp.coarse_off), partials,
              g_rp_tuning.slots_log2, g_rp_tuning.max_rounds_log2};
     if (segs && !prepared) {
       // concatenation only: there is no table to empty
@@ -1440,12 +1456,8 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_gather_kernel, dim3(rp.W), dim3(kRpBlock), 0, s, a);
     SHMT_LAUNCH_CHECK();
-    if (scanned) {
-      rc = launch_scan_partials(partials, nb, s);
-      if (rc) return rc;
-    }
     const RlUniqueArgs unq{total, elem_bytes, n, a.pos, 4, partials, unique_out, ranks, count_out, count_copy,
-                           scanned};
+                           2, a.coarse, static_cast<int>(kRpTile / kRlTile)};
     const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, a.pos, 4};
     hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, unq);
     SHMT_LAUNCH_CHECK();
@@ -1456,7 +1468,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   const RlInsertArgs ins{tbl, cap, total, elem_bytes, n, path};
   const RlFirstArgs fst{tbl, cap, total, elem_bytes, n, labels_out, partials, path};
   const RlUniqueArgs unq{total, elem_bytes, n, labels_out, elem_bytes, partials, unique_out, ranks, count_out,
-                         count_copy, scanned};
+                         count_copy, scanned, nullptr, 1};
   const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, labels_out, elem_bytes};
   // At most 1,024 workgroups insert, each walking its tiles in turn: random global atomics run at 20-26 G/s on
   // this part whatever the grid (a third of the rate of plain stores), and a workgroup's later tiles then find
