@@ -713,7 +713,7 @@ struct RpPlan {
   bool ok;
   int log2P;
   uint32_t P, W;
-  int64_t rec_off, pos_off, firstp_off, hist_off, bintot_off, binstart_off, coarse_off, end;
+  int64_t rec_off, pos_off, firstp_off, local_off, hist_off, bintot_off, binstart_off, coarse_off, tile_off, end;
 };
 
 // Where the partition passes keep their arrays inside the table memory (16 * cap bytes) of a
@@ -731,11 +731,13 @@ static RpPlan rp_plan(int64_t N) {
   p.rec_off = 0;
   p.pos_off = up(16 * N);
   p.firstp_off = p.pos_off + up(4 * N);
-  p.hist_off = p.firstp_off + up(4 * N);
+  p.local_off = p.firstp_off + up(4 * N);
+  p.hist_off = p.local_off + up(2 * N);
   p.bintot_off = p.hist_off + up(4ll * p.P * p.W);
   p.binstart_off = p.bintot_off + up(4ll * p.P);
   p.coarse_off = p.binstart_off + up(4ll * (p.P + 1));
-  p.end = p.coarse_off + up(4ll * p.W);
+  p.tile_off = p.coarse_off + up(4ll * p.W);
+  p.end = p.tile_off + up(8ll * p.W * (p.P + 1));
   p.ok = p.end <= rl_capacity(N) * 16;
   return p;
 }
@@ -750,6 +752,8 @@ struct RpArgs {
   uint32_t W;
   void *rec;
   uint32_t *pos, *firstp, *hist, *bintot, *binstart, *coarse;
+  uint16_t *local;  // position of every element's record among its tile's records in bin order
+  uint32_t *tile_runs;  // per tile: where its run of every bin starts in memory (P words), then among its records (P + 1 words)
   uint64_t *partials;
   int slots_log2, max_rounds_log2;
 };
@@ -850,14 +854,27 @@ __global__ __launch_bounds__(256) void rp_rows_kernel(RpArgs a) {
   if (lane == 0) a.bintot[b] = carry;
 }
 
+// The id a packed record stands for, as the count pass hashed it (4-byte ids are signed).
+__device__ __forceinline__ int64_t rp_packed_key(unsigned long long rec, int eb) {
+  const uint32_t k = static_cast<uint32_t>(rec >> 32);
+  return eb == 4 ? static_cast<int64_t>(static_cast<int32_t>(k)) : static_cast<int64_t>(k);
+}
+
+// Scattered 8-byte stores cost one L2 transaction each and leave half-filled lines behind; the records of a
+// tile are therefore put in bin order in LDS first (position = start of the bin among the tile's records +
+// rank within the bin) and written out from there, consecutive lanes to consecutive addresses of a run.
+// 16-byte records (ids beyond 32 bits) do not fit the LDS and are stored directly.
 __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
-  extern __shared__ uint32_t off[];  // P cursors
+  extern __shared__ uint32_t words[];  // run start in memory, record count, start among the tile's records: P (+ 1) each
+  __shared__ unsigned long long stage[kRpTile];  // first the de-duplication table and the ranks of its owners
   __shared__ uint32_t scan_lds[kRpBlock / kWave];
-  __shared__ unsigned long long dedup[kRpDedupSlots];
-  __shared__ uint32_t rep_pos[kRpDedupSlots];
   const int64_t N = rl_count(a.n);
-  rp_dedup_clear(dedup);
   const uint32_t P = 1u << a.log2P;
+  uint32_t *const run_at = words, *const cnt = words + P, *const lstart = words + 2 * P;
+  unsigned long long *const dedup = stage;
+  uint32_t *const rep_rank = reinterpret_cast<uint32_t *>(stage + kRpDedupSlots);
+  static_assert(kRpDedupSlots * 12 <= kRpTile * 8, "table and ranks fit the staging memory");
+  rp_dedup_clear(dedup);
   // where every bin starts: thread t sums `per` consecutive bin totals
   const uint32_t per = P > kRpBlock ? P / kRpBlock : 1u;
   const uint32_t b0 = threadIdx.x * per;
@@ -869,7 +886,8 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
   for (uint32_t j = 0; j < per; ++j) {
     const uint32_t b = b0 + j;
     if (b < P) {
-      off[b] = run + a.hist[static_cast<size_t>(b) * a.W + blockIdx.x];
+      run_at[b] = run + a.hist[static_cast<size_t>(b) * a.W + blockIdx.x];
+      cnt[b] = 0;
       if (blockIdx.x == 0) a.binstart[b] = run;
       run += a.bintot[b];
     }
@@ -881,7 +899,7 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
   const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
   int64_t idx[kRpItems], key[kRpItems];
   bool ok[kRpItems];
-  uint32_t hash[kRpItems], p[kRpItems];
+  uint32_t hash[kRpItems], rank[kRpItems];
   rp_load_chunk(a, lo, hi, idx, ok, key);
 #pragma unroll
   for (int j = 0; j < kRpItems; ++j) {
@@ -893,28 +911,57 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
 #pragma unroll
   for (int j = 0; j < kRpItems; ++j) {
     covered[j] = ok[j] && rp_covered(a, dedup, key[j], idx[j], hash[j]);
+    rank[j] = 0;
     if (ok[j] && !covered[j]) {
-      p[j] = atomicAdd(&off[hash[j] >> (32 - a.log2P)], 1u);
-      // the element a slot names tells the ones it covers where its record went
-      if (dedup[hash[j] & (kRpDedupSlots - 1)] == rp_dedup_word(key[j], idx[j])) rep_pos[hash[j] & (kRpDedupSlots - 1)] = p[j];
+      rank[j] = atomicAdd(&cnt[hash[j] >> (32 - a.log2P)], 1u);
+      // the element a slot names tells the ones it covers (same id, so same bin) where its record goes
+      if (dedup[hash[j] & (kRpDedupSlots - 1)] == rp_dedup_word(key[j], idx[j])) rep_rank[hash[j] & (kRpDedupSlots - 1)] = rank[j];
     }
   }
   __syncthreads();
 #pragma unroll
+  for (int j = 0; j < kRpItems; ++j)
+    if (covered[j]) rank[j] = rep_rank[hash[j] & (kRpDedupSlots - 1)];
+  // start of every bin among the tile's records (the scan's barriers also end the use of the table)
+  {
+    uint32_t part = 0;
+    for (uint32_t j = 0; j < per; ++j)
+      if (b0 + j < P) part += cnt[b0 + j];
+    uint32_t records;
+    uint32_t at = block_exclusive_scan<uint32_t, kRpBlock>(part, scan_lds, &records);
+    for (uint32_t j = 0; j < per; ++j) {
+      const uint32_t b = b0 + j;
+      if (b < P) {
+        lstart[b] = at;
+        at += cnt[b];
+      }
+    }
+    if (threadIdx.x == 0) lstart[P] = records;
+  }
+  __syncthreads();
+  uint32_t *const runs = a.tile_runs + static_cast<size_t>(blockIdx.x) * (2 * P + 1);
+  for (uint32_t t = threadIdx.x; t < 2 * P + 1; t += kRpBlock) runs[t] = t < P ? run_at[t] : lstart[t - P];
+#pragma unroll
   for (int j = 0; j < kRpItems; ++j) {
     if (!ok[j]) continue;
-    if (covered[j]) {
-      a.pos[idx[j]] = rep_pos[hash[j] & (kRpDedupSlots - 1)];
-      continue;
-    }
+    const uint32_t bin = hash[j] >> (32 - a.log2P);
+    const uint32_t at = lstart[bin] + rank[j];
+    a.local[idx[j]] = static_cast<uint16_t>(at);
+    if (covered[j]) continue;
     if (packed)
-      static_cast<unsigned long long *>(a.rec)[p[j]] =
-          (static_cast<unsigned long long>(static_cast<uint32_t>(key[j])) << 32) | static_cast<uint32_t>(idx[j]);
+      stage[at] = (static_cast<unsigned long long>(static_cast<uint32_t>(key[j])) << 32) | static_cast<uint32_t>(idx[j]);
     else
-      static_cast<uint4 *>(a.rec)[p[j]] =
+      static_cast<uint4 *>(a.rec)[run_at[bin] + rank[j]] =
           make_uint4(static_cast<uint32_t>(static_cast<uint64_t>(key[j])),
                      static_cast<uint32_t>(static_cast<uint64_t>(key[j]) >> 32), static_cast<uint32_t>(idx[j]), 0u);
-    a.pos[idx[j]] = p[j];
+  }
+  if (!packed) return;
+  __syncthreads();
+  const uint32_t records = lstart[P];
+  for (uint32_t q = threadIdx.x; q < records; q += kRpBlock) {
+    const unsigned long long rec = stage[q];
+    const uint32_t bin = hash_id(rp_packed_key(rec, a.eb)) >> (32 - a.log2P);
+    static_cast<unsigned long long *>(a.rec)[run_at[bin] + (q - lstart[bin])] = rec;
   }
 }
 
@@ -1120,36 +1167,47 @@ __global__ __launch_bounds__(kRpBlock) void rp_bins_kernel(RpArgs a) {
     rp_bin_body<false>(a, mem, shared_words);
 }
 
+// The results of the tile's records are read run by run, consecutive lanes from consecutive addresses, into
+// LDS in the tile's bin order; every element then picks the one of its record there.
 __global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) {
+  extern __shared__ uint32_t words[];  // run start in memory (P), start among the tile's records (P + 1)
+  __shared__ uint32_t result[kRpTile];
   __shared__ uint32_t firsts[kRpTile / kRlTile];
   const int64_t N = rl_count(a.n);
   const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
   if (lo >= N) return;
   const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
+  const uint32_t P = 1u << a.log2P;
+  const uint32_t *const runs = a.tile_runs + static_cast<size_t>(blockIdx.x) * (2 * P + 1);
+  for (uint32_t t = threadIdx.x; t < 2 * P + 1; t += kRpBlock) words[t] = runs[t];
   const int sub_tiles = static_cast<int>(kRpTile / kRlTile);
   for (int t = threadIdx.x; t < sub_tiles; t += kRpBlock) firsts[t] = 0;
   __syncthreads();
-  for (int64_t base = lo; base < hi; base += kRpTile) {
-    uint32_t p[kRpItems], f[kRpItems];
+  const uint32_t *const run_at = words, *const lstart = words + P;
+  const uint32_t records = lstart[P];
+  for (uint32_t q = threadIdx.x; q < records; q += kRpBlock) {
+    // the bin whose records include the q-th: the last one that starts at or before q
+    uint32_t bin = 0;
+    for (uint32_t step = P >> 1; step > 0; step >>= 1)
+      if (lstart[bin + step] <= q) bin += step;
+    result[q] = a.firstp[run_at[bin] + (q - lstart[bin])];
+  }
+  __syncthreads();
+  uint16_t at[kRpItems];
 #pragma unroll
-    for (int j = 0; j < kRpItems; ++j) {
-      const int64_t i = base + j * kRpBlock + threadIdx.x;
-      p[j] = i < hi ? a.pos[i] : 0u;
-    }
+  for (int j = 0; j < kRpItems; ++j) {
+    const int64_t i = lo + j * kRpBlock + threadIdx.x;
+    at[j] = i < hi ? a.local[i] : static_cast<uint16_t>(0);
+  }
 #pragma unroll
-    for (int j = 0; j < kRpItems; ++j) {
-      const int64_t i = base + j * kRpBlock + threadIdx.x;
-      f[j] = i < hi ? a.firstp[p[j]] : 0xFFFFFFFFu;
-    }
-#pragma unroll
-    for (int j = 0; j < kRpItems; ++j) {
-      const int64_t i = base + j * kRpBlock + threadIdx.x;
-      if (i < hi) a.pos[i] = f[j];  // the record's position is not needed any more: the slot takes the result
-      // a wave's 64 elements lie in one tile of kRlTile ids
-      const uint64_t wins = __builtin_amdgcn_ballot_w64(i < hi && f[j] == static_cast<uint32_t>(i));
-      if (lane_id() == 0 && wins)
-        atomicAdd(&firsts[(i - lo) / kRlTile], static_cast<uint32_t>(__builtin_popcountll(wins)));
-    }
+  for (int j = 0; j < kRpItems; ++j) {
+    const int64_t i = lo + j * kRpBlock + threadIdx.x;
+    const uint32_t f = i < hi ? result[at[j]] : 0xFFFFFFFFu;
+    if (i < hi) a.pos[i] = f;
+    // a wave's 64 elements lie in one tile of kRlTile ids
+    const uint64_t wins = __builtin_amdgcn_ballot_w64(i < hi && f == static_cast<uint32_t>(i));
+    if (lane_id() == 0 && wins)
+      atomicAdd(&firsts[(i - lo) / kRlTile], static_cast<uint32_t>(__builtin_popcountll(wins)));
   }
   __syncthreads();
   uint32_t all = 0;
@@ -1437,7 +1495,8 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     RpArgs a{total, elem_bytes, n, path, wide_mark, rp.log2P, rp.W, base + rp.rec_off,
              reinterpret_cast<uint32_t *>(base + rp.pos_off), reinterpret_cast<uint32_t *>(base + rp.firstp_off),
              reinterpret_cast<uint32_t *>(base + rp.hist_off), reinterpret_cast<uint32_t *>(base + rp.bintot_off),
-             reinterpret_cast<uint32_t *>(base + rp.binstart_off), reinterpret_cast<uint32_t *>(base + rp.coarse_off), partials,
+             reinterpret_cast<uint32_t *>(base + rp.binstart_off), reinterpret_cast<uint32_t *>(base + rp.coarse_off), reinterpret_cast<uint16_t *>(base + rp.local_off),
+             reinterpret_cast<uint32_t *>(base + rp.tile_off), partials,
              g_rp_tuning.slots_log2, g_rp_tuning.max_rounds_log2};
     if (segs && !prepared) {
       // concatenation only: there is no table to empty
@@ -1450,11 +1509,11 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_rows_kernel, dim3((rp.P + 3) / 4), dim3(256), 0, s, a);
     SHMT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(rp_scatter_kernel, dim3(rp.W), dim3(kRpBlock), rp.P * sizeof(uint32_t), s, a);
+    hipLaunchKernelGGL(rp_scatter_kernel, dim3(rp.W), dim3(kRpBlock), (3 * rp.P + 1) * sizeof(uint32_t), s, a);
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_bins_kernel, dim3(rp.P), dim3(kRpBlock), 0, s, a);
     SHMT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(rp_gather_kernel, dim3(rp.W), dim3(kRpBlock), 0, s, a);
+    hipLaunchKernelGGL(rp_gather_kernel, dim3(rp.W), dim3(kRpBlock), (2 * rp.P + 1) * sizeof(uint32_t), s, a);
     SHMT_LAUNCH_CHECK();
     const RlUniqueArgs unq{total, elem_bytes, n, a.pos, 4, partials, unique_out, ranks, count_out, count_copy,
                            2, a.coarse, static_cast<int>(kRpTile / kRlTile)};
