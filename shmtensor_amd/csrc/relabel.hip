@@ -19,7 +19,9 @@
 // the id, src/tensor_relabel.cu:111-117); ids known to fit 32 bits use the
 // same memory as packed 8-byte slots (see rl_packed_insert).
 // Up to 8,192 ids all of this is one launch of one workgroup with its table
-// in LDS (rl_small_kernel).
+// in LDS (rl_small_kernel). Beyond 2 M ids (and up to 8 M) fill, insert and
+// first are replaced by passes that partition the ids by hash and give every
+// partition a table in LDS (rp_*_kernel, further down).
 #include "common.h"
 #include "launchers.h"
 #include "scan_dev.h"
@@ -679,14 +681,16 @@ __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
 //   rows     exclusive prefix along every row of the matrix, bin totals
 //   scatter  a workgroup per tile again: record {id, index} of every element
 //            to its bin's run for this tile (bins are contiguous, runs in tile
-//            order), position of the record kept per element
+//            order), through LDS so that a run is written by consecutive
+//            lanes; per element the place of its record among the tile's
 //   bins     a workgroup per bin: smallest index per id through a table in
 //            LDS (the low bits of the hash address it), written per record
-//   gather   a workgroup per tile: first[i] = result of element i's record,
-//            kept in the 4-byte array that held the positions
-// Few, large bins: a tile's workgroup writes into P runs at a time, and the
-// lines of those runs have to stay in its L2 until they are full (measured on
-// 3.1 M ids, scatter / gather: 42 / 29 us with 1,024 bins, 29 / 18 us with 256).
+//   gather   a workgroup per tile: the results of its runs, read through LDS
+//            the same way, handed to the elements: first[i], 4 bytes each
+// Few, large bins: a tile's run for a bin should span whole lines (8,192 ids
+// over 256 bins: 32 records; measured on 3.1 M ids, scatter / gather 24 / 14 us
+// with 256 bins, 31 / 17 us with 1,024, and 42 / 29 us before the runs went
+// through LDS).
 // P = 256 up to 4 M ids, 512 up to 8 M; larger inputs keep the table in memory.
 // A bin's table has 16,384 slots (8,192 for ids beyond 32 bits); the ids of a
 // bin that do not fit (more than that many distinct ones, or ids crafted to
@@ -713,7 +717,7 @@ struct RpPlan {
   bool ok;
   int log2P;
   uint32_t P, W;
-  int64_t rec_off, pos_off, firstp_off, local_off, hist_off, bintot_off, binstart_off, coarse_off, tile_off, end;
+  int64_t rec_off, first_off, firstp_off, local_off, hist_off, bintot_off, binstart_off, coarse_off, tile_off, end;
 };
 
 // Where the partition passes keep their arrays inside the table memory (16 * cap bytes) of a
@@ -729,8 +733,8 @@ static RpPlan rp_plan(int64_t N) {
   p.W = static_cast<uint32_t>((N + kRpTile - 1) / kRpTile);
   auto up = [](int64_t x) { return (x + 255) & ~255ll; };
   p.rec_off = 0;
-  p.pos_off = up(16 * N);
-  p.firstp_off = p.pos_off + up(4 * N);
+  p.first_off = up(16 * N);
+  p.firstp_off = p.first_off + up(4 * N);
   p.local_off = p.firstp_off + up(4 * N);
   p.hist_off = p.local_off + up(2 * N);
   p.bintot_off = p.hist_off + up(4ll * p.P * p.W);
@@ -751,7 +755,9 @@ struct RpArgs {
   int log2P;
   uint32_t W;
   void *rec;
-  uint32_t *pos, *firstp, *hist, *bintot, *binstart, *coarse;
+  uint32_t *first;   // first-occurrence index of every element (what the unique and labels passes read)
+  uint32_t *firstp;  // the same per record, in the records' order
+  uint32_t *hist, *bintot, *binstart, *coarse;
   uint16_t *local;  // position of every element's record among its tile's records in bin order
   uint32_t *tile_runs;  // per tile: where its run of every bin starts in memory (P words), then among its records (P + 1 words)
   uint64_t *partials;
@@ -965,25 +971,43 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
   }
 }
 
-// The table of a bin: ids in the first part of the memory, claimed by a compare-and-swap, and the smallest
-// index seen for each behind them, lowered by an atomic minimum after a look (32-bit atomics, which the LDS
-// executes several times faster than 64-bit ones: a table of {id : 32 | index : 32} words under one 64-bit
-// atomic minimum per id measured 12 us per bin of 12,000 records for the inserts alone). Ids that fit 32 bits
-// are kept as such (16,384 slots in 128 KB), others in full (8,192 slots in 96 KB). The id that looks like
-// an empty slot (all ones) is kept in a word of its own.
+// The table of a bin: per slot an id, claimed by a compare-and-swap, and the smallest index seen for it,
+// lowered by an atomic minimum after a look (32-bit atomics, which the LDS executes several times faster than
+// 64-bit ones: slots {id : 32 | index : 32} under one 64-bit atomic minimum per id measured 12 us per bin of
+// 12,000 records for the inserts alone). Ids that fit 32 bits are kept as such, next to their index, so
+// that one 8-byte read shows both (16,384 slots in 128 KB); others in full, in an array in front of the
+// indices (8,192 slots in 96 KB). The id that looks like an empty slot (all ones) is kept in a word of its own.
 template <bool PACKED>
 struct RpTable {
   using Key = typename std::conditional<PACKED, uint32_t, unsigned long long>::type;
   static constexpr Key kEmpty = static_cast<Key>(~0ull);
-  Key *keys;
-  uint32_t *index;
+  unsigned long long *mem;
   uint32_t *all_ones;  // smallest index of the id kEmpty
   uint32_t mask;       // slots - 1
 
+  __device__ __forceinline__ Key *key_at(uint32_t p) const {
+    if (PACKED) return reinterpret_cast<Key *>(reinterpret_cast<uint32_t *>(mem) + 2 * p);
+    return reinterpret_cast<Key *>(mem) + p;
+  }
+  __device__ __forceinline__ uint32_t *index_at(uint32_t p) const {
+    if (PACKED) return reinterpret_cast<uint32_t *>(mem) + 2 * p + 1;
+    return reinterpret_cast<uint32_t *>(mem + mask + 1) + p;
+  }
+  __device__ __forceinline__ void look(uint32_t p, Key *key, uint32_t *index) const {
+    if (PACKED) {
+      const unsigned long long both = mem[p];
+      *key = static_cast<Key>(static_cast<uint32_t>(both));
+      *index = static_cast<uint32_t>(both >> 32);
+    } else {
+      *key = *key_at(p);
+      *index = *index_at(p);
+    }
+  }
+
   __device__ __forceinline__ void clear() const {
     for (uint32_t t = threadIdx.x; t <= mask; t += kRpBlock) {
-      keys[t] = kEmpty;
-      index[t] = 0xFFFFFFFFu;
+      mem[t] = ~0ull;
+      if (!PACKED) *index_at(t) = 0xFFFFFFFFu;
     }
     if (threadIdx.x == 0) *all_ones = 0xFFFFFFFFu;
   }
@@ -992,10 +1016,12 @@ struct RpTable {
   __device__ __forceinline__ bool insert_from(Key key, uint32_t i, uint32_t p) const {
     p &= mask;
     for (uint32_t probes = 0; probes <= mask; ++probes) {
-      Key k = keys[p];
-      if (k == kEmpty) k = atomicCAS(&keys[p], kEmpty, key);
+      Key k;
+      uint32_t cur;
+      look(p, &k, &cur);
+      if (k == kEmpty) k = atomicCAS(key_at(p), kEmpty, key);
       if (k == kEmpty || k == key) {
-        if (index[p] > i) atomicMin(&index[p], i);
+        if (cur > i) atomicMin(index_at(p), i);  // a look that is out of date can only show a larger index
         return true;
       }
       p = (p + 1) & mask;
@@ -1006,7 +1032,10 @@ struct RpTable {
   __device__ __forceinline__ uint32_t first_from(Key key, uint32_t p) const {
     p &= mask;
     for (uint32_t probes = 0; probes <= mask; ++probes) {
-      if (keys[p] == key) return index[p];
+      Key k;
+      uint32_t cur;
+      look(p, &k, &cur);
+      if (k == key) return cur;
       p = (p + 1) & mask;
     }
     return 0xFFFFFFFFu;  // cannot happen: every id was inserted
@@ -1067,8 +1096,7 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
   if (cnt == 0) return;
   uint32_t *const overflow = &shared_words[0];
   const uint32_t slots = PACKED ? (1u << a.slots_log2) : (1u << (a.slots_log2 - 1));
-  Key *const keys = reinterpret_cast<Key *>(mem);
-  const Table tbl{keys, reinterpret_cast<uint32_t *>(keys + slots), &shared_words[1], slots - 1};
+  const Table tbl{mem, &shared_words[1], slots - 1};
   for (int lg = 0; lg <= a.max_rounds_log2; ++lg) {
     const uint32_t round_mask = (1u << lg) - 1u;
     bool done = true;
@@ -1093,24 +1121,23 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
             atomicMin(tbl.all_ones, rec[j].i);
             on[j] = false;
           }
-          k[j] = on[j] ? tbl.keys[hash[j] & tbl.mask] : static_cast<Key>(0);
+          k[j] = 0;
+          cur[j] = 0;
+          if (on[j]) tbl.look(hash[j] & tbl.mask, &k[j], &cur[j]);
         }
 #pragma unroll
         for (int j = 0; j < kRpBinItems; ++j)
           if (on[j] && k[j] == Table::kEmpty)
-            k[j] = atomicCAS(&tbl.keys[hash[j] & tbl.mask], Table::kEmpty, static_cast<Key>(rec[j].key));
+            k[j] = atomicCAS(tbl.key_at(hash[j] & tbl.mask), Table::kEmpty, static_cast<Key>(rec[j].key));
 #pragma unroll
         for (int j = 0; j < kRpBinItems; ++j) {
-          const bool home = on[j] && (k[j] == Table::kEmpty || k[j] == static_cast<Key>(rec[j].key));
-          if (on[j] && !home) {
+          if (!on[j]) continue;
+          if (k[j] == Table::kEmpty || k[j] == static_cast<Key>(rec[j].key)) {
+            if (cur[j] > rec[j].i) atomicMin(tbl.index_at(hash[j] & tbl.mask), rec[j].i);
+          } else {
             fits &= tbl.insert_from(static_cast<Key>(rec[j].key), rec[j].i, hash[j] + 1);
-            on[j] = false;
           }
-          cur[j] = home ? tbl.index[hash[j] & tbl.mask] : 0u;
         }
-#pragma unroll
-        for (int j = 0; j < kRpBinItems; ++j)
-          if (on[j] && cur[j] > rec[j].i) atomicMin(&tbl.index[hash[j] & tbl.mask], rec[j].i);
       }
       if (!fits) *overflow = 1;
       __syncthreads();
@@ -1125,8 +1152,9 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
           uint32_t f[kRpBinItems];
 #pragma unroll
           for (int j = 0; j < kRpBinItems; ++j) {
-            k[j] = on[j] ? tbl.keys[hash[j] & tbl.mask] : static_cast<Key>(0);
-            f[j] = on[j] ? tbl.index[hash[j] & tbl.mask] : 0u;
+            k[j] = 0;
+            f[j] = 0;
+            if (on[j]) tbl.look(hash[j] & tbl.mask, &k[j], &f[j]);
           }
 #pragma unroll
           for (int j = 0; j < kRpBinItems; ++j) {
@@ -1203,7 +1231,7 @@ __global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) {
   for (int j = 0; j < kRpItems; ++j) {
     const int64_t i = lo + j * kRpBlock + threadIdx.x;
     const uint32_t f = i < hi ? result[at[j]] : 0xFFFFFFFFu;
-    if (i < hi) a.pos[i] = f;
+    if (i < hi) a.first[i] = f;
     // a wave's 64 elements lie in one tile of kRlTile ids
     const uint64_t wins = __builtin_amdgcn_ballot_w64(i < hi && f == static_cast<uint32_t>(i));
     if (lane_id() == 0 && wins)
@@ -1493,7 +1521,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     // fused hop do (and an earlier kernel that stored the mark already is just as good)
     if (path.mode == 0) path.mode = 2;
     RpArgs a{total, elem_bytes, n, path, wide_mark, rp.log2P, rp.W, base + rp.rec_off,
-             reinterpret_cast<uint32_t *>(base + rp.pos_off), reinterpret_cast<uint32_t *>(base + rp.firstp_off),
+             reinterpret_cast<uint32_t *>(base + rp.first_off), reinterpret_cast<uint32_t *>(base + rp.firstp_off),
              reinterpret_cast<uint32_t *>(base + rp.hist_off), reinterpret_cast<uint32_t *>(base + rp.bintot_off),
              reinterpret_cast<uint32_t *>(base + rp.binstart_off), reinterpret_cast<uint32_t *>(base + rp.coarse_off), reinterpret_cast<uint16_t *>(base + rp.local_off),
              reinterpret_cast<uint32_t *>(base + rp.tile_off), partials,
@@ -1515,9 +1543,9 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_gather_kernel, dim3(rp.W), dim3(kRpBlock), (2 * rp.P + 1) * sizeof(uint32_t), s, a);
     SHMT_LAUNCH_CHECK();
-    const RlUniqueArgs unq{total, elem_bytes, n, a.pos, 4, partials, unique_out, ranks, count_out, count_copy,
+    const RlUniqueArgs unq{total, elem_bytes, n, a.first, 4, partials, unique_out, ranks, count_out, count_copy,
                            2, a.coarse, static_cast<int>(kRpTile / kRlTile)};
-    const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, a.pos, 4};
+    const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, a.first, 4};
     hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, unq);
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, lab);
