@@ -27,6 +27,11 @@ enum StageKind : int {
   kStageRlFirst = 13,
   kStageRlUnique = 14,
   kStageRlLabels = 15,
+  kStageRpCount = 16,
+  kStageRpRows = 17,
+  kStageRpScatter = 18,
+  kStageRpGather = 19,
+  kStageRpBins = 20,  // + (largest table - this launch's table), log2 of the slots: 20 .. 22
 };
 
 struct Stage {
@@ -37,6 +42,7 @@ struct Stage {
 
 struct StageList {
   int n = 0;
+  int jobs = 1;  // how many jobs the caller means to merge (a job may choose its kernels by it)
   bool mergeable = true;
   Stage stage[kMaxStages];
 };
@@ -106,7 +112,8 @@ struct RelabelTable {
   uint64_t *wide_mark;  // where the earlier kernels store `nonce` when an id lies outside [0, 2^32)
   uint64_t nonce;
 };
-int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scratch_bytes, RelabelTable *out);
+int relabel_table(int64_t N, bool n_is_loose_bound, int merged_jobs, void *scratch, int64_t scratch_bytes,
+                  RelabelTable *out);  // merged_jobs: 0 for a launch sequence of its own
 int launch_relabel_passes(const void *total, int64_t n_bound, int64_t n_fixed, const int64_t *n_fixed_dev,
                           const void *n_extra_dev, int n_extra_bytes, int elem_bytes, void *scratch,
                           int64_t scratch_bytes, void *unique_out, void *labels_out, int64_t *count_out,

@@ -706,31 +706,45 @@ constexpr int64_t kRpBinIds = 16384; // ids per bin from which on the number of 
 constexpr int64_t kRpTile = 8192;    // ids per tile of the count / scatter / gather passes
 constexpr int kRpMaxRoundsLog2 = 10;
 constexpr int64_t kRpDefaultMin = kRlSelfPrefixTiles * kRlTile + 1;
+// Hops that share their launches with those of other batches (launchers.h) are sized for a bound of their
+// ids, and the five passes' fixed costs are paid once for all of them: from this bound and this many jobs on
+// they take the partition passes as well.
+constexpr int64_t kRpMergedMin = 512 * 1024;
+constexpr int kRpMergedMinJobs = 4;
+constexpr int kRpMinSlotsLog2 = 12;  // smallest table a bin pass is compiled for
 
 struct RpTuning {
-  int64_t min_ids;
+  int64_t min_ids, min_ids_merged;
   int slots_log2, max_rounds_log2;
 };
-static RpTuning g_rp_tuning{kRpDefaultMin, kRpSlotsLog2, kRpMaxRoundsLog2};
+static RpTuning g_rp_tuning{kRpDefaultMin, kRpMergedMin, kRpSlotsLog2, kRpMaxRoundsLog2};
 
 struct RpPlan {
   bool ok;
   int log2P;
+  int table_log2;  // which compiled table size the bin pass uses (the tuning may use less of it)
   uint32_t P, W;
   int64_t rec_off, first_off, firstp_off, local_off, hist_off, bintot_off, binstart_off, coarse_off, tile_off, end;
 };
 
 // Where the partition passes keep their arrays inside the table memory (16 * cap bytes) of a
 // scratch buffer sized for N ids; ok = false when N is outside the range this path serves.
-static RpPlan rp_plan(int64_t N) {
+static RpPlan rp_plan(int64_t N, int merged_jobs = 0, bool loose = false) {
   RpPlan p{};
-  if (N < g_rp_tuning.min_ids || N <= kRlSmallMax) return p;
+  const bool merged = merged_jobs >= kRpMergedMinJobs;
+  if (merged_jobs > 0 && !merged) return p;
+  if (N < (merged ? g_rp_tuning.min_ids_merged : g_rp_tuning.min_ids) || N <= kRlSmallMax) return p;
   int lg = kRpMinBinsLog2;
   while ((kRpBinIds << lg) < N) ++lg;
   if (lg > kRpMaxBinsLog2) return p;
   p.log2P = lg;
   p.P = 1u << lg;
   p.W = static_cast<uint32_t>((N + kRpTile - 1) / kRpTile);
+  // at least one slot per id the bin may hold if every id of the input is distinct; when N is a loose bound of
+  // the id count (a chained hop: typically three times what turns up) half of that, a bin that does get more
+  // taking two rounds
+  p.table_log2 = kRpMinSlotsLog2;
+  while (p.table_log2 < kRpSlotsLog2 && (static_cast<int64_t>(p.P) << p.table_log2) < (loose ? N / 2 : N)) ++p.table_log2;
   auto up = [](int64_t x) { return (x + 255) & ~255ll; };
   p.rec_off = 0;
   p.first_off = up(16 * N);
@@ -811,15 +825,20 @@ __device__ __forceinline__ bool rp_covered(const RpArgs &a, const unsigned long 
   return a.eb == 4 || static_cast<const int64_t *>(a.total)[static_cast<uint32_t>(v >> 32)] == key;
 }
 
-__global__ __launch_bounds__(kRpBlock) void rp_count_kernel(RpArgs a) {
+__device__ __forceinline__ void rp_count_body(unsigned bx, const RpArgs &a) {
   extern __shared__ uint32_t hist[];  // P counters
   __shared__ unsigned long long dedup[kRpDedupSlots];
   const int64_t N = rl_count(a.n);
   const uint32_t P = 1u << a.log2P;
+  const int64_t lo = static_cast<int64_t>(bx) * kRpTile;
+  if (lo >= N) {
+    // launched for a bound of N: a tile past the ids has an empty column
+    for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) a.hist[static_cast<size_t>(b) * a.W + bx] = 0;
+    return;
+  }
   for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) hist[b] = 0;
   rp_dedup_clear(dedup);
   __syncthreads();
-  const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
   const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
   int64_t idx[kRpItems], key[kRpItems];
   bool ok[kRpItems];
@@ -840,12 +859,18 @@ __global__ __launch_bounds__(kRpBlock) void rp_count_kernel(RpArgs a) {
   for (int j = 0; j < kRpItems; ++j)
     if (ok[j] && !rp_covered(a, dedup, key[j], idx[j], hash[j])) atomicAdd(&hist[hash[j] >> (32 - a.log2P)], 1u);
   __syncthreads();
-  for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) a.hist[static_cast<size_t>(b) * a.W + blockIdx.x] = hist[b];
+  for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) a.hist[static_cast<size_t>(b) * a.W + bx] = hist[b];
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_count_kernel(RpArgs a) { rp_count_body(blockIdx.x, a); }
+
+__global__ __launch_bounds__(kRpBlock) void rp_count_jobs(Jobs<RpArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rp_count_body(blockIdx.x, j.a[blockIdx.y]);
 }
 
 // One wave per bin: the row's counts become the offsets of the tiles' runs inside the bin.
-__global__ __launch_bounds__(256) void rp_rows_kernel(RpArgs a) {
-  const uint32_t b = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+__device__ __forceinline__ void rp_rows_body(unsigned bx, const RpArgs &a) {
+  const uint32_t b = bx * (256 / kWave) + threadIdx.x / kWave;
   if (b >= (1u << a.log2P)) return;
   uint32_t *const row = a.hist + static_cast<size_t>(b) * a.W;
   const uint32_t lane = lane_id();
@@ -860,6 +885,12 @@ __global__ __launch_bounds__(256) void rp_rows_kernel(RpArgs a) {
   if (lane == 0) a.bintot[b] = carry;
 }
 
+__global__ __launch_bounds__(256) void rp_rows_kernel(RpArgs a) { rp_rows_body(blockIdx.x, a); }
+
+__global__ __launch_bounds__(256) void rp_rows_jobs(Jobs<RpArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rp_rows_body(blockIdx.x, j.a[blockIdx.y]);
+}
+
 // The id a packed record stands for, as the count pass hashed it (4-byte ids are signed).
 __device__ __forceinline__ int64_t rp_packed_key(unsigned long long rec, int eb) {
   const uint32_t k = static_cast<uint32_t>(rec >> 32);
@@ -870,12 +901,14 @@ __device__ __forceinline__ int64_t rp_packed_key(unsigned long long rec, int eb)
 // tile are therefore put in bin order in LDS first (position = start of the bin among the tile's records +
 // rank within the bin) and written out from there, consecutive lanes to consecutive addresses of a run.
 // 16-byte records (ids beyond 32 bits) do not fit the LDS and are stored directly.
-__global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
+__device__ __forceinline__ void rp_scatter_body(unsigned bx, const RpArgs &a) {
   extern __shared__ uint32_t words[];  // run start in memory, record count, start among the tile's records: P (+ 1) each
   __shared__ unsigned long long stage[kRpTile];  // first the de-duplication table and the ranks of its owners
   __shared__ uint32_t scan_lds[kRpBlock / kWave];
   const int64_t N = rl_count(a.n);
   const uint32_t P = 1u << a.log2P;
+  // launched for a bound of N: a tile past the ids has nothing to scatter (tile 0 also publishes the bin starts)
+  if (bx > 0 && static_cast<int64_t>(bx) * kRpTile >= N) return;
   uint32_t *const run_at = words, *const cnt = words + P, *const lstart = words + 2 * P;
   unsigned long long *const dedup = stage;
   uint32_t *const rep_rank = reinterpret_cast<uint32_t *>(stage + kRpDedupSlots);
@@ -892,16 +925,16 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
   for (uint32_t j = 0; j < per; ++j) {
     const uint32_t b = b0 + j;
     if (b < P) {
-      run_at[b] = run + a.hist[static_cast<size_t>(b) * a.W + blockIdx.x];
+      run_at[b] = run + a.hist[static_cast<size_t>(b) * a.W + bx];
       cnt[b] = 0;
-      if (blockIdx.x == 0) a.binstart[b] = run;
+      if (bx == 0) a.binstart[b] = run;
       run += a.bintot[b];
     }
   }
-  if (blockIdx.x == 0 && threadIdx.x == 0) a.binstart[P] = all;
+  if (bx == 0 && threadIdx.x == 0) a.binstart[P] = all;
   __syncthreads();
   const bool packed = rl_packed(a.path);
-  const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
+  const int64_t lo = static_cast<int64_t>(bx) * kRpTile;
   const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
   int64_t idx[kRpItems], key[kRpItems];
   bool ok[kRpItems];
@@ -945,7 +978,7 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
     if (threadIdx.x == 0) lstart[P] = records;
   }
   __syncthreads();
-  uint32_t *const runs = a.tile_runs + static_cast<size_t>(blockIdx.x) * (2 * P + 1);
+  uint32_t *const runs = a.tile_runs + static_cast<size_t>(bx) * (2 * P + 1);
   for (uint32_t t = threadIdx.x; t < 2 * P + 1; t += kRpBlock) runs[t] = t < P ? run_at[t] : lstart[t - P];
 #pragma unroll
   for (int j = 0; j < kRpItems; ++j) {
@@ -969,6 +1002,12 @@ __global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) {
     const uint32_t bin = hash_id(rp_packed_key(rec, a.eb)) >> (32 - a.log2P);
     static_cast<unsigned long long *>(a.rec)[run_at[bin] + (q - lstart[bin])] = rec;
   }
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_scatter_kernel(RpArgs a) { rp_scatter_body(blockIdx.x, a); }
+
+__global__ __launch_bounds__(kRpBlock) void rp_scatter_jobs(Jobs<RpArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rp_scatter_body(blockIdx.x, j.a[blockIdx.y]);
 }
 
 // The table of a bin: per slot an id, claimed by a compare-and-swap, and the smallest index seen for it,
@@ -1005,7 +1044,7 @@ struct RpTable {
   }
 
   __device__ __forceinline__ void clear() const {
-    for (uint32_t t = threadIdx.x; t <= mask; t += kRpBlock) {
+    for (uint32_t t = threadIdx.x; t <= mask; t += blockDim.x) {
       mem[t] = ~0ull;
       if (!PACKED) *index_at(t) = 0xFFFFFFFFu;
     }
@@ -1067,7 +1106,7 @@ __device__ __forceinline__ bool rp_mine(int64_t key, uint32_t round_mask, uint32
   return round_mask == 0 || (rp_class(key) & round_mask) == round;
 }
 
-// kRpBinItems records of a bin, element e0 + j * kRpBlock for j = 0 .., all loads in flight together.
+// kRpBinItems records of a bin, element e0 + j * (threads of the workgroup) for j = 0 .., all loads in flight together.
 template <bool PACKED>
 __device__ __forceinline__ void rp_load_records(const RpArgs &a, uint32_t start, uint32_t cnt, uint32_t e0,
                                                 uint32_t round_mask, uint32_t round,
@@ -1077,8 +1116,8 @@ __device__ __forceinline__ void rp_load_records(const RpArgs &a, uint32_t start,
   for (int j = 0; j < kRpBinItems; ++j) {
     rec[j].key = 0;
     rec[j].i = 0;
-    on[j] = e0 + j * kRpBlock < cnt;
-    if (on[j]) rec[j].load(a.rec, start + e0 + j * kRpBlock);
+    on[j] = e0 + j * blockDim.x < cnt;
+    if (on[j]) rec[j].load(a.rec, start + e0 + j * blockDim.x);
   }
 #pragma unroll
   for (int j = 0; j < kRpBinItems; ++j) {
@@ -1088,11 +1127,12 @@ __device__ __forceinline__ void rp_load_records(const RpArgs &a, uint32_t start,
 }
 
 template <bool PACKED>
-__device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long *mem, uint32_t *shared_words) {
+__device__ __forceinline__ void rp_bin_body(unsigned bx, const RpArgs &a, unsigned long long *mem,
+                                            uint32_t *shared_words) {
   using Table = RpTable<PACKED>;
   using Key = typename Table::Key;
-  const uint32_t start = a.binstart[blockIdx.x];
-  const uint32_t cnt = a.binstart[blockIdx.x + 1] - start;
+  const uint32_t start = a.binstart[bx];
+  const uint32_t cnt = a.binstart[bx + 1] - start;
   if (cnt == 0) return;
   uint32_t *const overflow = &shared_words[0];
   const uint32_t slots = PACKED ? (1u << a.slots_log2) : (1u << (a.slots_log2 - 1));
@@ -1105,7 +1145,7 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
       if (threadIdx.x == 0) *overflow = 0;
       __syncthreads();
       bool fits = true;
-      for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * kRpBlock) {
+      for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * blockDim.x) {
         RpRecord<PACKED> rec[kRpBinItems];
         uint32_t hash[kRpBinItems];
         bool on[kRpBinItems];
@@ -1143,7 +1183,7 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
       __syncthreads();
       done = *overflow == 0;
       if (done) {
-        for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * kRpBlock) {
+        for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * blockDim.x) {
           RpRecord<PACKED> rec[kRpBinItems];
           uint32_t hash[kRpBinItems];
           bool on[kRpBinItems];
@@ -1164,7 +1204,7 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
               f[j] = *tbl.all_ones;
             else if (k[j] != key)
               f[j] = tbl.first_from(key, hash[j] + 1);
-            a.firstp[start + e0 + j * kRpBlock] = f[j];
+            a.firstp[start + e0 + j * blockDim.x] = f[j];
           }
         }
       }
@@ -1173,7 +1213,7 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
     if (done) return;
   }
   // every pair: the ids of this bin defeat both hashes
-  for (uint32_t e = threadIdx.x; e < cnt; e += kRpBlock) {
+  for (uint32_t e = threadIdx.x; e < cnt; e += blockDim.x) {
     RpRecord<PACKED> mine;
     mine.load(a.rec, start + e);
     uint32_t first = mine.i;
@@ -1186,27 +1226,42 @@ __device__ __forceinline__ void rp_bin_body(const RpArgs &a, unsigned long long 
   }
 }
 
-__global__ __launch_bounds__(kRpBlock) void rp_bins_kernel(RpArgs a) {
-  __shared__ unsigned long long mem[1 << kRpSlotsLog2];
+// TABLE_LOG2: the table this instantiation has room for (a.slots_log2 <= TABLE_LOG2 of it are used). Small
+// bins take small tables and small workgroups, so that several of them share a compute unit.
+constexpr int rp_bins_threads(int table_log2) { return table_log2 >= 14 ? 1024 : (table_log2 == 13 ? 512 : 256); }
+
+template <int TABLE_LOG2>
+__device__ __forceinline__ void rp_bins_body(unsigned bx, const RpArgs &a) {
+  __shared__ unsigned long long mem[1 << TABLE_LOG2];
   __shared__ uint32_t shared_words[2];
   if (rl_packed(a.path))
-    rp_bin_body<true>(a, mem, shared_words);
+    rp_bin_body<true>(bx, a, mem, shared_words);
   else
-    rp_bin_body<false>(a, mem, shared_words);
+    rp_bin_body<false>(bx, a, mem, shared_words);
+}
+
+template <int TABLE_LOG2>
+__global__ __launch_bounds__(rp_bins_threads(TABLE_LOG2)) void rp_bins_kernel(RpArgs a) {
+  rp_bins_body<TABLE_LOG2>(blockIdx.x, a);
+}
+
+template <int TABLE_LOG2>
+__global__ __launch_bounds__(rp_bins_threads(TABLE_LOG2)) void rp_bins_jobs(Jobs<RpArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rp_bins_body<TABLE_LOG2>(blockIdx.x, j.a[blockIdx.y]);
 }
 
 // The results of the tile's records are read run by run, consecutive lanes from consecutive addresses, into
 // LDS in the tile's bin order; every element then picks the one of its record there.
-__global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) {
+__device__ __forceinline__ void rp_gather_body(unsigned bx, const RpArgs &a) {
   extern __shared__ uint32_t words[];  // run start in memory (P), start among the tile's records (P + 1)
   __shared__ uint32_t result[kRpTile];
   __shared__ uint32_t firsts[kRpTile / kRlTile];
   const int64_t N = rl_count(a.n);
-  const int64_t lo = static_cast<int64_t>(blockIdx.x) * kRpTile;
+  const int64_t lo = static_cast<int64_t>(bx) * kRpTile;
   if (lo >= N) return;
   const int64_t hi = lo + kRpTile < N ? lo + kRpTile : N;
   const uint32_t P = 1u << a.log2P;
-  const uint32_t *const runs = a.tile_runs + static_cast<size_t>(blockIdx.x) * (2 * P + 1);
+  const uint32_t *const runs = a.tile_runs + static_cast<size_t>(bx) * (2 * P + 1);
   for (uint32_t t = threadIdx.x; t < 2 * P + 1; t += kRpBlock) words[t] = runs[t];
   const int sub_tiles = static_cast<int>(kRpTile / kRlTile);
   for (int t = threadIdx.x; t < sub_tiles; t += kRpBlock) firsts[t] = 0;
@@ -1248,8 +1303,14 @@ __global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) {
   static_assert(kRpTile / kRlTile <= kWave, "the first wave sums a tile's counts");
   if (threadIdx.x < kWave) {
     all = wave_last(wave_inclusive_scan(all));
-    if (threadIdx.x == 0) a.coarse[blockIdx.x] = all;
+    if (threadIdx.x == 0) a.coarse[bx] = all;
   }
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_gather_kernel(RpArgs a) { rp_gather_body(blockIdx.x, a); }
+
+__global__ __launch_bounds__(kRpBlock) void rp_gather_jobs(Jobs<RpArgs> j) {
+  if (blockIdx.x < j.blocks[blockIdx.y]) rp_gather_body(blockIdx.x, j.a[blockIdx.y]);
 }
 
 // A value no earlier call has used (and that uninitialised memory is unlikely to hold).
@@ -1511,21 +1572,36 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
 
   int rc = SHMT_OK;
   const int scanned = nb > kRlSelfPrefixTiles;
-  const RpPlan rp = rp_plan(N);
-  if (rp.ok && defer) {
-    defer->mergeable = false;
+  // a job among fewer merged ones than the partition passes pay for keeps the table (and stays mergeable)
+  const RpPlan rp = rp_plan(N, defer ? (prepared ? defer->jobs : 1) : 0, n.fixed_dev != nullptr);
+  if (!rp.ok && defer && rp_plan(N).ok) {
+    defer->mergeable = false;  // a hop of this size on its own takes the partition passes: one by one then
     return SHMT_OK;
   }
   if (rp.ok) {
     // 8-byte ids: the count pass looks at every id itself, so it can vouch for them like the kernels of a
     // fused hop do (and an earlier kernel that stored the mark already is just as good)
     if (path.mode == 0) path.mode = 2;
+    const int slots_log2 = g_rp_tuning.slots_log2 < rp.table_log2 ? g_rp_tuning.slots_log2 : rp.table_log2;
     RpArgs a{total, elem_bytes, n, path, wide_mark, rp.log2P, rp.W, base + rp.rec_off,
              reinterpret_cast<uint32_t *>(base + rp.first_off), reinterpret_cast<uint32_t *>(base + rp.firstp_off),
              reinterpret_cast<uint32_t *>(base + rp.hist_off), reinterpret_cast<uint32_t *>(base + rp.bintot_off),
-             reinterpret_cast<uint32_t *>(base + rp.binstart_off), reinterpret_cast<uint32_t *>(base + rp.coarse_off), reinterpret_cast<uint16_t *>(base + rp.local_off),
-             reinterpret_cast<uint32_t *>(base + rp.tile_off), partials,
-             g_rp_tuning.slots_log2, g_rp_tuning.max_rounds_log2};
+             reinterpret_cast<uint32_t *>(base + rp.binstart_off), reinterpret_cast<uint32_t *>(base + rp.coarse_off),
+             reinterpret_cast<uint16_t *>(base + rp.local_off), reinterpret_cast<uint32_t *>(base + rp.tile_off),
+             partials, slots_log2, g_rp_tuning.max_rounds_log2};
+    const RlUniqueArgs unq{total, elem_bytes, n, a.first, 4, partials, unique_out, ranks, count_out, count_copy,
+                           2, a.coarse, static_cast<int>(kRpTile / kRlTile)};
+    const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, a.first, 4};
+    if (defer) {
+      stage_push(defer, kStageRpCount, rp.W, kRpBlock, a);
+      stage_push(defer, kStageRpRows, (rp.P + 3) / 4, 256, a);
+      stage_push(defer, kStageRpScatter, rp.W, kRpBlock, a);
+      stage_push(defer, kStageRpBins + (kRpSlotsLog2 - rp.table_log2), rp.P, rp_bins_threads(rp.table_log2), a);
+      stage_push(defer, kStageRpGather, rp.W, kRpBlock, a);
+      stage_push(defer, kStageRlUnique, static_cast<unsigned>(nb), kRlBlock, unq);
+      stage_push(defer, kStageRlLabels, grid_for(N, 256), 256, lab);
+      return SHMT_OK;
+    }
     if (segs && !prepared) {
       // concatenation only: there is no table to empty
       hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(N, 256 * 4)), dim3(256), 0, s,
@@ -1539,13 +1615,15 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_scatter_kernel, dim3(rp.W), dim3(kRpBlock), (3 * rp.P + 1) * sizeof(uint32_t), s, a);
     SHMT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(rp_bins_kernel, dim3(rp.P), dim3(kRpBlock), 0, s, a);
+    if (rp.table_log2 >= 14)
+      hipLaunchKernelGGL(rp_bins_kernel<14>, dim3(rp.P), dim3(rp_bins_threads(14)), 0, s, a);
+    else if (rp.table_log2 == 13)
+      hipLaunchKernelGGL(rp_bins_kernel<13>, dim3(rp.P), dim3(rp_bins_threads(13)), 0, s, a);
+    else
+      hipLaunchKernelGGL(rp_bins_kernel<12>, dim3(rp.P), dim3(rp_bins_threads(12)), 0, s, a);
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_gather_kernel, dim3(rp.W), dim3(kRpBlock), (2 * rp.P + 1) * sizeof(uint32_t), s, a);
     SHMT_LAUNCH_CHECK();
-    const RlUniqueArgs unq{total, elem_bytes, n, a.first, 4, partials, unique_out, ranks, count_out, count_copy,
-                           2, a.coarse, static_cast<int>(kRpTile / kRlTile)};
-    const RlLabelsArgs lab{labels_out, elem_bytes, n, ranks, a.first, 4};
     hipLaunchKernelGGL(rl_unique_kernel, dim3(static_cast<unsigned>(nb)), dim3(kRlBlock), 0, s, unq);
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rl_labels_kernel, dim3(grid_for(N, 256)), dim3(256), 0, s, lab);
@@ -1604,7 +1682,8 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
 
 namespace shmt {
 
-int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scratch_bytes, RelabelTable *out) {
+int relabel_table(int64_t N, bool n_is_loose_bound, int merged_jobs, void *scratch, int64_t scratch_bytes,
+                  RelabelTable *out) {
   SHMT_REQUIRE(N >= 1 && N < (1ll << 31), "relabel: N must be in [1, 2^31)");
   const RlLayout l = rl_layout(N);
   if (scratch == nullptr || scratch_bytes < l.total) {
@@ -1619,7 +1698,7 @@ int relabel_table(int64_t N, bool n_is_loose_bound, void *scratch, int64_t scrat
   // it did produce) half the slots are used: still one 16-byte slot per id in the worst case, and
   // half as much to empty.
   // Nor is there when the partition passes take the input (rp_plan).
-  out->n16 = (N <= kRlSmallMax || rp_plan(N).ok) ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
+  out->n16 = (N <= kRlSmallMax || rp_plan(N, merged_jobs).ok) ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
   out->wide_mark = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + l.flag_off);
   out->nonce = relabel_nonce();
   return SHMT_OK;
@@ -1668,6 +1747,30 @@ int launch_merged_relabel_stage(int n_jobs, const Stage *const *stages, hipStrea
       hipLaunchKernelGGL(rl_labels_jobs, dim3(blocks, n_jobs), dim3(threads), 0, s, j);
       break;
     }
+    case kStageRpCount:
+    case kStageRpRows:
+    case kStageRpScatter:
+    case kStageRpGather:
+    case kStageRpBins:
+    case kStageRpBins + 1:
+    case kStageRpBins + 2: {
+      Jobs<RpArgs> j;
+      const unsigned blocks = jobs_from_stages(n_jobs, stages, &j);
+      int log2P = 0;  // the LDS arrays are sized for the job with the most bins
+      for (int i = 0; i < n_jobs; ++i) log2P = j.a[i].log2P > log2P ? j.a[i].log2P : log2P;
+      const size_t P = static_cast<size_t>(1) << log2P;
+      const dim3 grid(blocks, n_jobs), wg(threads);
+      switch (stages[0]->kind) {
+        case kStageRpCount: hipLaunchKernelGGL(rp_count_jobs, grid, wg, P * sizeof(uint32_t), s, j); break;
+        case kStageRpRows: hipLaunchKernelGGL(rp_rows_jobs, grid, wg, 0, s, j); break;
+        case kStageRpScatter: hipLaunchKernelGGL(rp_scatter_jobs, grid, wg, (3 * P + 1) * sizeof(uint32_t), s, j); break;
+        case kStageRpGather: hipLaunchKernelGGL(rp_gather_jobs, grid, wg, (2 * P + 1) * sizeof(uint32_t), s, j); break;
+        case kStageRpBins: hipLaunchKernelGGL(rp_bins_jobs<14>, grid, wg, 0, s, j); break;
+        case kStageRpBins + 1: hipLaunchKernelGGL(rp_bins_jobs<13>, grid, wg, 0, s, j); break;
+        default: hipLaunchKernelGGL(rp_bins_jobs<12>, grid, wg, 0, s, j); break;
+      }
+      break;
+    }
     default:
       set_error("internal: stage kind %d has no merged relabel launch", stages[0]->kind);
       return SHMT_EINVAL;
@@ -1693,6 +1796,7 @@ int shmt_relabel_tuning(int64_t partition_min_ids, int lds_slots_log2, int max_r
   SHMT_REQUIRE(max_rounds_log2 >= -1 && max_rounds_log2 <= 20,
                "shmt_relabel_tuning: max_rounds_log2 must be -1 (default) or in [0, 20]");
   g_rp_tuning.min_ids = partition_min_ids <= 0 ? kRpDefaultMin : partition_min_ids;
+  g_rp_tuning.min_ids_merged = partition_min_ids <= 0 ? kRpMergedMin : (partition_min_ids < kRpMergedMin ? partition_min_ids : kRpMergedMin);
   g_rp_tuning.slots_log2 = lds_slots_log2 == 0 ? kRpSlotsLog2 : lds_slots_log2;
   g_rp_tuning.max_rounds_log2 = max_rounds_log2 < 0 ? kRpMaxRoundsLog2 : max_rounds_log2;
   return SHMT_OK;

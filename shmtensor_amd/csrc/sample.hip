@@ -1098,7 +1098,8 @@ static int hop_impl(const void *indptr, int ptr_bytes, const void *indices, int 
                "shmt_sample_hop: null buffer");
   const int64_t n_max = S + S * k;
   RelabelTable table;
-  int rc = relabel_table(n_max, S_len != nullptr, scratch, scratch_bytes, &table);
+  int rc = relabel_table(n_max, S_len != nullptr, launcher.defer ? launcher.defer->jobs : 0, scratch, scratch_bytes,
+                         &table);
   if (rc) return rc;
   PlanHopExtras plan_hop{total_out, elem_bytes, S_len, nullptr, nullptr, 0};
   rc = plan_impl(indptr, ptr_bytes, cache_indptr, map, seeds, seed_bytes, S, k, replace, sub_indptr, plan,
@@ -1164,6 +1165,7 @@ int shmt_sample_hops_chained(const shmt_hop_job *jobs, int n_jobs, void *stream)
     StageList lists[kMaxJobs];
     bool merge = n > 1;
     for (int j = 0; j < n && merge; ++j) {
+      lists[j].jobs = n;
       const int rc = hop_job(jobs[first + j], Launcher{s, &lists[j]});
       if (rc) return rc;
       merge = lists[j].mergeable && lists[j].n == lists[0].n;

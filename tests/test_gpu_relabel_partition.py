@@ -111,22 +111,23 @@ def _same(a, b):
 
 
 @pytest.mark.parametrize("idx_dt", [torch.int32, torch.int64])
-def test_fused_hop_and_chained_batches_through_partitions(capi, tuning, idx_dt):
+@pytest.mark.parametrize("n_batches,in_flight", [(4, 4), (8, 8), (11, 8), (3, 3)])
+def test_fused_hop_and_chained_batches_through_partitions(capi, tuning, idx_dt, n_batches, in_flight):
     """The fused hop (the pick kernel writes the relabel input and would have emptied the table) and
-    sample_blocks (hops chained on the device, launches shared between batches) give what they give
-    with the default setting."""
+    sample_blocks (hops chained on the device; from four batches on their partition passes share their
+    launches, fewer keep the table in memory) give what they give with the default setting."""
     indptr, indices = rmat_csr(15, 12, 3)
     indptr, indices = indptr.cuda(), indices.to(idx_dt).cuda()
     n = indptr.numel() - 1
     g = torch.Generator().manual_seed(4)
     seeds = torch.randint(0, n, (3000,), generator=g).to(idx_dt).cuda()
-    batches = [torch.randperm(n, generator=g)[:700].to(idx_dt).cuda() for _ in range(4)]
+    batches = [torch.randperm(n, generator=g)[:700 - 13 * b].to(idx_dt).cuda() for b in range(n_batches)]
     got = {}
     for min_ids in (0, 8193):
         tuning(min_ids)
         hop = capi.sample_hop(indptr, indices, None, None, None, seeds, 10, False, seed=5)
         blocks = capi.sample_blocks(indptr, indices, None, None, None, batches, [5, 6, 7], False,
-                                    seeds_rng=[5, 6, 7, 8], max_in_flight=4)
+                                    seeds_rng=list(range(5, 5 + n_batches)), max_in_flight=in_flight)
         torch.cuda.synchronize()
         got[min_ids] = (hop, blocks)
     _same(got[0][0], got[8193][0])
