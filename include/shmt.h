@@ -328,13 +328,17 @@ int shmt_relabel_wide(const void *total, int64_t N, void *scratch,
                       void *labels_out, int64_t *count_out, void *stream);
 /* How large inputs are relabelled (no counterpart in the reference, whose
  * four passes all probe one table in memory, src/tensor_relabel.cu:147-203).
- * From partition_min_ids ids on (and up to 2^26) the first-occurrence index of
+ * From partition_min_ids ids on (and up to 2^23) the first-occurrence index of
  * every id is found by partitioning the ids by hash and giving every
  * partition a table in LDS, which reads and writes memory in streams instead
  * of touching one random line per id and pass; results are identical.
- * partition_min_ids <= 0 restores the default (2,097,153: inputs whose tile
- * counts need a scan launch of their own). lds_slots_log2 (0 = default, 14)
- * and max_rounds_log2 (-1 = default, 10) shrink a partition's table and the
+ * partition_min_ids <= 0 restores the defaults: 2,097,153 for a hop whose size
+ * is only a loose bound of its ids (the chained hops of shmt_sample_hop_chained),
+ * 1,048,576 for calls that know their size, 524,288 for hops that share their
+ * launches with those of three or more other batches
+ * (shmt_sample_hops_chained); a value given lowers all three to it.
+ * lds_slots_log2 (0 = default, 14) and max_rounds_log2 (-1 = default, 10)
+ * shrink a partition's table and the
  * number of rounds a partition may take before all pairs of its ids are
  * compared; they exist so that tests can drive those rare paths. Process-wide,
  * not synchronised with calls in flight on other threads.                    */

@@ -710,6 +710,8 @@ constexpr int64_t kRpDefaultMin = kRlSelfPrefixTiles * kRlTile + 1;
 // ids, and the five passes' fixed costs are paid once for all of them: from this bound and this many jobs on
 // they take the partition passes as well.
 constexpr int64_t kRpMergedMin = 512 * 1024;
+// A call that knows its number of ids (not merely a loose bound of it) gains from about a million on.
+constexpr int64_t kRpExactMin = 1024 * 1024;
 constexpr int kRpMergedMinJobs = 4;
 constexpr int kRpMinSlotsLog2 = 12;  // smallest table a bin pass is compiled for
 
@@ -733,7 +735,8 @@ static RpPlan rp_plan(int64_t N, int merged_jobs = 0, bool loose = false) {
   RpPlan p{};
   const bool merged = merged_jobs >= kRpMergedMinJobs;
   if (merged_jobs > 0 && !merged) return p;
-  if (N < (merged ? g_rp_tuning.min_ids_merged : g_rp_tuning.min_ids) || N <= kRlSmallMax) return p;
+  const int64_t exact_min = g_rp_tuning.min_ids < kRpExactMin ? g_rp_tuning.min_ids : kRpExactMin;
+  if (N < (merged ? g_rp_tuning.min_ids_merged : (loose ? g_rp_tuning.min_ids : exact_min)) || N <= kRlSmallMax) return p;
   int lg = kRpMinBinsLog2;
   while ((kRpBinIds << lg) < N) ++lg;
   if (lg > kRpMaxBinsLog2) return p;
@@ -1574,7 +1577,7 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
   const int scanned = nb > kRlSelfPrefixTiles;
   // a job among fewer merged ones than the partition passes pay for keeps the table (and stays mergeable)
   const RpPlan rp = rp_plan(N, defer ? (prepared ? defer->jobs : 1) : 0, n.fixed_dev != nullptr);
-  if (!rp.ok && defer && rp_plan(N).ok) {
+  if (!rp.ok && defer && rp_plan(N, 0, n.fixed_dev != nullptr).ok) {
     defer->mergeable = false;  // a hop of this size on its own takes the partition passes: one by one then
     return SHMT_OK;
   }
@@ -1698,7 +1701,7 @@ int relabel_table(int64_t N, bool n_is_loose_bound, int merged_jobs, void *scrat
   // it did produce) half the slots are used: still one 16-byte slot per id in the worst case, and
   // half as much to empty.
   // Nor is there when the partition passes take the input (rp_plan).
-  out->n16 = (N <= kRlSmallMax || rp_plan(N, merged_jobs).ok) ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
+  out->n16 = (N <= kRlSmallMax || rp_plan(N, merged_jobs, n_is_loose_bound).ok) ? 0 : (n_is_loose_bound ? (l.cap / 2 + 7) & ~7ll : l.cap);
   out->wide_mark = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + l.flag_off);
   out->nonce = relabel_nonce();
   return SHMT_OK;
