@@ -138,6 +138,37 @@ def test_fused_hop_and_chained_batches_through_partitions(capi, tuning, idx_dt, 
             _same(hop_x, hop_y)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_inputs_tables_and_round_limits(capi, cabi, oracle, tuning, seed):
+    """Seeded random cases: sizes, id universes from 3 values to 2^40, one to three tensors of mixed widths,
+    tables of 4 to 16,384 slots, round limits from 'all pairs at once' to the default."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(6):
+        n = int(rng.choice([rng.integers(8193, 20000), rng.integers(20000, 200000)]))
+        universe = int(rng.choice([3, 100, n // 10 + 2, n, 10 * n, 2**31 - 1, 2**40]))
+        slots = int(rng.choice([0, 0, 2, 3, 5, 8, 11, 14]))
+        rounds = int(rng.choice([-1, -1, 0, 1, 3]))
+        kind = str(rng.choice(["plain", "neg", "hub", "top32"]))
+        print("case", seed, case, n, universe, slots, rounds, kind, flush=True)
+        ids = rng.integers(0, universe, size=n).astype(np.int64)
+        if kind == "neg":
+            ids[::7] = -ids[::7] - 2
+        elif kind == "hub":
+            ids[rng.random(n) < rng.random() * 0.6] = ids[0]
+        elif kind == "top32":
+            ids[::5] = 2**32 - 1 - (ids[::5] % 3)
+        fits32 = ids.min() >= -2**31 and ids.max() < 2**31
+        nseg = int(rng.integers(1, 4))
+        parts = np.split(ids, np.sort(rng.integers(0, n, size=nseg - 1)))
+        parts = [p.astype(np.int32 if (fits32 and rng.random() < 0.5) else np.int64) for p in parts]
+        tuning(8193, slots, rounds)
+        u, labs = capi.tensor_relabel([torch.from_numpy(p).cuda() for p in parts])
+        ou, olabs = oracle.relabel([p.astype(np.int64) for p in parts])
+        assert np.array_equal(u.cpu().numpy().astype(np.int64), ou)
+        for l, o in zip(labs, olabs):
+            assert np.array_equal(l.cpu().numpy().astype(np.int64), o)
+
+
 def test_tuning_rejects_bad_values(cabi):
     lib = cabi.load()
     assert lib.shmt_relabel_tuning(0, 1, -1) != 0
