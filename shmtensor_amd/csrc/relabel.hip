@@ -1054,8 +1054,8 @@ struct RpTable {
     if (threadIdx.x == 0) *all_ones = 0xFFFFFFFFu;
   }
 
-  // From slot p on (key != kEmpty).
-  __device__ __forceinline__ bool insert_from(Key key, uint32_t i, uint32_t p) const {
+  // From slot p on (key != kEmpty); *slot: where the id sits (ids never move once they have a slot).
+  __device__ __forceinline__ bool insert_from(Key key, uint32_t i, uint32_t p, uint32_t *slot) const {
     p &= mask;
     for (uint32_t probes = 0; probes <= mask; ++probes) {
       Key k;
@@ -1064,6 +1064,7 @@ struct RpTable {
       if (k == kEmpty) k = atomicCAS(key_at(p), kEmpty, key);
       if (k == kEmpty || k == key) {
         if (cur > i) atomicMin(index_at(p), i);  // a look that is out of date can only show a larger index
+        *slot = p;
         return true;
       }
       p = (p + 1) & mask;
@@ -1102,6 +1103,7 @@ struct RpRecord {
 };
 
 constexpr int kRpBinItems = 8;  // records a thread has in flight while it walks over a bin
+constexpr int kRpHeldPasses = 1;  // passes of kRpBinItems records per thread whose table slots stay in registers
 
 // A bin whose ids do not fit its table is worked through in 2, 4, ... rounds over classes of its ids (bits
 // of the second hash).
@@ -1140,6 +1142,10 @@ __device__ __forceinline__ void rp_bin_body(unsigned bx, const RpArgs &a, unsign
   uint32_t *const overflow = &shared_words[0];
   const uint32_t slots = PACKED ? (1u << a.slots_log2) : (1u << (a.slots_log2 - 1));
   const Table tbl{mem, &shared_words[1], slots - 1};
+  // Where the records of the first kRpHeldPasses passes over the bin went (a slot, or one of the two marks):
+  // their results are then one LDS read each, without reading, hashing and probing a second time.
+  constexpr uint32_t kNotMine = 0xFFFFFFFFu, kAllOnes = 0xFFFFFFFEu;
+  uint32_t where[kRpHeldPasses][kRpBinItems];
   for (int lg = 0; lg <= a.max_rounds_log2; ++lg) {
     const uint32_t round_mask = (1u << lg) - 1u;
     bool done = true;
@@ -1148,21 +1154,24 @@ __device__ __forceinline__ void rp_bin_body(unsigned bx, const RpArgs &a, unsign
       if (threadIdx.x == 0) *overflow = 0;
       __syncthreads();
       bool fits = true;
-      for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * blockDim.x) {
+      // one pass: kRpBinItems records per thread; `slot_out` is null beyond the passes whose slots are kept
+      auto insert_pass = [&](uint32_t e0, uint32_t *slot_out) {
         RpRecord<PACKED> rec[kRpBinItems];
         uint32_t hash[kRpBinItems];
         bool on[kRpBinItems];
         rp_load_records<PACKED>(a, start, cnt, e0, round_mask, r, rec, hash, on);
         // the home slots of all records are looked at together, then claimed together, then their indices
-        // looked at and lowered together; only a record that met another id goes on along its probe sequence
+        // lowered together; only a record that met another id goes on along its probe sequence
         Key k[kRpBinItems];
-        uint32_t cur[kRpBinItems];
+        uint32_t cur[kRpBinItems], slot[kRpBinItems];
 #pragma unroll
         for (int j = 0; j < kRpBinItems; ++j) {
           const Key key = static_cast<Key>(rec[j].key);
+          slot[j] = kNotMine;
           if (on[j] && key == Table::kEmpty) {
             atomicMin(tbl.all_ones, rec[j].i);
             on[j] = false;
+            slot[j] = kAllOnes;
           }
           k[j] = 0;
           cur[j] = 0;
@@ -1177,16 +1186,39 @@ __device__ __forceinline__ void rp_bin_body(unsigned bx, const RpArgs &a, unsign
           if (!on[j]) continue;
           if (k[j] == Table::kEmpty || k[j] == static_cast<Key>(rec[j].key)) {
             if (cur[j] > rec[j].i) atomicMin(tbl.index_at(hash[j] & tbl.mask), rec[j].i);
+            slot[j] = hash[j] & tbl.mask;
           } else {
-            fits &= tbl.insert_from(static_cast<Key>(rec[j].key), rec[j].i, hash[j] + 1);
+            fits &= tbl.insert_from(static_cast<Key>(rec[j].key), rec[j].i, hash[j] + 1, &slot[j]);
           }
         }
+        if (slot_out) {
+#pragma unroll
+          for (int j = 0; j < kRpBinItems; ++j) slot_out[j] = slot[j];
+        }
+      };
+      const uint32_t pass_records = kRpBinItems * blockDim.x;
+#pragma unroll
+      for (int pass = 0; pass < kRpHeldPasses; ++pass) {
+#pragma unroll
+        for (int j = 0; j < kRpBinItems; ++j) where[pass][j] = kNotMine;
+        if (pass * pass_records < cnt) insert_pass(threadIdx.x + pass * pass_records, where[pass]);
       }
+      for (uint32_t e0 = threadIdx.x + kRpHeldPasses * pass_records; e0 < cnt; e0 += pass_records) insert_pass(e0, nullptr);
       if (!fits) *overflow = 1;
       __syncthreads();
       done = *overflow == 0;
       if (done) {
-        for (uint32_t e0 = threadIdx.x; e0 < cnt; e0 += kRpBinItems * blockDim.x) {
+#pragma unroll
+        for (int pass = 0; pass < kRpHeldPasses; ++pass) {
+#pragma unroll
+          for (int j = 0; j < kRpBinItems; ++j) {
+            const uint32_t w = where[pass][j];
+            if (w != kNotMine)
+              a.firstp[start + threadIdx.x + pass * pass_records + j * blockDim.x] =
+                  w == kAllOnes ? *tbl.all_ones : *tbl.index_at(w);
+          }
+        }
+        for (uint32_t e0 = threadIdx.x + kRpHeldPasses * pass_records; e0 < cnt; e0 += pass_records) {
           RpRecord<PACKED> rec[kRpBinItems];
           uint32_t hash[kRpBinItems];
           bool on[kRpBinItems];
