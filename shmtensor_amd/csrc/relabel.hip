@@ -671,10 +671,11 @@ __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
 // The insert and first-occurrence passes above touch a random line of a table
 // that no cache holds once per id and pass, and the part moves such lines at
 // 50 G per second whatever the kernel does (3.1 M ids: 74 + 54 us, plus 22 us to
-// empty the table). From kRpDefaultMin ids on the same two results -- the
-// first-occurrence index of every element and the number of first occurrences
-// per tile of kRlTile ids -- come from five passes that read and write memory
-// in runs instead:
+// empty the table). From a million ids on (kRpExactMin; kRpDefaultMin for a
+// hop sized by a loose bound, kRpMergedMin for hops that share their launches)
+// the same two results -- the first-occurrence index of every element and the
+// number of first occurrences per tile of kRlTile ids -- come from five passes
+// that read and write memory in runs instead:
 //   count    a workgroup per tile of kRpTile ids: histogram of the ids over P
 //            bins (bin = top bits of the id's hash), one column of the P x W
 //            matrix; ids that repeat within the tile are counted once
@@ -692,11 +693,12 @@ __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
 // with 256 bins, 31 / 17 us with 1,024, and 42 / 29 us before the runs went
 // through LDS).
 // P = 256 up to 4 M ids, 512 up to 8 M; larger inputs keep the table in memory.
-// A bin's table has 16,384 slots (8,192 for ids beyond 32 bits); the ids of a
-// bin that do not fit (more than that many distinct ones, or ids crafted to
-// collide) are worked through in 2, 4, ... rounds over classes of a second
-// hash, and by comparing all pairs when 2^kRpMaxRoundsLog2 rounds do not do:
-// slower, never wrong. Records are {id : 32 | index : 32} when the ids fit 32
+// A bin's table has 4,096 to 16,384 slots (half for ids beyond 32 bits), as
+// many as the bin can hold ids when all of the input's are distinct, in
+// workgroups of 256 to 1,024 threads; the ids of a bin that do not fit (more
+// than that many distinct ones, or ids crafted to collide) are worked through
+// in 2, 4, ... rounds over classes of a second hash, and by comparing all
+// pairs when 2^kRpMaxRoundsLog2 rounds do not do: slower, never wrong. Records are {id : 32 | index : 32} when the ids fit 32
 // bits and 16 bytes otherwise; everything lives in the memory the table in
 // memory would have had.
 constexpr int kRpBlock = 1024;
