@@ -328,7 +328,7 @@ int shmt_relabel_wide(const void *total, int64_t N, void *scratch,
                       void *labels_out, int64_t *count_out, void *stream);
 /* How large inputs are relabelled (no counterpart in the reference, whose
  * four passes all probe one table in memory, src/tensor_relabel.cu:147-203).
- * From partition_min_ids ids on (and up to 2^23) the first-occurrence index of
+ * From partition_min_ids ids on (and up to 7,340,032) the first-occurrence index of
  * every id is found by partitioning the ids by hash and giving every
  * partition a table in LDS, which reads and writes memory in streams instead
  * of touching one random line per id and pass; results are identical.

@@ -19,7 +19,7 @@
 // the id, src/tensor_relabel.cu:111-117); ids known to fit 32 bits use the
 // same memory as packed 8-byte slots (see rl_packed_insert).
 // Up to 8,192 ids all of this is one launch of one workgroup with its table
-// in LDS (rl_small_kernel). Beyond 2 M ids (and up to 8 M) fill, insert and
+// in LDS (rl_small_kernel). Beyond 1 M ids (and up to 7.3 M) fill, insert and
 // first are replaced by passes that partition the ids by hash and give every
 // partition a table in LDS (rp_*_kernel, further down).
 #include "common.h"
@@ -692,10 +692,11 @@ __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
 // over 256 bins: 32 records; measured on 3.1 M ids, scatter / gather 24 / 14 us
 // with 256 bins, 31 / 17 us with 1,024, and 42 / 29 us before the runs went
 // through LDS).
-// P = 256 up to 4 M ids, 512 up to 8 M; larger inputs keep the table in memory.
-// A bin's table has 4,096 to 16,384 slots (half for ids beyond 32 bits), as
-// many as the bin can hold ids when all of the input's are distinct, in
-// workgroups of 256 to 1,024 threads; the ids of a bin that do not fit (more
+// P = 256 up to 3.67 M ids, 512 up to 7.34 M (a bin's table is at most 7/8 full
+// when every id of the input is distinct); larger inputs keep the table in memory.
+// A bin's table has 4,096 to 16,384 slots (half for ids beyond 32 bits), two
+// per id the bin can hold when all of the input's are distinct as far as
+// that goes, in workgroups of 256 to 1,024 threads; the ids of a bin that do not fit (more
 // than that many distinct ones, or ids crafted to collide) are worked through
 // in 2, 4, ... rounds over classes of a second hash, and by comparing all
 // pairs when 2^kRpMaxRoundsLog2 rounds do not do: slower, never wrong. Records are {id : 32 | index : 32} when the ids fit 32
@@ -704,7 +705,7 @@ __global__ void rl_zero_count_kernel(int64_t *count_out, int64_t *count_copy) {
 constexpr int kRpBlock = 1024;
 constexpr int kRpSlotsLog2 = 14;     // 16,384 slots of 4 + 4 bytes = 128 KB of LDS
 constexpr int kRpMinBinsLog2 = 8, kRpMaxBinsLog2 = 9;
-constexpr int64_t kRpBinIds = 16384; // ids per bin from which on the number of bins grows
+constexpr int64_t kRpBinIds = 14336; // ids per bin from which on the number of bins grows: 7/8 of the largest table
 constexpr int64_t kRpTile = 8192;    // ids per tile of the count / scatter / gather passes
 constexpr int kRpMaxRoundsLog2 = 10;
 constexpr int64_t kRpDefaultMin = kRlSelfPrefixTiles * kRlTile + 1;
@@ -745,11 +746,11 @@ static RpPlan rp_plan(int64_t N, int merged_jobs = 0, bool loose = false) {
   p.log2P = lg;
   p.P = 1u << lg;
   p.W = static_cast<uint32_t>((N + kRpTile - 1) / kRpTile);
-  // at least one slot per id the bin may hold if every id of the input is distinct; when N is a loose bound of
-  // the id count (a chained hop: typically three times what turns up) half of that, a bin that does get more
-  // taking two rounds
+  // two slots per id the bin may hold if every id of the input is distinct, as far as the largest table goes;
+  // when N is a loose bound of the id count (a chained hop: typically three times what turns up) a quarter of
+  // that, a bin that does get more taking two rounds
   p.table_log2 = kRpMinSlotsLog2;
-  while (p.table_log2 < kRpSlotsLog2 && (static_cast<int64_t>(p.P) << p.table_log2) < (loose ? N / 2 : N)) ++p.table_log2;
+  while (p.table_log2 < kRpSlotsLog2 && (static_cast<int64_t>(p.P) << p.table_log2) < (loose ? N / 2 : 2 * N)) ++p.table_log2;
   auto up = [](int64_t x) { return (x + 255) & ~255ll; };
   p.rec_off = 0;
   p.first_off = up(16 * N);
@@ -1056,10 +1057,23 @@ struct RpTable {
     if (threadIdx.x == 0) *all_ones = 0xFFFFFFFFu;
   }
 
-  // From slot p on (key != kEmpty); *slot: where the id sits (ids never move once they have a slot).
-  __device__ __forceinline__ bool insert_from(Key key, uint32_t i, uint32_t p, uint32_t *slot) const {
-    p &= mask;
-    for (uint32_t probes = 0; probes <= mask; ++probes) {
+  // An id sits within kMaxProbes slots of its home slot or not at all: a table so full that probe sequences
+  // get longer (a bin of nearly as many distinct ids as it has slots) counts as one that does not fit, and
+  // the bin takes two rounds at half the load instead of walking through thousands of slots per id.
+  static constexpr uint32_t kMaxProbes = 256;
+
+  // The probe sequence of an id: its home slot (low bits of the hash), then steps of an odd stride taken from
+  // the hash's upper bits. LDS has no lines to stay within, so a stride costs nothing and keeps the sequences
+  // of a nearly full table short (1 / (1 - load) probes where slot-by-slot probing needs the square of that).
+  __device__ __forceinline__ uint32_t stride(uint32_t hash) const { return ((hash >> 15) | 1u) & mask; }
+
+  // From the second slot of the sequence on (key != kEmpty); *slot: where the id sits (ids never move once
+  // they have a slot).
+  __device__ __forceinline__ bool insert_from(Key key, uint32_t i, uint32_t hash, uint32_t *slot) const {
+    const uint32_t step = stride(hash);
+    uint32_t p = (hash + step) & mask;
+    const uint32_t limit = mask < kMaxProbes ? mask : kMaxProbes;
+    for (uint32_t probes = 0; probes < limit; ++probes) {
       Key k;
       uint32_t cur;
       look(p, &k, &cur);
@@ -1069,19 +1083,21 @@ struct RpTable {
         *slot = p;
         return true;
       }
-      p = (p + 1) & mask;
+      p = (p + step) & mask;
     }
     return false;
   }
 
-  __device__ __forceinline__ uint32_t first_from(Key key, uint32_t p) const {
-    p &= mask;
-    for (uint32_t probes = 0; probes <= mask; ++probes) {
+  __device__ __forceinline__ uint32_t first_from(Key key, uint32_t hash) const {
+    const uint32_t step = stride(hash);
+    uint32_t p = (hash + step) & mask;
+    const uint32_t limit = mask < kMaxProbes ? mask : kMaxProbes;
+    for (uint32_t probes = 0; probes < limit; ++probes) {
       Key k;
       uint32_t cur;
       look(p, &k, &cur);
       if (k == key) return cur;
-      p = (p + 1) & mask;
+      p = (p + step) & mask;
     }
     return 0xFFFFFFFFu;  // cannot happen: every id was inserted
   }
@@ -1190,7 +1206,7 @@ __device__ __forceinline__ void rp_bin_body(unsigned bx, const RpArgs &a, unsign
             if (cur[j] > rec[j].i) atomicMin(tbl.index_at(hash[j] & tbl.mask), rec[j].i);
             slot[j] = hash[j] & tbl.mask;
           } else {
-            fits &= tbl.insert_from(static_cast<Key>(rec[j].key), rec[j].i, hash[j] + 1, &slot[j]);
+            fits &= tbl.insert_from(static_cast<Key>(rec[j].key), rec[j].i, hash[j], &slot[j]);
           }
         }
         if (slot_out) {
@@ -1240,7 +1256,7 @@ __device__ __forceinline__ void rp_bin_body(unsigned bx, const RpArgs &a, unsign
             if (key == Table::kEmpty)
               f[j] = *tbl.all_ones;
             else if (k[j] != key)
-              f[j] = tbl.first_from(key, hash[j] + 1);
+              f[j] = tbl.first_from(key, hash[j]);
             a.firstp[start + e0 + j * blockDim.x] = f[j];
           }
         }
