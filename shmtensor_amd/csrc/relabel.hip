@@ -831,7 +831,10 @@ __device__ __forceinline__ bool rp_covered(const RpArgs &a, const unsigned long 
   return a.eb == 4 || static_cast<const int64_t *>(a.total)[static_cast<uint32_t>(v >> 32)] == key;
 }
 
-__device__ __forceinline__ void rp_count_body(unsigned bx, const RpArgs &a) {
+// SEGS: the ids are still in the caller's segments; the pass also writes their concatenation (`total`), so
+// that no launch of its own reads and writes every id just for that.
+template <bool SEGS>
+__device__ __forceinline__ void rp_count_body(unsigned bx, const RpArgs &a, const RlSegments &segs) {
   extern __shared__ uint32_t hist[];  // P counters
   __shared__ unsigned long long dedup[kRpDedupSlots];
   const int64_t N = rl_count(a.n);
@@ -849,7 +852,39 @@ __device__ __forceinline__ void rp_count_body(unsigned bx, const RpArgs &a) {
   int64_t idx[kRpItems], key[kRpItems];
   bool ok[kRpItems];
   uint32_t hash[kRpItems];
-  rp_load_chunk(a, lo, hi, idx, ok, key);
+  if (SEGS) {
+    // as a rule a tile lies within one segment: one pointer and one width for all its loads
+    int first_seg = 0, last_seg = 0;
+    while (first_seg + 1 < segs.n && lo >= segs.start[first_seg + 1]) ++first_seg;
+    while (last_seg + 1 < segs.n && hi - 1 >= segs.start[last_seg + 1]) ++last_seg;
+#pragma unroll
+    for (int j = 0; j < kRpItems; ++j) {
+      idx[j] = lo + j * kRpBlock + threadIdx.x;
+      ok[j] = idx[j] < hi;
+      key[j] = 0;
+    }
+    if (first_seg == last_seg) {
+      int64_t at[kRpItems];
+#pragma unroll
+      for (int j = 0; j < kRpItems; ++j) at[j] = idx[j] - segs.start[first_seg];
+      load_ints<kRpItems>(segs.ptr[first_seg], at, ok, segs.bytes[first_seg], key);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kRpItems; ++j) {
+        if (!ok[j]) continue;
+        int sgm = first_seg;
+        while (sgm < last_seg && idx[j] >= segs.start[sgm + 1]) ++sgm;
+        key[j] = load_int(segs.ptr[sgm], idx[j] - segs.start[sgm], segs.bytes[sgm]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kRpItems; ++j)
+      if (ok[j]) store_int(const_cast<void *>(a.total), idx[j], a.eb, key[j]);
+    // the repeats test below reads ids of this tile back from `total`
+    __syncthreads();
+  } else {
+    rp_load_chunk(a, lo, hi, idx, ok, key);
+  }
   bool wide = false;
 #pragma unroll
   for (int j = 0; j < kRpItems; ++j) {
@@ -868,10 +903,16 @@ __device__ __forceinline__ void rp_count_body(unsigned bx, const RpArgs &a) {
   for (uint32_t b = threadIdx.x; b < P; b += kRpBlock) a.hist[static_cast<size_t>(b) * a.W + bx] = hist[b];
 }
 
-__global__ __launch_bounds__(kRpBlock) void rp_count_kernel(RpArgs a) { rp_count_body(blockIdx.x, a); }
+__global__ __launch_bounds__(kRpBlock) void rp_count_kernel(RpArgs a) {
+  rp_count_body<false>(blockIdx.x, a, RlSegments{});
+}
+
+__global__ __launch_bounds__(kRpBlock) void rp_count_segments_kernel(RpArgs a, RlSegments segs) {
+  rp_count_body<true>(blockIdx.x, a, segs);
+}
 
 __global__ __launch_bounds__(kRpBlock) void rp_count_jobs(Jobs<RpArgs> j) {
-  if (blockIdx.x < j.blocks[blockIdx.y]) rp_count_body(blockIdx.x, j.a[blockIdx.y]);
+  if (blockIdx.x < j.blocks[blockIdx.y]) rp_count_body<false>(blockIdx.x, j.a[blockIdx.y], RlSegments{});
 }
 
 // One wave per bin: the row's counts become the offsets of the tiles' runs inside the bin.
@@ -1655,14 +1696,10 @@ static int relabel_impl(const void *total, const RlSegments *segs, int64_t N, Rl
       stage_push(defer, kStageRlLabels, grid_for(N, 256), 256, lab);
       return SHMT_OK;
     }
-    if (segs && !prepared) {
-      // concatenation only: there is no table to empty
-      hipLaunchKernelGGL(rl_fill_concat_kernel, dim3(grid_for(N, 256 * 4)), dim3(256), 0, s,
-                         static_cast<uint4 *>(nullptr), static_cast<int64_t>(0), *segs, const_cast<void *>(total),
-                         elem_bytes, n, wide_mark, nonce);
-      SHMT_LAUNCH_CHECK();
-    }
-    hipLaunchKernelGGL(rp_count_kernel, dim3(rp.W), dim3(kRpBlock), rp.P * sizeof(uint32_t), s, a);
+    if (segs && !prepared)  // the count pass concatenates on the way: there is no table to empty
+      hipLaunchKernelGGL(rp_count_segments_kernel, dim3(rp.W), dim3(kRpBlock), rp.P * sizeof(uint32_t), s, a, *segs);
+    else
+      hipLaunchKernelGGL(rp_count_kernel, dim3(rp.W), dim3(kRpBlock), rp.P * sizeof(uint32_t), s, a);
     SHMT_LAUNCH_CHECK();
     hipLaunchKernelGGL(rp_rows_kernel, dim3((rp.P + 3) / 4), dim3(256), 0, s, a);
     SHMT_LAUNCH_CHECK();
