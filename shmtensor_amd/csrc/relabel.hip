@@ -576,46 +576,68 @@ __device__ __forceinline__ void rl_small_body(const RlSmallArgs &a, const RlSegm
   }
   __syncthreads();
   // insert: claim the first free slot of the probe sequence with the element's index, or lower the
-  // index of the slot that already stands for the same key
+  // index of the slot that already stands for the same key. One workgroup on one compute unit is bound by
+  // the latency of its dependent LDS accesses, so the first probes of a thread's eight elements are made side
+  // by side (look, claim, compare, lower: four round trips for all eight instead of up to four each), and
+  // only an element that meets another id at its home slot walks on alone. A key never leaves its slot:
+  // where it sits is kept for the next phase.
+  uint32_t slot[kRlSmallItems], cur[kRlSmallItems];
+  bool open[kRlSmallItems];
 #pragma unroll
   for (int j = 0; j < kRlSmallItems; ++j) {
     const uint32_t i = j * kRlSmallBlock + t;
-    if (static_cast<int>(i) < N) {
-      uint32_t p = hash_id(id[j]) & (kRlSmallSlots - 1);
-      for (int probes = 0; probes < kRlSmallSlots; ++probes) {
-        uint32_t cur = tbl[p];
-        if (cur == 0xFFFFFFFFu) {
-          cur = atomicCAS(&tbl[p], 0xFFFFFFFFu, i);
-          if (cur == 0xFFFFFFFFu) break;
-        }
-        if (keys[cur] == id[j]) {
-          if (cur > i) atomicMin(&tbl[p], i);
-          break;
-        }
-        p = (p + 1) & (kRlSmallSlots - 1);
-      }
+    open[j] = static_cast<int>(i) < N;
+    slot[j] = hash_id(id[j]) & (kRlSmallSlots - 1);
+    cur[j] = open[j] ? tbl[slot[j]] : 0u;
+  }
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const uint32_t i = j * kRlSmallBlock + t;
+    if (open[j] && cur[j] == 0xFFFFFFFFu) {
+      cur[j] = atomicCAS(&tbl[slot[j]], 0xFFFFFFFFu, i);
+      if (cur[j] == 0xFFFFFFFFu) open[j] = false;  // claimed
     }
   }
+  int64_t there[kRlSmallItems];
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) there[j] = open[j] ? keys[cur[j]] : 0;
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const uint32_t i = j * kRlSmallBlock + t;
+    if (!open[j]) continue;
+    if (there[j] == id[j]) {
+      if (cur[j] > i) atomicMin(&tbl[slot[j]], i);
+      continue;
+    }
+    uint32_t p = (slot[j] + 1) & (kRlSmallSlots - 1);
+    for (int probes = 1; probes < kRlSmallSlots; ++probes) {
+      uint32_t c = tbl[p];
+      if (c == 0xFFFFFFFFu) {
+        c = atomicCAS(&tbl[p], 0xFFFFFFFFu, i);
+        if (c == 0xFFFFFFFFu) break;
+      }
+      if (keys[c] == id[j]) {
+        if (c > i) atomicMin(&tbl[p], i);
+        break;
+      }
+      p = (p + 1) & (kRlSmallSlots - 1);
+    }
+    slot[j] = p;
+  }
   __syncthreads();
-  // first occurrence of every element; count the elements that are their own first occurrence,
-  // eight 16-bit counters (one per j) packed into two words
+  // first occurrence of every element: what its key's slot holds now; count the elements that are their own
+  // first occurrence, eight 16-bit counters (one per j) packed into two words
   uint32_t first[kRlSmallItems];
   uint64_t lo = 0, hi = 0;
 #pragma unroll
   for (int j = 0; j < kRlSmallItems; ++j) {
     const uint32_t i = j * kRlSmallBlock + t;
-    first[j] = 0xFFFFFFFFu;
+    first[j] = static_cast<int>(i) < N ? tbl[slot[j]] : 0xFFFFFFFFu;
+  }
+#pragma unroll
+  for (int j = 0; j < kRlSmallItems; ++j) {
+    const uint32_t i = j * kRlSmallBlock + t;
     if (static_cast<int>(i) < N) {
-      uint32_t p = hash_id(id[j]) & (kRlSmallSlots - 1);
-      for (int probes = 0; probes < kRlSmallSlots; ++probes) {
-        const uint32_t cur = tbl[p];
-        if (cur == 0xFFFFFFFFu) break;  // cannot happen: every key was inserted
-        if (keys[cur] == id[j]) {
-          first[j] = cur;
-          break;
-        }
-        p = (p + 1) & (kRlSmallSlots - 1);
-      }
       const uint64_t win = first[j] == i;
       if (j < 4) lo += win << (16 * j); else hi += win << (16 * (j - 4));
     }
